@@ -1,0 +1,224 @@
+/*
+ * parrot_hip.h -- C ABI of libparrot_hip.so: the attention hot path of
+ * Parrot's builtin engine on AMD MI355X (gfx950).
+ *
+ * Conventions (they mirror the reference's native extension, which takes
+ * tensors owned by the caller, launches on the caller's current stream and
+ * neither synchronises nor allocates -- csrc/attention/attention_post_kernels.cu:416):
+ *   - every pointer is a DEVICE pointer owned by the caller unless it says host;
+ *   - strides and sizes are in ELEMENTS unless the name ends in _bytes;
+ *   - all launches are asynchronous on `stream` (a hipStream_t passed as void*);
+ *   - no entry point allocates, frees or synchronises; scratch comes in through
+ *     a workspace argument whose size the matching *_workspace_bytes() reports;
+ *   - return value: PH_OK or a PH_ERR_* code; ph_status_string() names it.
+ *     The reference raises RuntimeError through TORCH_CHECK for unsupported
+ *     head size / dtype (csrc/attention/attention_kernels.cu:482,535,568); the
+ *     Python layer turns a non-zero status into the same exception class.
+ *   - KV pools are token-granular: [slots, H, D], the reference's
+ *     MemLayout.NORMAL (parrot/engine/builtin/mem.py:43-56); a "block table"
+ *     of the reference with block_size 1 is a list of slot ids here.
+ */
+#ifndef PARROT_HIP_H
+#define PARROT_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum { PH_F16 = 0, PH_BF16 = 1 } ph_dtype;
+typedef enum { PH_IDX_I32 = 0, PH_IDX_I64 = 1 } ph_index_type;
+
+enum {
+  PH_OK = 0,
+  PH_ERR_DTYPE = 1,     /* unsupported element type */
+  PH_ERR_HEAD_DIM = 2,  /* unsupported head size */
+  PH_ERR_ALIGN = 3,     /* pointer or stride not aligned as the kernel needs */
+  PH_ERR_ARG = 4,       /* inconsistent sizes, null pointer, negative count */
+  PH_ERR_WORKSPACE = 5, /* workspace too small */
+  PH_ERR_LAUNCH = 6     /* hipLaunchKernel reported an error */
+};
+
+const char* ph_status_string(int status);
+/* Library ABI version; bumped whenever a signature changes. */
+int ph_abi_version(void);
+
+/* ------------------------------------------------------------------------ */
+/* Token move: dest[dst_idx[i], :, :] = src[src_idx[i], :, :], i < n.
+ * Replaces discontinuous_move_tokens and its Triton kernel
+ * (parrot/engine/builtin/kernels/tokens_moving.py:25-100): rows are
+ * [num_heads, head_dim] with free strides on all three axes.
+ * src_idx == NULL means the identity (row i); same for dst_idx.
+ * dst indices must be unique (the reference has the same requirement).
+ * Bit-exact copy; elem_bytes in {1,2,4,8}. */
+int ph_move_tokens(const void* src, void* dst,
+                   const void* src_idx, const void* dst_idx, int index_type,
+                   int64_t n, int64_t num_heads, int64_t head_dim, int elem_bytes,
+                   int64_t src_stride_n, int64_t src_stride_h, int64_t src_stride_d,
+                   int64_t dst_stride_n, int64_t dst_stride_h, int64_t dst_stride_d,
+                   void* stream);
+
+/* KV append: k_cache[slot[t]] = k[t], v_cache[slot[t]] = v[t] in ONE launch.
+ * Replaces vllm_reshape_and_cache -> cache_ops.reshape_and_cache
+ * (parrot/engine/builtin/kernels/vllm/reshape_and_cache.py:9-22,
+ * 3rdparty/vllm/csrc/cache_kernels.cu:142-224) on the token-granular layout,
+ * and the arange-source token move of attn_func.py:143-155.
+ * k, v: [T, H, D] with row stride k_stride_n / v_stride_n (heads contiguous);
+ * caches: [slots, H, D] with row stride cache_stride_n. */
+int ph_kv_append(const void* k, const void* v, void* k_cache, void* v_cache,
+                 const void* slot_mapping, int index_type,
+                 int64_t num_tokens, int64_t num_heads, int64_t head_dim, int dtype,
+                 int64_t k_stride_n, int64_t v_stride_n, int64_t cache_stride_n,
+                 void* stream);
+
+/* ------------------------------------------------------------------------ */
+/* RMSNorm: out = w * t(x * rsqrt(mean(x^2) + eps)).
+ * Replaces layernorm_ops.rms_norm (3rdparty/vllm/csrc/layernorm_kernels.cu:9-63,
+ * wrapper parrot/engine/builtin/kernels/vllm/rms_norm.py:9-16) when
+ * round_before_weight != 0 (the normalised value is rounded to the element
+ * type before the weight multiply, :32), and rmsnorm_forward
+ * (parrot/engine/builtin/kernels/rms_norm.py:15-78) when it is 0 (one rounding).
+ * x, out: [rows, n] with row strides; w: [n]. */
+int ph_rms_norm(void* out, const void* x, const void* weight, float eps,
+                int64_t rows, int64_t n, int64_t x_stride, int64_t out_stride,
+                int dtype, int round_before_weight, void* stream);
+
+/* NeoX RoPE on q and k in place, one launch, cos/sin looked up by position.
+ * Replaces pos_encoding_ops.rotary_embedding_neox
+ * (3rdparty/vllm/csrc/pos_encoding_kernels.cu:6-104, wrapper
+ * parrot/engine/builtin/kernels/vllm/rotary_embed.py:10-25).
+ * q: [T, num_q_heads*head_dim] row stride q_stride; k likewise (they are chunk
+ * views of the fused qkv, models/llama.py:111-112); k may be NULL.
+ * cos_sin_cache: [max_pos, rot_dim] = cat(cos, sin); positions: int64 [T].
+ * Arithmetic follows the reference kernel: each product and the sum are rounded
+ * to the element type (:36-42). */
+int ph_rope_neox(const int64_t* positions, void* q, void* k, const void* cos_sin_cache,
+                 int64_t num_tokens, int64_t num_q_heads, int64_t num_k_heads,
+                 int64_t head_dim, int64_t rot_dim,
+                 int64_t q_stride, int64_t k_stride, int dtype, void* stream);
+
+/* NeoX RoPE in place with per-token cos / sin rows already gathered.
+ * Replaces rotary_embedding(state, cos, sin)
+ * (parrot/engine/builtin/kernels/rotary_embedding.py:24-143).
+ * state: [T, H, D] strides (stride_n, stride_h, 1); cos, sin: [T, 1, D/2] with
+ * row stride cs_stride. */
+int ph_rotary_embedding(void* state, const void* cos, const void* sin,
+                        int64_t num_tokens, int64_t num_heads, int64_t head_dim,
+                        int64_t stride_n, int64_t stride_h, int64_t cs_stride,
+                        int dtype, void* stream);
+
+/* ------------------------------------------------------------------------ */
+/* Decode attention (one query token per request) over slot tables.
+ *
+ * A request b attends over   prefix_slots[group(b)]  ||  suffix slots of b.
+ * Partials are (O, m, l) in the exp2 domain: y = q.k*scale*log2(e),
+ * m = max y, l = sum 2^(y-m), O = sum 2^(y-m) v / l
+ * (parrot/engine/builtin/kernels/shared_flash_decoding.py:98-134); the merge
+ * is M = max, L = sum 2^(m-M) l, O = sum 2^(m-M) l O / L
+ * (csrc/attention/attention_post_kernels.cu:321-340).
+ *
+ * ph_decode_attention replaces, depending on its arguments:
+ *   - flash_paged_attention / paged_flash_attention (shared prefix + suffix +
+ *     merge; shared_flash_decoding.py:285-376 = triton_flash_attention :202-277
+ *     + attention_ops.single_query_cached_kv_post_attention,
+ *     csrc/attention.cpp:34-47), when num_groups >= 1;
+ *   - vllm_paged_attention -> attention_ops.single_query_cached_kv_attention
+ *     (parrot/engine/builtin/kernels/vllm/paged_attention.py:12-38,
+ *     3rdparty/vllm/csrc/attention.cpp:4-15), when num_groups == 0.
+ *
+ * q, out: [B, H, D], row strides q_stride / out_stride (heads contiguous).
+ * k_cache, v_cache: [slots, H, D], row stride cache_stride_n.
+ * Prefix groups (num_groups may be 0):
+ *   prefix_slots: int32, all groups' prefix slot lists back to back;
+ *   prefix_cu:    int32 [num_groups+1] offsets into prefix_slots   (DEVICE);
+ *   group_req_cu: int32 [num_groups+1]: requests group_req_cu[g] ..
+ *                 group_req_cu[g+1]-1 belong to group g (requests of one group
+ *                 are contiguous; requests outside every range have no
+ *                 prefix).  Passed twice: a DEVICE copy for the kernels and a
+ *                 HOST copy for the launch geometry;
+ *   max_prefix_len: host upper bound of any group's prefix length.
+ * Suffix (per request) slot table, two forms:
+ *   suffix_offsets != NULL: int64 [B] start of request b's list inside
+ *                 suffix_slots (ragged, back to back);
+ *   suffix_offsets == NULL: suffix_slots is a padded 2-D table, request b's
+ *                 list starts at b * suffix_table_stride (the reference's
+ *                 paged_block_tables [B, max]).
+ *   suffix_lens:  int32 [B] (DEVICE); max_suffix_len: host upper bound.
+ * chunk_tokens: suffix split size (multiple of 16), 0 = choose.
+ * workspace: at least ph_decode_workspace_bytes(...) bytes, 256-byte aligned.
+ */
+size_t ph_decode_workspace_bytes(int64_t num_reqs, int64_t num_heads, int64_t head_dim,
+                                 int64_t num_groups, int64_t max_prefix_len,
+                                 int64_t max_suffix_len, int64_t chunk_tokens);
+
+int ph_decode_attention(void* out, const void* q, const void* k_cache, const void* v_cache,
+                        int64_t num_reqs, int64_t num_heads, int64_t head_dim, int dtype,
+                        int64_t q_stride, int64_t out_stride, int64_t cache_stride_n,
+                        float scale,
+                        int64_t num_groups, const int32_t* prefix_slots, const int32_t* prefix_cu,
+                        const int32_t* group_req_cu, const int32_t* group_req_cu_host,
+                        int64_t max_prefix_len,
+                        const int32_t* suffix_slots, const int64_t* suffix_offsets,
+                        int64_t suffix_table_stride, const int32_t* suffix_lens,
+                        int64_t max_suffix_len, int64_t chunk_tokens,
+                        void* workspace, size_t workspace_bytes, void* stream);
+
+/* The two halves of the shared-prefix op, exposed separately because the
+ * reference's extension does (csrc/attention.cpp:19-47):
+ *
+ * ph_prefix_attention: prefix phase only -- writes the normalised O (element
+ * type), and m / l as fp32 [B, H].  Replaces triton_flash_attention(...,
+ * save_mid_results=True) (shared_flash_decoding.py:202-277).
+ *
+ * ph_suffix_post_attention: suffix phase, then merge with the partial that
+ * already sits in out / prev_m / prev_l; out is in/out.  Replaces
+ * attention_ops.single_query_cached_kv_post_attention
+ * (csrc/attention/attention_post_kernels.cu:74-341). */
+int ph_prefix_attention(void* out, float* m_out, float* l_out,
+                        const void* q, const void* k_cache, const void* v_cache,
+                        int64_t num_reqs, int64_t num_heads, int64_t head_dim, int dtype,
+                        int64_t q_stride, int64_t out_stride, int64_t cache_stride_n, float scale,
+                        const int32_t* prefix_slots, int64_t prefix_len,
+                        void* workspace, size_t workspace_bytes, void* stream);
+
+int ph_suffix_post_attention(void* out, const float* prev_m, const float* prev_l,
+                             const void* q, const void* k_cache, const void* v_cache,
+                             int64_t num_reqs, int64_t num_heads, int64_t head_dim, int dtype,
+                             int64_t q_stride, int64_t out_stride, int64_t cache_stride_n, float scale,
+                             const int32_t* suffix_slots, const int64_t* suffix_offsets,
+                             int64_t suffix_table_stride, const int32_t* suffix_lens,
+                             int64_t max_suffix_len, int64_t chunk_tokens,
+                             void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------ */
+/* Prefill with parent context: packed ragged chunks, each causal
+ * (bottom-right aligned) over ancestors' + own KV read through a slot table.
+ * Replaces the gather (move_tokens_from_blocked_{k,v}_cache) + xformers
+ * memory_efficient_attention_forward with
+ * BlockDiagonalCausalFromBottomRightMask of
+ * parrot/engine/builtin/attn_func.py:635-674, i.e. the kernel declared and left
+ * unimplemented in parrot/engine/builtin/kernels/flash_attention_with_context.py:37-56.
+ * q, out: [T, H, D] packed chunk after chunk, row strides q_stride/out_stride.
+ * q_cu:  int32 [num_chunks+1] query offsets (DEVICE);
+ * kv_cu: int32 [num_chunks+1] offsets into ctx_slots (DEVICE);
+ * ctx_slots: int32, every chunk's whole context (ancestors || own), in order.
+ * Query r of chunk c sees key j iff j <= r + (kv_len_c - q_len_c).
+ * The new tokens' K/V must already be in the cache (append first).
+ * max_kv_len: host upper bound of any chunk's context length.
+ * workspace: at least ph_prefill_workspace_bytes(...) bytes, 256-byte aligned. */
+size_t ph_prefill_workspace_bytes(int64_t num_tokens, int64_t num_heads, int64_t head_dim,
+                                  int64_t max_kv_len);
+
+int ph_prefill_attention(void* out, const void* q, const void* k_cache, const void* v_cache,
+                         int64_t num_tokens, int64_t num_chunks, int64_t num_heads, int64_t head_dim,
+                         int dtype, int64_t q_stride, int64_t out_stride, int64_t cache_stride_n,
+                         float scale, const int32_t* q_cu, const int32_t* kv_cu,
+                         const int32_t* ctx_slots, int64_t max_kv_len,
+                         void* workspace, size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PARROT_HIP_H */

@@ -1,0 +1,437 @@
+// Host entry points of the decode-attention family: launch geometry, workspace
+// carving, argument checks.  No allocation, no synchronisation: everything is
+// enqueued on the caller's stream.
+#include "decode.hpp"
+
+namespace ph {
+
+struct DecodePlan {
+  int chunk;         // suffix tokens per part
+  int n_chunks;      // suffix parts per request
+  int split_tokens;  // prefix tokens per part
+  int n_splits;      // prefix parts
+  int parts() const { return n_chunks + n_splits; }
+};
+
+static int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
+static int64_t cdiv(int64_t x, int64_t m) { return (x + m - 1) / m; }
+
+constexpr int kPrefixTile = 64;        // tokens per LDS tile of the MFMA kernel
+constexpr int kPrefixQueryTile = 64;   // queries per workgroup of the MFMA kernel
+
+static DecodePlan plan_decode(int64_t B, int64_t H, int64_t groups, int64_t max_prefix, int64_t max_suffix,
+                              int64_t chunk_tokens) {
+  DecodePlan p{};
+  if (max_suffix > 0) {
+    int64_t chunk = chunk_tokens;
+    if (chunk <= 0) {
+      // Aim for about 2048 (request, chunk) items assuming mean length = max/2.
+      const int64_t want = B * max_suffix / 2 / 2048;
+      chunk = 32;
+      while (chunk < want && chunk < 1024) chunk *= 2;
+    }
+    chunk = round_up(chunk, 16);
+    p.chunk = (int)chunk;
+    p.n_chunks = (int)cdiv(max_suffix, chunk);
+  } else {
+    p.chunk = 32;
+    p.n_chunks = 0;
+  }
+  if (groups > 0 && max_prefix > 0) {
+    // About 512 workgroups over (group, head, query tile, split).
+    const int64_t mtiles = cdiv(cdiv(B, groups), kPrefixQueryTile);
+    int64_t splits = cdiv(512, groups * H * (mtiles > 0 ? mtiles : 1));
+    const int64_t max_splits = cdiv(max_prefix, 2 * kPrefixTile);
+    if (splits > max_splits) splits = max_splits;
+    if (splits < 1) splits = 1;
+    const int64_t st = round_up(cdiv(max_prefix, splits), kPrefixTile);
+    p.split_tokens = (int)st;
+    p.n_splits = (int)cdiv(max_prefix, st);
+  }
+  return p;
+}
+
+static size_t plan_bytes(const DecodePlan& p, int64_t B, int64_t H, int64_t D) {
+  const size_t rows = (size_t)p.parts() * B * H;
+  return round_up((int64_t)(rows * D * sizeof(float)), 256) + round_up((int64_t)(rows * 2 * sizeof(float)), 256);
+}
+
+struct Carve {
+  float* opart;
+  float* ml;
+};
+static Carve carve(void* ws, const DecodePlan& p, int64_t B, int64_t H, int64_t D) {
+  const size_t rows = (size_t)p.parts() * B * H;
+  Carve c;
+  c.opart = (float*)ws;
+  c.ml = (float*)((char*)ws + round_up((int64_t)(rows * D * sizeof(float)), 256));
+  return c;
+}
+
+static int check_common(const void* out, const void* q, const void* kc, const void* vc, int64_t B, int64_t H,
+                        int64_t D, int dtype, int64_t q_stride, int64_t out_stride, int64_t row_stride) {
+  if (dtype != PH_F16 && dtype != PH_BF16) return PH_ERR_DTYPE;
+  if (D != 64 && D != 128 && D != 256) return PH_ERR_HEAD_DIM;
+  if (B < 0 || H <= 0 || B > (1 << 24) || H > 4096) return PH_ERR_ARG;
+  if (B == 0) return PH_OK;
+  if (!out || !q || !kc || !vc) return PH_ERR_ARG;
+  if (q_stride < H * D || out_stride < H * D || row_stride < H * D) return PH_ERR_ARG;
+  if (!aligned16(out) || !aligned16(q) || !aligned16(kc) || !aligned16(vc) || q_stride % 8 || out_stride % 8 ||
+      row_stride % 8)
+    return PH_ERR_ALIGN;
+  return PH_OK;
+}
+
+// Prefix phase: matrix-core kernel for head size 128; other head sizes run the
+// per-request gather kernel once per group over the shared slot list.
+static int run_prefix(PrefixArgs& pa, int dtype, int D, int num_groups, const int32_t* group_req_cu_host,
+                      int max_group_reqs, hipStream_t st) {
+  if (prefix_mfma_supported(dtype, D)) return launch_prefix_mfma(pa, dtype, D, num_groups, max_group_reqs, st);
+  int rc = launch_clear_ml(pa.ml, (int64_t)pa.n_splits * pa.B * pa.H, st);
+  if (rc != PH_OK) return rc;
+  for (int g = 0; g < num_groups; ++g) {
+    PartialArgs sa{};
+    sa.q = pa.q;
+    sa.q_stride = pa.q_stride;
+    sa.kc = pa.kc;
+    sa.vc = pa.vc;
+    sa.row_stride = pa.row_stride;
+    sa.slots = pa.slots;
+    sa.shared_cu = pa.prefix_cu ? pa.prefix_cu + g : nullptr;
+    sa.shared_len = pa.prefix_cu ? -1 : pa.fixed_prefix_len;
+    sa.chunk = pa.split_tokens;
+    sa.n_chunks = pa.n_splits;
+    sa.part_base = 0;
+    sa.opart = pa.opart;
+    sa.ml = pa.ml;
+    sa.B = pa.B;
+    sa.H = pa.H;
+    sa.req_begin = group_req_cu_host ? group_req_cu_host[g] : 0;
+    sa.num_reqs = group_req_cu_host ? group_req_cu_host[g + 1] - group_req_cu_host[g] : pa.B;
+    sa.scale_log2e = pa.scale_log2e;
+    rc = launch_partial(sa, dtype, D, st);
+    if (rc != PH_OK) return rc;
+  }
+  return PH_OK;
+}
+
+// Per-token (offset, length) of the prefill-as-ragged-decode formulation.
+__global__ __launch_bounds__(256) void prefill_rows_kernel(const int32_t* q_cu, const int32_t* kv_cu, int num_chunks,
+                                                           int num_tokens, int64_t* offsets, int32_t* lens) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= num_tokens) return;
+  int lo = 0, hi = num_chunks;  // last chunk with q_cu[c] <= i
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (q_cu[mid] <= i) lo = mid; else hi = mid;
+  }
+  const int qn = q_cu[lo + 1] - q_cu[lo];
+  const int kvn = kv_cu[lo + 1] - kv_cu[lo];
+  offsets[i] = kv_cu[lo];
+  lens[i] = kvn - qn + (i - q_cu[lo]) + 1;
+}
+
+}  // namespace ph
+
+using namespace ph;
+
+extern "C" const char* ph_status_string(int status) {
+  switch (status) {
+    case PH_OK: return "ok";
+    case PH_ERR_DTYPE: return "unsupported data type";
+    case PH_ERR_HEAD_DIM: return "unsupported head size";
+    case PH_ERR_ALIGN: return "pointer or stride not 16-byte aligned";
+    case PH_ERR_ARG: return "invalid argument";
+    case PH_ERR_WORKSPACE: return "workspace too small";
+    case PH_ERR_LAUNCH: return "kernel launch failed";
+    default: return "unknown status";
+  }
+}
+
+extern "C" int ph_abi_version(void) { return 1; }
+
+extern "C" size_t ph_decode_workspace_bytes(int64_t num_reqs, int64_t num_heads, int64_t head_dim,
+                                            int64_t num_groups, int64_t max_prefix_len, int64_t max_suffix_len,
+                                            int64_t chunk_tokens) {
+  if (num_reqs <= 0 || num_heads <= 0 || head_dim <= 0) return 0;
+  const DecodePlan p = plan_decode(num_reqs, num_heads, num_groups, max_prefix_len, max_suffix_len, chunk_tokens);
+  return plan_bytes(p, num_reqs, num_heads, head_dim);
+}
+
+extern "C" int ph_decode_attention(void* out, const void* q, const void* k_cache, const void* v_cache,
+                                   int64_t num_reqs, int64_t num_heads, int64_t head_dim, int dtype,
+                                   int64_t q_stride, int64_t out_stride, int64_t cache_stride_n, float scale,
+                                   int64_t num_groups, const int32_t* prefix_slots, const int32_t* prefix_cu,
+                                   const int32_t* group_req_cu, const int32_t* group_req_cu_host,
+                                   int64_t max_prefix_len, const int32_t* suffix_slots,
+                                   const int64_t* suffix_offsets, int64_t suffix_table_stride,
+                                   const int32_t* suffix_lens, int64_t max_suffix_len, int64_t chunk_tokens,
+                                   void* workspace, size_t workspace_bytes, void* stream) {
+  const int B = (int)num_reqs, H = (int)num_heads, D = (int)head_dim;
+  int rc = check_common(out, q, k_cache, v_cache, num_reqs, num_heads, head_dim, dtype, q_stride, out_stride,
+                        cache_stride_n);
+  if (rc != PH_OK || num_reqs == 0) return rc;
+  if (num_groups < 0 || max_prefix_len < 0 || max_suffix_len < 0) return PH_ERR_ARG;
+  const bool has_prefix = num_groups > 0 && max_prefix_len > 0;
+  const bool has_suffix = max_suffix_len > 0;
+  if (has_prefix && (!prefix_slots || !prefix_cu || !group_req_cu || !group_req_cu_host)) return PH_ERR_ARG;
+  if (has_suffix && (!suffix_slots || !suffix_lens)) return PH_ERR_ARG;
+  const DecodePlan p =
+      plan_decode(num_reqs, num_heads, has_prefix ? num_groups : 0, max_prefix_len, max_suffix_len, chunk_tokens);
+  if (plan_bytes(p, B, H, D) > workspace_bytes || (p.parts() > 0 && !workspace)) return PH_ERR_WORKSPACE;
+  if (((uintptr_t)workspace & 255u) != 0) return PH_ERR_ALIGN;
+  const Carve ws = carve(workspace, p, B, H, D);
+  hipStream_t st = (hipStream_t)stream;
+  const float sl2 = scale * kLog2e;
+
+  if (has_prefix) {
+    int covered = 0, max_group_reqs = 0;
+    for (int g = 0; g < num_groups; ++g) {
+      const int r0 = group_req_cu_host[g], r1 = group_req_cu_host[g + 1];
+      if (r0 < 0 || r1 < r0 || r1 > B) return PH_ERR_ARG;
+      covered += r1 - r0;
+      if (r1 - r0 > max_group_reqs) max_group_reqs = r1 - r0;
+    }
+    if (covered != B) {  // requests outside every group: their prefix parts must read as empty
+      rc = launch_clear_ml(ws.ml, (int64_t)p.n_splits * B * H, st);
+      if (rc != PH_OK) return rc;
+    }
+    PrefixArgs pa{};
+    pa.q = (const uint16_t*)q;
+    pa.q_stride = q_stride;
+    pa.kc = (const uint16_t*)k_cache;
+    pa.vc = (const uint16_t*)v_cache;
+    pa.row_stride = cache_stride_n;
+    pa.slots = prefix_slots;
+    pa.prefix_cu = prefix_cu;
+    pa.group_req_cu = group_req_cu;
+    pa.fixed_prefix_len = -1;
+    pa.split_tokens = p.split_tokens;
+    pa.n_splits = p.n_splits;
+    pa.opart = ws.opart;
+    pa.ml = ws.ml;
+    pa.B = B;
+    pa.H = H;
+    pa.scale_log2e = sl2;
+    rc = run_prefix(pa, dtype, D, (int)num_groups, group_req_cu_host, max_group_reqs, st);
+    if (rc != PH_OK) return rc;
+  }
+  if (has_suffix) {
+    PartialArgs sa{};
+    sa.q = (const uint16_t*)q;
+    sa.q_stride = q_stride;
+    sa.kc = (const uint16_t*)k_cache;
+    sa.vc = (const uint16_t*)v_cache;
+    sa.row_stride = cache_stride_n;
+    sa.slots = suffix_slots;
+    sa.offsets = suffix_offsets;
+    sa.table_stride = suffix_table_stride;
+    sa.lens = suffix_lens;
+    sa.shared_cu = nullptr;
+    sa.shared_len = -1;
+    sa.chunk = p.chunk;
+    sa.n_chunks = p.n_chunks;
+    sa.part_base = p.n_splits;
+    sa.opart = ws.opart;
+    sa.ml = ws.ml;
+    sa.B = B;
+    sa.H = H;
+    sa.req_begin = 0;
+    sa.num_reqs = B;
+    sa.scale_log2e = sl2;
+    rc = launch_partial(sa, dtype, D, st);
+    if (rc != PH_OK) return rc;
+  }
+  MergeArgs ma{};
+  ma.opart = ws.opart;
+  ma.ml = ws.ml;
+  ma.out = (uint16_t*)out;
+  ma.out_stride = out_stride;
+  ma.B = B;
+  ma.H = H;
+  ma.nA = has_prefix ? p.n_splits : 0;
+  ma.baseB = p.n_splits;
+  ma.lens = has_suffix ? suffix_lens : nullptr;
+  ma.chunk = p.chunk;
+  return launch_merge(ma, dtype, D, st);
+}
+
+extern "C" int ph_prefix_attention(void* out, float* m_out, float* l_out, const void* q, const void* k_cache,
+                                   const void* v_cache, int64_t num_reqs, int64_t num_heads, int64_t head_dim,
+                                   int dtype, int64_t q_stride, int64_t out_stride, int64_t cache_stride_n,
+                                   float scale, const int32_t* prefix_slots, int64_t prefix_len, void* workspace,
+                                   size_t workspace_bytes, void* stream) {
+  const int B = (int)num_reqs, H = (int)num_heads, D = (int)head_dim;
+  int rc = check_common(out, q, k_cache, v_cache, num_reqs, num_heads, head_dim, dtype, q_stride, out_stride,
+                        cache_stride_n);
+  if (rc != PH_OK || num_reqs == 0) return rc;
+  if (prefix_len < 0 || !m_out || !l_out || (prefix_len > 0 && !prefix_slots)) return PH_ERR_ARG;
+  const DecodePlan p = plan_decode(num_reqs, num_heads, prefix_len > 0 ? 1 : 0, prefix_len, 0, 0);
+  if (plan_bytes(p, B, H, D) > workspace_bytes || (p.parts() > 0 && !workspace)) return PH_ERR_WORKSPACE;
+  if (((uintptr_t)workspace & 255u) != 0) return PH_ERR_ALIGN;
+  const Carve ws = carve(workspace, p, B, H, D);
+  hipStream_t st = (hipStream_t)stream;
+  if (prefix_len > 0) {
+    PrefixArgs pa{};
+    pa.q = (const uint16_t*)q;
+    pa.q_stride = q_stride;
+    pa.kc = (const uint16_t*)k_cache;
+    pa.vc = (const uint16_t*)v_cache;
+    pa.row_stride = cache_stride_n;
+    pa.slots = prefix_slots;
+    pa.prefix_cu = nullptr;
+    pa.group_req_cu = nullptr;
+    pa.fixed_prefix_len = (int)prefix_len;
+    pa.split_tokens = p.split_tokens;
+    pa.n_splits = p.n_splits;
+    pa.opart = ws.opart;
+    pa.ml = ws.ml;
+    pa.B = B;
+    pa.H = H;
+    pa.scale_log2e = scale * kLog2e;
+    rc = run_prefix(pa, dtype, D, 1, nullptr, B, st);
+    if (rc != PH_OK) return rc;
+  }
+  MergeArgs ma{};
+  ma.opart = ws.opart;
+  ma.ml = ws.ml;
+  ma.out = (uint16_t*)out;
+  ma.out_stride = out_stride;
+  ma.B = B;
+  ma.H = H;
+  ma.nA = p.n_splits;
+  ma.baseB = p.n_splits;
+  ma.lens = nullptr;
+  ma.chunk = p.chunk;
+  ma.m_out = m_out;
+  ma.l_out = l_out;
+  return launch_merge(ma, dtype, D, st);
+}
+
+extern "C" int ph_suffix_post_attention(void* out, const float* prev_m, const float* prev_l, const void* q,
+                                        const void* k_cache, const void* v_cache, int64_t num_reqs,
+                                        int64_t num_heads, int64_t head_dim, int dtype, int64_t q_stride,
+                                        int64_t out_stride, int64_t cache_stride_n, float scale,
+                                        const int32_t* suffix_slots, const int64_t* suffix_offsets,
+                                        int64_t suffix_table_stride, const int32_t* suffix_lens,
+                                        int64_t max_suffix_len, int64_t chunk_tokens, void* workspace,
+                                        size_t workspace_bytes, void* stream) {
+  const int B = (int)num_reqs, H = (int)num_heads, D = (int)head_dim;
+  int rc = check_common(out, q, k_cache, v_cache, num_reqs, num_heads, head_dim, dtype, q_stride, out_stride,
+                        cache_stride_n);
+  if (rc != PH_OK || num_reqs == 0) return rc;
+  if (max_suffix_len < 0 || !prev_m || !prev_l) return PH_ERR_ARG;
+  const bool has_suffix = max_suffix_len > 0;
+  if (has_suffix && (!suffix_slots || !suffix_lens)) return PH_ERR_ARG;
+  const DecodePlan p = plan_decode(num_reqs, num_heads, 0, 0, max_suffix_len, chunk_tokens);
+  if (plan_bytes(p, B, H, D) > workspace_bytes || (p.parts() > 0 && !workspace)) return PH_ERR_WORKSPACE;
+  if (((uintptr_t)workspace & 255u) != 0) return PH_ERR_ALIGN;
+  const Carve ws = carve(workspace, p, B, H, D);
+  hipStream_t st = (hipStream_t)stream;
+  if (has_suffix) {
+    PartialArgs sa{};
+    sa.q = (const uint16_t*)q;
+    sa.q_stride = q_stride;
+    sa.kc = (const uint16_t*)k_cache;
+    sa.vc = (const uint16_t*)v_cache;
+    sa.row_stride = cache_stride_n;
+    sa.slots = suffix_slots;
+    sa.offsets = suffix_offsets;
+    sa.table_stride = suffix_table_stride;
+    sa.lens = suffix_lens;
+    sa.shared_cu = nullptr;
+    sa.shared_len = -1;
+    sa.chunk = p.chunk;
+    sa.n_chunks = p.n_chunks;
+    sa.part_base = 0;
+    sa.opart = ws.opart;
+    sa.ml = ws.ml;
+    sa.B = B;
+    sa.H = H;
+    sa.req_begin = 0;
+    sa.num_reqs = B;
+    sa.scale_log2e = scale * kLog2e;
+    rc = launch_partial(sa, dtype, D, st);
+    if (rc != PH_OK) return rc;
+  }
+  MergeArgs ma{};
+  ma.opart = ws.opart;
+  ma.ml = ws.ml;
+  ma.out = (uint16_t*)out;
+  ma.out_stride = out_stride;
+  ma.B = B;
+  ma.H = H;
+  ma.nA = 0;
+  ma.baseB = 0;
+  ma.lens = has_suffix ? suffix_lens : nullptr;
+  ma.chunk = p.chunk;
+  ma.prev_m = prev_m;
+  ma.prev_l = prev_l;
+  return launch_merge(ma, dtype, D, st);
+}
+
+extern "C" size_t ph_prefill_workspace_bytes(int64_t num_tokens, int64_t num_heads, int64_t head_dim,
+                                             int64_t max_kv_len) {
+  if (num_tokens <= 0 || num_heads <= 0 || head_dim <= 0) return 0;
+  const DecodePlan p = plan_decode(num_tokens, num_heads, 0, 0, max_kv_len, 0);
+  return (size_t)round_up(num_tokens * 8, 256) + (size_t)round_up(num_tokens * 4, 256) +
+         plan_bytes(p, num_tokens, num_heads, head_dim);
+}
+
+extern "C" int ph_prefill_attention(void* out, const void* q, const void* k_cache, const void* v_cache,
+                                    int64_t num_tokens, int64_t num_chunks, int64_t num_heads, int64_t head_dim,
+                                    int dtype, int64_t q_stride, int64_t out_stride, int64_t cache_stride_n,
+                                    float scale, const int32_t* q_cu, const int32_t* kv_cu,
+                                    const int32_t* ctx_slots, int64_t max_kv_len, void* workspace,
+                                    size_t workspace_bytes, void* stream) {
+  const int T = (int)num_tokens, H = (int)num_heads, D = (int)head_dim;
+  int rc = check_common(out, q, k_cache, v_cache, num_tokens, num_heads, head_dim, dtype, q_stride, out_stride,
+                        cache_stride_n);
+  if (rc != PH_OK || num_tokens == 0) return rc;
+  if (num_chunks <= 0 || max_kv_len <= 0 || !q_cu || !kv_cu || !ctx_slots) return PH_ERR_ARG;
+  if (ph_prefill_workspace_bytes(num_tokens, num_heads, head_dim, max_kv_len) > workspace_bytes || !workspace)
+    return PH_ERR_WORKSPACE;
+  if (((uintptr_t)workspace & 255u) != 0) return PH_ERR_ALIGN;
+  hipStream_t st = (hipStream_t)stream;
+  int64_t* offsets = (int64_t*)workspace;
+  int32_t* lens = (int32_t*)((char*)workspace + round_up(num_tokens * 8, 256));
+  void* dws = (char*)lens + round_up(num_tokens * 4, 256);
+  hipLaunchKernelGGL(prefill_rows_kernel, dim3((T + 255) / 256), dim3(256), 0, st, q_cu, kv_cu, (int)num_chunks, T,
+                     offsets, lens);
+  if ((rc = launch_status()) != PH_OK) return rc;
+  const DecodePlan p = plan_decode(num_tokens, num_heads, 0, 0, max_kv_len, 0);
+  const Carve ws = carve(dws, p, T, H, D);
+  PartialArgs sa{};
+  sa.q = (const uint16_t*)q;
+  sa.q_stride = q_stride;
+  sa.kc = (const uint16_t*)k_cache;
+  sa.vc = (const uint16_t*)v_cache;
+  sa.row_stride = cache_stride_n;
+  sa.slots = ctx_slots;
+  sa.offsets = offsets;
+  sa.lens = lens;
+  sa.shared_len = -1;
+  sa.chunk = p.chunk;
+  sa.n_chunks = p.n_chunks;
+  sa.part_base = 0;
+  sa.opart = ws.opart;
+  sa.ml = ws.ml;
+  sa.B = T;
+  sa.H = H;
+  sa.req_begin = 0;
+  sa.num_reqs = T;
+  sa.scale_log2e = scale * kLog2e;
+  if ((rc = launch_partial(sa, dtype, D, st)) != PH_OK) return rc;
+  MergeArgs ma{};
+  ma.opart = ws.opart;
+  ma.ml = ws.ml;
+  ma.out = (uint16_t*)out;
+  ma.out_stride = out_stride;
+  ma.B = T;
+  ma.H = H;
+  ma.nA = 0;
+  ma.baseB = 0;
+  ma.lens = lens;
+  ma.chunk = p.chunk;
+  return launch_merge(ma, dtype, D, st);
+}

@@ -1,0 +1,102 @@
+// Shared device helpers for the gfx950 kernels: 16-bit element traits,
+// 128-bit vector I/O, wave64 reductions, launch checks.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/parrot_hip.h"
+
+namespace ph {
+
+constexpr int kWave = 64;
+constexpr float kLog2e = 1.4426950408889634f;
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+struct F16 {};   // IEEE binary16
+struct BF16 {};  // bfloat16
+
+template <typename E>
+struct Elem;
+
+template <>
+struct Elem<F16> {
+  static __device__ __forceinline__ float lo(uint32_t w) {
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xffffu));
+  }
+  static __device__ __forceinline__ float hi(uint32_t w) {
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16));
+  }
+  static __device__ __forceinline__ float one(uint16_t b) { return (float)__builtin_bit_cast(_Float16, b); }
+  static __device__ __forceinline__ uint16_t bits(float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }
+  // acc + a.lo*b.lo + a.hi*b.hi with fp32 accumulate (v_dot2_f32_f16)
+  static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float acc) {
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, a), __builtin_bit_cast(half2_t, b), acc, false);
+  }
+};
+
+template <>
+struct Elem<BF16> {
+  static __device__ __forceinline__ float lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
+  static __device__ __forceinline__ float hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
+  static __device__ __forceinline__ float one(uint16_t b) { return __builtin_bit_cast(float, (uint32_t)b << 16); }
+  static __device__ __forceinline__ uint16_t bits(float f) {  // round to nearest even
+    uint32_t u = __builtin_bit_cast(uint32_t, f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);  // quiet NaN
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+  }
+  static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float acc) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), acc, false);
+  }
+};
+
+template <typename E>
+__device__ __forceinline__ uint32_t pack2(float a, float b) {
+  return (uint32_t)Elem<E>::bits(a) | ((uint32_t)Elem<E>::bits(b) << 16);
+}
+
+// Round a float to the element type and back (the "t(.)" of the reference's
+// element-type arithmetic).
+template <typename E>
+__device__ __forceinline__ float rnd(float f) {
+  return Elem<E>::one(Elem<E>::bits(f));
+}
+
+__device__ __forceinline__ u32x4 ld16(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
+__device__ __forceinline__ void st16(void* p, u32x4 v) { *reinterpret_cast<u32x4*>(p) = v; }
+__device__ __forceinline__ u32x4 ld16_nt(const void* p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+}
+__device__ __forceinline__ void st16_nt(void* p, u32x4 v) {
+  __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
+}
+
+// Butterfly sum over aligned groups of W lanes (W a power of two <= 64); every
+// lane of the group ends with the group's sum.
+template <int W>
+__device__ __forceinline__ float group_sum(float v) {
+#pragma unroll
+  for (int s = W / 2; s >= 1; s >>= 1) v += __shfl_xor(v, s, kWave);
+  return v;
+}
+template <int W>
+__device__ __forceinline__ float group_max(float v) {
+#pragma unroll
+  for (int s = W / 2; s >= 1; s >>= 1) v = fmaxf(v, __shfl_xor(v, s, kWave));
+  return v;
+}
+
+inline int launch_status() { return hipGetLastError() == hipSuccess ? PH_OK : PH_ERR_LAUNCH; }
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace ph

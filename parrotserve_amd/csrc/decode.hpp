@@ -1,0 +1,74 @@
+// Argument blocks shared by the decode-attention kernels and their host entry
+// points.  Partials live in a caller-provided workspace:
+//   opart [parts, B, H, D] fp32 (normalised O of each part)
+//   ml    [parts, B, H, 2] fp32 (m in the exp2 domain, l; l == 0 marks an empty part)
+#pragma once
+
+#include "common.hpp"
+
+namespace ph {
+
+struct PartialArgs {
+  const uint16_t* q;
+  int64_t q_stride;
+  const uint16_t* kc;
+  const uint16_t* vc;
+  int64_t row_stride;       // elements between consecutive slots
+  const int32_t* slots;     // slot table base
+  const int64_t* offsets;   // per-request start inside `slots`, or null
+  int64_t table_stride;     // start = b * table_stride when offsets is null
+  const int32_t* lens;      // per-request list length
+  const int32_t* shared_cu; // if set: every request uses slots[cu[0] .. cu[1])
+  int shared_len;           // if >= 0 (and shared_cu null): every request uses slots[0 .. shared_len)
+  int chunk;                // tokens per part
+  int n_chunks;             // parts per request in this launch (grid extent)
+  int part_base;            // first part index written
+  float* opart;
+  float* ml;
+  int B, H;                 // full batch size / head count (workspace extents)
+  int req_begin, num_reqs;  // requests covered by this launch
+  float scale_log2e;
+};
+
+struct MergeArgs {
+  const float* opart;
+  const float* ml;
+  uint16_t* out;
+  int64_t out_stride;
+  int B, H;
+  int nA;                   // parts [0, nA) are candidates for every request
+  int baseB;                // parts [baseB, baseB + ceil(lens[b]/chunk)) likewise
+  const int32_t* lens;      // may be null (no B range)
+  int chunk;
+  const float* prev_m;      // optional partial already in out/prev_m/prev_l
+  const float* prev_l;
+  float* m_out;             // optional export of the merged m / l
+  float* l_out;
+};
+
+struct PrefixArgs {
+  const uint16_t* q;
+  int64_t q_stride;
+  const uint16_t* kc;
+  const uint16_t* vc;
+  int64_t row_stride;
+  const int32_t* slots;        // all groups' prefix slots
+  const int32_t* prefix_cu;    // [G+1] device
+  const int32_t* group_req_cu; // [G+1] device
+  int fixed_prefix_len;        // used when prefix_cu is null: one group, all requests, slots[0 .. len)
+  int split_tokens;            // tokens per split (multiple of the tile)
+  int n_splits;                // parts [0, n_splits)
+  float* opart;
+  float* ml;
+  int B, H;
+  float scale_log2e;
+};
+
+int launch_partial(const PartialArgs& a, int dtype, int D, hipStream_t st);
+int launch_merge(const MergeArgs& a, int dtype, int D, hipStream_t st);
+int launch_clear_ml(float* ml, int64_t entries, hipStream_t st);
+// MFMA shared-prefix kernel: grid (split, head, group x m-tile).
+int launch_prefix_mfma(const PrefixArgs& a, int dtype, int D, int num_groups, int max_group_reqs, hipStream_t st);
+bool prefix_mfma_supported(int dtype, int D);
+
+}  // namespace ph

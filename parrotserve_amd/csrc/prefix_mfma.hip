@@ -1,0 +1,316 @@
+// Shared-prefix flash-decoding on CDNA4 matrix cores.
+//
+// All queries of a group attend over the SAME prefix slots, so per head the
+// phase is a dense contraction: S^T = K Q^T (tokens x queries), O^T = V^T P^T.
+// Workgroup = (split of the prefix, head, group x 64-query tile), 4 waves.
+// Each wave owns every fourth 32-token tile of the split and ALL queries of
+// the tile, so each K/V byte is fetched from HBM once per (group, query tile)
+// and crosses LDS once: global -> registers (coalesced 128-bit gathers by slot)
+// -> wave-private LDS tile -> MFMA operand layout.  No workgroup barrier in
+// the main loop.  Online softmax in the exp2 domain, fp32 accumulation in
+// v_mfma_f32_32x32x16_{f16,bf16}.  The four waves' partials are folded through
+// LDS at the end and one (O, m, l) part per (split, request, head) is written.
+//
+// Operand layouts (lane = 32*h + r):
+//   A (32 x 16): lane holds row r, 8 contraction elements chosen by (h, step)
+//   B (16 x 32): lane holds column r, the same 8 contraction elements
+//   C (32 x 32): lane holds column r, rows 8*j + 4*h + i at register 4*j + i
+// The contraction index is a free permutation as long as A and B agree, which
+// lets the fp32 S^T registers feed the second product as its B operand with no
+// cross-lane movement: V^T is stored in LDS with tokens permuted to match.
+//
+// Math restated from parrot/engine/builtin/kernels/shared_flash_decoding.py:34-134.
+#include "decode.hpp"
+
+namespace ph {
+
+template <typename E>
+struct Mfma32;
+template <>
+struct Mfma32<F16> {
+  static __device__ __forceinline__ float16_t run(u32x4 a, u32x4 b, float16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, b), c,
+                                                  0, 0, 0);
+  }
+};
+template <>
+struct Mfma32<BF16> {
+  static __device__ __forceinline__ float16_t run(u32x4 a, u32x4 b, float16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b),
+                                                   c, 0, 0, 0);
+  }
+};
+
+constexpr int kPD = 128;             // head size handled by this kernel
+constexpr int kTile = 32;            // tokens per wave tile
+constexpr int kWaveLds = 16384;      // K tile 8 KB + V^T tile 8 KB
+constexpr int kVtOff = 8192;
+
+__device__ __forceinline__ u32x4 lds_ld16(const char* p) { return *reinterpret_cast<const u32x4*>(p); }
+
+// position of token t (0..31) inside a V^T row so that the 8 tokens a lane
+// needs for contraction step u sit in one 16-byte chunk
+__device__ __forceinline__ int vt_pos(int t) {
+  const int i = t & 3, hh = (t >> 2) & 1, j = t >> 3;
+  return (j >> 1) * 16 + hh * 8 + (j & 1) * 4 + i;
+}
+
+template <typename E, int NQB>
+__global__ __launch_bounds__(256, 1) void prefix_mfma_kernel(PrefixArgs a, int mtiles) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int split = blockIdx.x, head = blockIdx.y;
+  const int g = blockIdx.z / mtiles, mt = blockIdx.z - g * mtiles;
+  int r0 = 0, r1 = a.B, poff = 0, plen = a.fixed_prefix_len;
+  if (a.prefix_cu) {
+    r0 = a.group_req_cu[g];
+    r1 = a.group_req_cu[g + 1];
+    poff = a.prefix_cu[g];
+    plen = a.prefix_cu[g + 1] - poff;
+  }
+  const int qbase = r0 + mt * 32 * NQB;
+  const int nq = min(32 * NQB, r1 - qbase);
+  if (nq <= 0) return;
+  const int s0 = split * a.split_tokens;
+  const int s1 = min(plen, s0 + a.split_tokens);
+  if (s0 >= plen) {  // this group's prefix ends before the split: mark the part empty
+    for (int q = threadIdx.x; q < nq; q += 256) {
+      const int64_t pr = ((int64_t)split * a.B + qbase + q) * a.H + head;
+      a.ml[pr * 2] = -INFINITY;
+      a.ml[pr * 2 + 1] = 0.f;
+    }
+    return;
+  }
+
+  const int lane = threadIdx.x & 63;
+  const int w = threadIdx.x >> 6;
+  const int h = lane >> 5, ql = lane & 31;
+  char* wl = smem + w * kWaveLds;
+  const int32_t* slots = a.slots + poff;
+
+  // Q as the B operand: column = query ql (+32 nb), contraction chunk (h, s) = dims 64h + 8s .. +8
+  u32x4 qop[NQB][8];
+#pragma unroll
+  for (int nb = 0; nb < NQB; ++nb) {
+    const int q = 32 * nb + ql;
+    const bool ok = q < nq;
+    const uint16_t* qp = a.q + (int64_t)(qbase + (ok ? q : 0)) * a.q_stride + head * kPD + 64 * h;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      u32x4 v = ld16(qp + 8 * s);
+      if (!ok) v = u32x4{0, 0, 0, 0};
+      qop[nb][s] = v;
+    }
+  }
+
+  float16_t oacc[4][NQB];
+  float m[NQB], lsum[NQB];
+#pragma unroll
+  for (int nb = 0; nb < NQB; ++nb) {
+    m[nb] = -INFINITY;
+    lsum[nb] = 0.f;
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) oacc[db][nb][r] = 0.f;
+  }
+
+  // global -> register staging: instruction r covers tokens 4r .. 4r+3, 16 lanes per token row
+  const int tl = lane >> 4, c = lane & 15;
+  const int64_t col = (int64_t)head * kPD + c * 8;
+  u32x4 kreg[8], vreg[8];
+  int tb = s0 + kTile * w;
+  if (tb < s1) {
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      const int tok = min(tb + 4 * r + tl, s1 - 1);
+      const int64_t ro = (int64_t)slots[tok] * a.row_stride + col;
+      kreg[r] = ld16(a.kc + ro);
+      vreg[r] = ld16(a.vc + ro);
+    }
+  }
+
+  for (; tb < s1; tb += 4 * kTile) {
+    // registers -> LDS: K row-major with XOR-swizzled 16-byte chunks, V transposed
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      const int t = 4 * r + tl;
+      *reinterpret_cast<u32x4*>(wl + t * 256 + ((c ^ (t & 15)) * 16)) = kreg[r];
+      const int pos = vt_pos(t);
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const int d = 8 * c + k;
+        const uint16_t val = (uint16_t)(vreg[r][k >> 1] >> ((k & 1) * 16));
+        *reinterpret_cast<uint16_t*>(wl + kVtOff + d * 64 + (((pos >> 3) ^ ((d >> 2) & 3)) * 16) + (pos & 7) * 2) =
+            val;
+      }
+    }
+    // prefetch the wave's next tile while this one is consumed
+    const int nt = tb + 4 * kTile;
+    if (nt < s1) {
+#pragma unroll
+      for (int r = 0; r < 8; ++r) {
+        const int tok = min(nt + 4 * r + tl, s1 - 1);
+        const int64_t ro = (int64_t)slots[tok] * a.row_stride + col;
+        kreg[r] = ld16(a.kc + ro);
+        vreg[r] = ld16(a.vc + ro);
+      }
+    }
+
+    // S^T = K Q^T
+    float16_t sacc[NQB];
+#pragma unroll
+    for (int nb = 0; nb < NQB; ++nb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sacc[nb][r] = 0.f;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      const u32x4 ka = lds_ld16(wl + ql * 256 + (((8 * h + s) ^ (ql & 15)) * 16));
+#pragma unroll
+      for (int nb = 0; nb < NQB; ++nb) sacc[nb] = Mfma32<E>::run(ka, qop[nb][s], sacc[nb]);
+    }
+
+    // online softmax; P^T packed straight into B-operand form
+    u32x4 pop[NQB][2];
+#pragma unroll
+    for (int nb = 0; nb < NQB; ++nb) {
+      float x[16];
+      float mloc = -INFINITY;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int t = 8 * (r >> 2) + 4 * h + (r & 3);
+        x[r] = (tb + t < s1) ? sacc[nb][r] * a.scale_log2e : -INFINITY;
+        mloc = fmaxf(mloc, x[r]);
+      }
+      mloc = fmaxf(mloc, __shfl_xor(mloc, 32, kWave));
+      const float mn = fmaxf(m[nb], mloc);
+      const float alpha = __builtin_amdgcn_exp2f(m[nb] - mn);
+      m[nb] = mn;
+      float ps = 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        x[r] = __builtin_amdgcn_exp2f(x[r] - mn);
+        ps += x[r];
+      }
+      lsum[nb] = lsum[nb] * alpha + ps;
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[db][nb][r] *= alpha;
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) pop[nb][u][e] = pack2<E>(x[8 * u + 2 * e], x[8 * u + 2 * e + 1]);
+    }
+
+    // O^T += V^T P^T
+#pragma unroll
+    for (int db = 0; db < 4; ++db) {
+      const int d = 32 * db + ql;
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const u32x4 va = lds_ld16(wl + kVtOff + d * 64 + (((2 * u + h) ^ ((d >> 2) & 3)) * 16));
+#pragma unroll
+        for (int nb = 0; nb < NQB; ++nb) oacc[db][nb] = Mfma32<E>::run(va, pop[nb][u], oacc[db][nb]);
+      }
+    }
+  }
+
+  // fold the four waves: (2,3) -> (0,1), then 1 -> 0
+  constexpr int kDump = (4 * NQB * 16 + 2 * NQB) * 64 * 4;  // bytes per dumped wave
+  auto dump = [&](char* base) {
+    float* f = reinterpret_cast<float*>(base);
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int nb = 0; nb < NQB; ++nb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) f[((db * NQB + nb) * 16 + r) * 64 + lane] = oacc[db][nb][r];
+#pragma unroll
+    for (int nb = 0; nb < NQB; ++nb) {
+      f[(4 * NQB * 16 + nb) * 64 + lane] = m[nb];
+      f[(4 * NQB * 16 + NQB + nb) * 64 + lane] = lsum[nb];
+    }
+  };
+  auto fold = [&](const char* base) {
+    const float* f = reinterpret_cast<const float*>(base);
+#pragma unroll
+    for (int nb = 0; nb < NQB; ++nb) {
+      const float mo = f[(4 * NQB * 16 + nb) * 64 + lane];
+      const float lo = f[(4 * NQB * 16 + NQB + nb) * 64 + lane];
+      const float mn = fmaxf(m[nb], mo);
+      const float sa = (m[nb] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m[nb] - mn);
+      const float sb = (mo == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mo - mn);
+      m[nb] = mn;
+      lsum[nb] = lsum[nb] * sa + lo * sb;
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          oacc[db][nb][r] = oacc[db][nb][r] * sa + f[((db * NQB + nb) * 16 + r) * 64 + lane] * sb;
+    }
+  };
+  __syncthreads();
+  if (w >= 2) dump(smem + (w - 2) * kDump);
+  __syncthreads();
+  if (w < 2) fold(smem + w * kDump);
+  __syncthreads();
+  if (w == 1) dump(smem);
+  __syncthreads();
+  if (w != 0) return;
+  fold(smem);
+
+#pragma unroll
+  for (int nb = 0; nb < NQB; ++nb) {
+    const float L = lsum[nb] + __shfl_xor(lsum[nb], 32, kWave);
+    const int q = 32 * nb + ql;
+    if (q < nq) {
+      const float inv = 1.f / L;
+      const int64_t pr = ((int64_t)split * a.B + qbase + q) * a.H + head;
+      float* op = a.opart + pr * kPD;
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          float4_t v = {oacc[db][nb][4 * j] * inv, oacc[db][nb][4 * j + 1] * inv, oacc[db][nb][4 * j + 2] * inv,
+                        oacc[db][nb][4 * j + 3] * inv};
+          *reinterpret_cast<float4_t*>(op + 32 * db + 8 * j + 4 * h) = v;
+        }
+      if (h == 0) {
+        a.ml[pr * 2] = m[nb];
+        a.ml[pr * 2 + 1] = L;
+      }
+    }
+  }
+}
+
+template <typename E>
+static int launch_prefix_t(const PrefixArgs& a, int num_groups, int max_group_reqs, hipStream_t st) {
+  const int nqb = max_group_reqs <= 32 ? 1 : 2;
+  const int mtiles = (max_group_reqs + 32 * nqb - 1) / (32 * nqb);
+  dim3 grid(a.n_splits, a.H, num_groups * mtiles), block(256);
+  if (nqb == 1) {
+    constexpr int lds = 4 * kWaveLds > 2 * (4 * 1 * 16 + 2) * 256 ? 4 * kWaveLds : 2 * (4 * 1 * 16 + 2) * 256;
+    hipLaunchKernelGGL((prefix_mfma_kernel<E, 1>), grid, block, lds, st, a, mtiles);
+  } else {
+    constexpr int lds = 4 * kWaveLds > 2 * (4 * 2 * 16 + 4) * 256 ? 4 * kWaveLds : 2 * (4 * 2 * 16 + 4) * 256;
+    static bool attr_set = false;
+    if (!attr_set) {
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&prefix_mfma_kernel<E, 2>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+      attr_set = true;
+    }
+    hipLaunchKernelGGL((prefix_mfma_kernel<E, 2>), grid, block, lds, st, a, mtiles);
+  }
+  return launch_status();
+}
+
+bool prefix_mfma_supported(int dtype, int D) { return D == kPD && (dtype == PH_F16 || dtype == PH_BF16); }
+
+int launch_prefix_mfma(const PrefixArgs& a, int dtype, int D, int num_groups, int max_group_reqs, hipStream_t st) {
+  if (D != kPD) return PH_ERR_HEAD_DIM;
+  if (num_groups <= 0 || max_group_reqs <= 0 || a.n_splits <= 0) return PH_OK;
+  return dtype == PH_F16 ? launch_prefix_t<F16>(a, num_groups, max_group_reqs, st)
+                         : launch_prefix_t<BF16>(a, num_groups, max_group_reqs, st);
+}
+
+}  // namespace ph

@@ -1,0 +1,456 @@
+"""Kernel surface of Parrot's builtin engine, backed by libparrot_hip.so.
+
+Same names, argument order and in-place behaviour as
+``parrot/engine/builtin/kernels/__init__.py:7-16`` of the reference, on the
+token-granular KV layout ``[slots, H, D]`` (``MemLayout.NORMAL`` with
+``block_size == 1``, parrot/engine/builtin/mem.py:43-56): a block table is a
+list of slot ids and a context length is its row count.
+
+Every function launches hand-written HIP kernels through the C ABI on the
+current torch stream.  torch is used for device memory and streams only; there
+is no PyTorch fallback.
+"""
+from __future__ import annotations
+
+import dataclasses
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import PH_BF16, PH_F16, PH_IDX_I32, PH_IDX_I64, check
+
+__all__ = [
+    "discontinuous_move_tokens",
+    "move_tokens_from_blocked_k_cache",
+    "move_tokens_from_blocked_v_cache",
+    "rotary_embedding",
+    "rmsnorm_forward",
+    "vllm_paged_attention",
+    "vllm_reshape_and_cache",
+    "vllm_rms_norm",
+    "vllm_rotary_emb",
+    "flash_paged_attention",
+    "paged_flash_attention",
+    "DecodeTables",
+    "PrefillTables",
+    "decode_attention",
+    "prefill_attention",
+    "kv_append",
+]
+
+
+# --------------------------------------------------------------------------- #
+# plumbing
+# --------------------------------------------------------------------------- #
+def _dtype_code(t: torch.Tensor) -> int:
+    if t.dtype == torch.float16:
+        return PH_F16
+    if t.dtype == torch.bfloat16:
+        return PH_BF16
+    # TORCH_CHECK(false, "Unsupported data type") in the reference's launcher
+    raise RuntimeError(f"Unsupported data type: {t.dtype}")
+
+
+def _index_code(t: torch.Tensor) -> int:
+    if t.dtype == torch.int32:
+        return PH_IDX_I32
+    if t.dtype == torch.int64:
+        return PH_IDX_I64
+    raise ValueError(f"index tensor must be int32 or int64, got {t.dtype}")
+
+
+def _require_gpu(*ts: torch.Tensor) -> torch.device:
+    dev = None
+    for t in ts:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise RuntimeError("parrotserve_amd kernels run on the GPU only; got a CPU tensor (no CPU fallback)")
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise ValueError("all tensors must live on the same device")
+    return dev
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+_workspaces: Dict[Tuple[int, int], torch.Tensor] = {}
+
+
+def _workspace(nbytes: int, device: torch.device) -> torch.Tensor:
+    """Grow-only scratch buffer per (device, stream); reuse is ordered by the stream."""
+    key = (device.index or 0, _stream())
+    buf = _workspaces.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _workspaces[key] = buf
+    return buf
+
+
+# --------------------------------------------------------------------------- #
+# token move / KV append
+# --------------------------------------------------------------------------- #
+@torch.inference_mode()
+def discontinuous_move_tokens(src_storage, dest_storage, src_indices, dest_indices):
+    """``dest_storage[dest_indices[i]] = src_storage[src_indices[i]]``
+    (parrot/engine/builtin/kernels/tokens_moving.py:67-100).  Storages are
+    ``[tokens, H, D]`` with free strides; indices are int64 or int32 ``[n]``."""
+    assert src_indices.shape == dest_indices.shape, "src_indices and dest_indices must have the same shape"
+    assert dest_storage.shape[1:] == src_storage.shape[1:], "storage shape mismatch"
+    assert src_storage.dtype == dest_storage.dtype, "storage dtype mismatch"
+    assert src_indices.dtype == dest_indices.dtype, "index dtype mismatch"
+    _require_gpu(src_storage, dest_storage, src_indices, dest_indices)
+    src_indices = src_indices.contiguous()
+    dest_indices = dest_indices.contiguous()
+    n = src_indices.shape[0]
+    num_heads, head_dim = src_storage.shape[1:]
+    rc = _lib.load().ph_move_tokens(
+        _ptr(src_storage), _ptr(dest_storage), _ptr(src_indices), _ptr(dest_indices), _index_code(src_indices),
+        n, num_heads, head_dim, src_storage.element_size(),
+        src_storage.stride(0), src_storage.stride(1), src_storage.stride(2),
+        dest_storage.stride(0), dest_storage.stride(1), dest_storage.stride(2), _stream())
+    check(rc, "discontinuous_move_tokens")
+
+
+def _move_from_cache(cache, dest_storage, src_slot_indices, dest_indices, name):
+    if cache.dim() != 3:
+        raise ValueError(
+            f"{name}: only the token-granular cache layout [slots, H, D] is supported "
+            f"(got a {cache.dim()}-d cache; the blocked vLLM layouts are not used by this build)")
+    discontinuous_move_tokens(cache, dest_storage, src_slot_indices, dest_indices)
+
+
+def move_tokens_from_blocked_k_cache(blocked_k_cache, dest_storage, src_slot_indices, dest_indices):
+    """Gather token rows of the K cache by slot id into ``dest_storage``
+    (parrot/engine/builtin/kernels/tokens_moving.py:104-218).  With
+    ``block_size == 1`` the blocked K layout degenerates to ``[slots, H, D]``,
+    the only layout accepted here."""
+    _move_from_cache(blocked_k_cache, dest_storage, src_slot_indices, dest_indices, "move_tokens_from_blocked_k_cache")
+
+
+def move_tokens_from_blocked_v_cache(blocked_v_cache, dest_storage, src_slot_indices, dest_indices):
+    """V twin of the above (tokens_moving.py:222-313)."""
+    _move_from_cache(blocked_v_cache, dest_storage, src_slot_indices, dest_indices, "move_tokens_from_blocked_v_cache")
+
+
+@torch.inference_mode()
+def kv_append(key, value, key_cache, value_cache, slot_mapping):
+    """``key_cache[slot[t]] = key[t]`` and the same for V, one launch."""
+    assert key.shape == value.shape and key.dim() == 3
+    assert key_cache.shape == value_cache.shape and key_cache.dim() == 3
+    assert key.shape[1:] == key_cache.shape[1:], "head shape mismatch"
+    assert key.dtype == value.dtype == key_cache.dtype == value_cache.dtype
+    _require_gpu(key, value, key_cache, value_cache, slot_mapping)
+    slot_mapping = slot_mapping.reshape(-1).contiguous()
+    T, H, D = key.shape
+    assert slot_mapping.shape[0] == T, "slot_mapping must hold one slot per token"
+    for t in (key, value, key_cache, value_cache):
+        assert t.stride(2) == 1 and t.stride(1) == D, "heads of a token must be contiguous"
+    assert key_cache.stride(0) == value_cache.stride(0)
+    rc = _lib.load().ph_kv_append(
+        _ptr(key), _ptr(value), _ptr(key_cache), _ptr(value_cache), _ptr(slot_mapping), _index_code(slot_mapping),
+        T, H, D, _dtype_code(key), key.stride(0), value.stride(0), key_cache.stride(0), _stream())
+    check(rc, "kv_append")
+
+
+def vllm_reshape_and_cache(key_to_cache, value_to_cache, key_cache, value_cache, slot_mapping):
+    """``cache_ops.reshape_and_cache`` on the token-granular layout
+    (parrot/engine/builtin/kernels/vllm/reshape_and_cache.py:9-22)."""
+    kv_append(key_to_cache, value_to_cache, key_cache, value_cache, slot_mapping)
+
+
+# --------------------------------------------------------------------------- #
+# RMSNorm / RoPE
+# --------------------------------------------------------------------------- #
+def _rms(x, weight, eps, round_first, name):
+    _require_gpu(x, weight)
+    assert x.shape[-1] == weight.shape[0], "weight size mismatch"
+    assert x.dtype == weight.dtype, "weight dtype mismatch"
+    x2 = x.reshape(-1, x.shape[-1])
+    if x2.stride(1) != 1:
+        x2 = x2.contiguous()
+    out = torch.empty((x2.shape[0], x2.shape[1]), dtype=x.dtype, device=x.device)
+    rc = _lib.load().ph_rms_norm(_ptr(out), _ptr(x2), _ptr(weight.contiguous()), float(eps), x2.shape[0], x2.shape[1],
+                                 x2.stride(0), out.stride(0), _dtype_code(x), int(round_first), _stream())
+    check(rc, name)
+    return out.view(x.shape)
+
+
+@torch.inference_mode()
+def vllm_rms_norm(input, weight, eps):
+    """``layernorm_ops.rms_norm`` (parrot/engine/builtin/kernels/vllm/rms_norm.py:9-16):
+    the normalised value is rounded to the element type before the weight multiply."""
+    return _rms(input, weight, eps, True, "vllm_rms_norm")
+
+
+@torch.inference_mode()
+def rmsnorm_forward(x, weight, eps):
+    """Triton twin (parrot/engine/builtin/kernels/rms_norm.py:49-78): fp32 math, one rounding."""
+    return _rms(x, weight, eps, False, "rmsnorm_forward")
+
+
+@torch.inference_mode()
+def vllm_rotary_emb(positions, query, key, cos_sin_cache, head_size):
+    """NeoX rotary embedding of ``query`` and ``key`` in place
+    (parrot/engine/builtin/kernels/vllm/rotary_embed.py:10-25).  query / key are
+    ``[T, heads*head_size]`` and may be row-strided chunk views of a fused qkv."""
+    _require_gpu(positions, query, key, cos_sin_cache)
+    assert positions.dtype == torch.int64, "positions must be int64"
+    assert query.dim() == 2 and key.dim() == 2 and query.stride(1) == 1 and key.stride(1) == 1
+    assert query.dtype == key.dtype == cos_sin_cache.dtype
+    T = positions.shape[0]
+    assert query.shape[0] == T and key.shape[0] == T
+    assert cos_sin_cache.is_contiguous()
+    rc = _lib.load().ph_rope_neox(
+        _ptr(positions.contiguous()), _ptr(query), _ptr(key), _ptr(cos_sin_cache), T,
+        query.shape[1] // head_size, key.shape[1] // head_size, head_size, cos_sin_cache.shape[1],
+        query.stride(0), key.stride(0), _dtype_code(query), _stream())
+    check(rc, "vllm_rotary_emb")
+
+
+@torch.inference_mode()
+def rotary_embedding(state, cos, sin):
+    """In-place NeoX rotation of ``state [T, H, D]`` with per-token ``cos``,
+    ``sin`` of shape ``[T, 1, D/2]`` (parrot/engine/builtin/kernels/rotary_embedding.py:107-143)."""
+    _require_gpu(state, cos, sin)
+    assert state.dim() == 3 and state.stride(2) == 1
+    T, H, D = state.shape
+    assert cos.shape == sin.shape == (T, 1, D // 2), "cos/sin must be [T, 1, D/2]"
+    assert cos.dtype == sin.dtype == state.dtype
+    assert cos.stride(2) == 1 and sin.stride(2) == 1 and cos.stride(0) == sin.stride(0)
+    rc = _lib.load().ph_rotary_embedding(_ptr(state), _ptr(cos), _ptr(sin), T, H, D, state.stride(0), state.stride(1),
+                                         cos.stride(0), _dtype_code(state), _stream())
+    check(rc, "rotary_embedding")
+
+
+# --------------------------------------------------------------------------- #
+# decode attention
+# --------------------------------------------------------------------------- #
+@dataclasses.dataclass
+class DecodeTables:
+    """Per-iteration slot tables of the decode requests (built once, used by
+    every layer).  Device tensors are int32 unless noted."""
+
+    num_reqs: int
+    # prefix groups
+    num_groups: int = 0
+    prefix_slots: Optional[torch.Tensor] = None  # all groups back to back
+    prefix_cu: Optional[torch.Tensor] = None  # [G+1] device
+    group_req_cu: Optional[torch.Tensor] = None  # [G+1] device
+    group_req_cu_host: Optional[torch.Tensor] = None  # [G+1] CPU int32
+    max_prefix_len: int = 0
+    # per-request suffix
+    suffix_slots: Optional[torch.Tensor] = None  # ragged (with offsets) or [B, max] padded
+    suffix_offsets: Optional[torch.Tensor] = None  # int64 [B] device, None for a padded table
+    suffix_table_stride: int = 0
+    suffix_lens: Optional[torch.Tensor] = None  # [B] device
+    max_suffix_len: int = 0
+    chunk_tokens: int = 0  # 0 = let the library choose
+
+    @staticmethod
+    def build(prefix_lists: Sequence[Sequence[int]], group_req_cu: Sequence[int],
+              suffix_lists: Sequence[Sequence[int]], device) -> "DecodeTables":
+        """From python lists: ``prefix_lists[g]`` is group g's slot list shared by
+        requests ``group_req_cu[g] .. group_req_cu[g+1]-1``; ``suffix_lists[b]`` is
+        request b's own slot list."""
+        B = len(suffix_lists)
+        t = DecodeTables(num_reqs=B)
+        G = len(prefix_lists)
+        if G > 0:
+            assert len(group_req_cu) == G + 1
+            cu = [0]
+            flat: List[int] = []
+            for p in prefix_lists:
+                flat.extend(p)
+                cu.append(len(flat))
+            t.num_groups = G
+            t.max_prefix_len = max(len(p) for p in prefix_lists)
+            t.prefix_slots = torch.tensor(flat if flat else [0], dtype=torch.int32, device=device)
+            t.prefix_cu = torch.tensor(cu, dtype=torch.int32, device=device)
+            t.group_req_cu_host = torch.tensor(list(group_req_cu), dtype=torch.int32)
+            t.group_req_cu = t.group_req_cu_host.to(device)
+        lens = [len(s) for s in suffix_lists]
+        t.max_suffix_len = max(lens) if lens else 0
+        total = sum(lens)
+        if t.max_suffix_len > 0:
+            flat = [x for s in suffix_lists for x in s]
+            offs = [0] * B
+            acc = 0
+            for i, n in enumerate(lens):
+                offs[i] = acc
+                acc += n
+            t.suffix_slots = torch.tensor(flat, dtype=torch.int32, device=device)
+            t.suffix_offsets = torch.tensor(offs, dtype=torch.int64, device=device)
+            t.suffix_lens = torch.tensor(lens, dtype=torch.int32, device=device)
+            # parts of about 1/2048 of the batch's tokens, 32 .. 1024 tokens each
+            chunk = 32
+            while chunk < total // 2048 and chunk < 1024:
+                chunk *= 2
+            t.chunk_tokens = chunk
+        return t
+
+
+@torch.inference_mode()
+def decode_attention(query: torch.Tensor, key_cache: torch.Tensor, value_cache: torch.Tensor, tables: DecodeTables,
+                     scale: Optional[float] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Shared-prefix (or plain ragged) decode attention: prefix phase on the
+    matrix cores, per-request suffix phase, log-sum-exp merge."""
+    _require_gpu(query, key_cache, value_cache)
+    assert query.dim() == 3 and key_cache.dim() == 3 and value_cache.shape == key_cache.shape
+    B, H, D = query.shape
+    assert B == tables.num_reqs
+    assert key_cache.shape[1:] == (H, D), "cache head shape mismatch"
+    assert query.dtype == key_cache.dtype == value_cache.dtype
+    assert query.stride(2) == 1 and query.stride(1) == D
+    assert key_cache.stride(2) == 1 and key_cache.stride(1) == D and key_cache.stride() == value_cache.stride()
+    if out is None:
+        out = torch.empty((B, H, D), dtype=query.dtype, device=query.device)
+    if B == 0:
+        return out
+    scale = D ** -0.5 if scale is None else scale
+    lib = _lib.load()
+    nbytes = lib.ph_decode_workspace_bytes(B, H, D, tables.num_groups, tables.max_prefix_len, tables.max_suffix_len,
+                                           tables.chunk_tokens)
+    ws = _workspace(nbytes, query.device)
+    rc = lib.ph_decode_attention(
+        _ptr(out), _ptr(query), _ptr(key_cache), _ptr(value_cache), B, H, D, _dtype_code(query),
+        query.stride(0), out.stride(0), key_cache.stride(0), float(scale),
+        tables.num_groups, _ptr(tables.prefix_slots), _ptr(tables.prefix_cu), _ptr(tables.group_req_cu),
+        _ptr(tables.group_req_cu_host), tables.max_prefix_len,
+        _ptr(tables.suffix_slots), _ptr(tables.suffix_offsets), tables.suffix_table_stride, _ptr(tables.suffix_lens),
+        tables.max_suffix_len, tables.chunk_tokens, _ptr(ws), ws.numel(), _stream())
+    check(rc, "decode_attention")
+    return out
+
+
+_small_cache: Dict[Tuple, Tuple[torch.Tensor, torch.Tensor, torch.Tensor]] = {}
+
+
+def _single_group_cu(P: int, B: int, device) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    key = (P, B, str(device))
+    hit = _small_cache.get(key)
+    if hit is None:
+        if len(_small_cache) > 256:
+            _small_cache.clear()
+        host = torch.tensor([0, B], dtype=torch.int32)
+        hit = (torch.tensor([0, P], dtype=torch.int32, device=device), host.to(device), host)
+        _small_cache[key] = hit
+    return hit
+
+
+def _check_paged_args(query, key_cache, value_cache, head_mapping, context_lens, block_tables):
+    if key_cache.dim() != 3 or value_cache.dim() != 3:
+        raise ValueError("key_cache / value_cache must be token-granular [slots, H, D] (block_size 1)")
+    assert head_mapping.shape[0] == query.shape[1], "head_mapping must have one entry per head (MQA/GQA unsupported)"
+    assert block_tables.dim() == 2 and block_tables.dtype == torch.int32
+    assert context_lens.dtype == torch.int32 and context_lens.shape[0] == query.shape[0]
+    assert block_tables.shape[0] == query.shape[0]
+
+
+@torch.inference_mode()
+def vllm_paged_attention(query, key_cache, value_cache, head_mapping, context_lens, block_tables):
+    """Non-shared ragged decode (parrot/engine/builtin/kernels/vllm/paged_attention.py:12-38):
+    request i attends over ``block_tables[i, :context_lens[i]]``."""
+    _check_paged_args(query, key_cache, value_cache, head_mapping, context_lens, block_tables)
+    block_tables = block_tables if block_tables.stride(1) == 1 else block_tables.contiguous()
+    t = DecodeTables(num_reqs=query.shape[0], suffix_slots=block_tables, suffix_offsets=None,
+                     suffix_table_stride=block_tables.stride(0), suffix_lens=context_lens.contiguous(),
+                     max_suffix_len=block_tables.shape[1])
+    return decode_attention(query, key_cache, value_cache, t)
+
+
+@torch.inference_mode()
+def flash_paged_attention(query, key_cache, value_cache, head_mapping, flash_context_len, flash_block_table,
+                          paged_context_lens, paged_block_tables):
+    """Shared-prefix decode (parrot/engine/builtin/kernels/shared_flash_decoding.py:285-329):
+    all requests attend over ``flash_block_table[:flash_context_len]`` plus their
+    own ``paged_block_tables[i, :paged_context_lens[i]]``."""
+    _check_paged_args(query, key_cache, value_cache, head_mapping, paged_context_lens, paged_block_tables)
+    B = query.shape[0]
+    P = int(flash_context_len)
+    paged_block_tables = paged_block_tables if paged_block_tables.stride(1) == 1 else paged_block_tables.contiguous()
+    t = DecodeTables(num_reqs=B, suffix_slots=paged_block_tables, suffix_offsets=None,
+                     suffix_table_stride=paged_block_tables.stride(0), suffix_lens=paged_context_lens.contiguous(),
+                     max_suffix_len=paged_block_tables.shape[1])
+    if P > 0:
+        assert flash_block_table.dtype == torch.int32 and flash_block_table.numel() >= P
+        cu, gcu, gcu_host = _single_group_cu(P, B, query.device)
+        t.num_groups = 1
+        t.prefix_slots = flash_block_table.contiguous()
+        t.prefix_cu, t.group_req_cu, t.group_req_cu_host = cu, gcu, gcu_host
+        t.max_prefix_len = P
+    return decode_attention(query, key_cache, value_cache, t)
+
+
+def paged_flash_attention(query, key_cache, value_cache, head_mapping, flash_context_len, flash_block_table,
+                          paged_context_lens, paged_block_tables):
+    """Same result with the phases in the other order in the reference
+    (shared_flash_decoding.py:332-376); here both names run the same launches."""
+    return flash_paged_attention(query, key_cache, value_cache, head_mapping, flash_context_len, flash_block_table,
+                                 paged_context_lens, paged_block_tables)
+
+
+# --------------------------------------------------------------------------- #
+# prefill with parent context
+# --------------------------------------------------------------------------- #
+@dataclasses.dataclass
+class PrefillTables:
+    num_tokens: int
+    num_chunks: int
+    q_cu: torch.Tensor  # int32 [C+1] device
+    kv_cu: torch.Tensor  # int32 [C+1] device
+    ctx_slots: torch.Tensor  # int32 device
+    max_kv_len: int
+
+    @staticmethod
+    def build(q_lens: Sequence[int], ctx_slot_lists: Sequence[Sequence[int]], device) -> "PrefillTables":
+        q_cu, kv_cu, flat = [0], [0], []
+        for n, s in zip(q_lens, ctx_slot_lists):
+            assert len(s) >= n, "a chunk's context must include its own tokens"
+            q_cu.append(q_cu[-1] + n)
+            flat.extend(s)
+            kv_cu.append(len(flat))
+        return PrefillTables(
+            num_tokens=q_cu[-1], num_chunks=len(q_lens),
+            q_cu=torch.tensor(q_cu, dtype=torch.int32, device=device),
+            kv_cu=torch.tensor(kv_cu, dtype=torch.int32, device=device),
+            ctx_slots=torch.tensor(flat if flat else [0], dtype=torch.int32, device=device),
+            max_kv_len=max((len(s) for s in ctx_slot_lists), default=0))
+
+
+@torch.inference_mode()
+def prefill_attention(query, key_cache, value_cache, tables: PrefillTables, scale: Optional[float] = None,
+                      out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Packed ragged prefill, each chunk causal (bottom-right aligned) over its
+    ancestors' and its own KV read through the slot table -- the op the
+    reference assembles from a gather plus xformers' block-diagonal FMHA
+    (parrot/engine/builtin/attn_func.py:635-674)."""
+    _require_gpu(query, key_cache, value_cache)
+    T, H, D = query.shape
+    assert T == tables.num_tokens
+    assert key_cache.shape[1:] == (H, D) and value_cache.shape == key_cache.shape
+    assert query.dtype == key_cache.dtype == value_cache.dtype
+    assert query.stride(2) == 1 and query.stride(1) == D
+    assert key_cache.stride(2) == 1 and key_cache.stride(1) == D and key_cache.stride() == value_cache.stride()
+    if out is None:
+        out = torch.empty((T, H, D), dtype=query.dtype, device=query.device)
+    if T == 0:
+        return out
+    scale = D ** -0.5 if scale is None else scale
+    lib = _lib.load()
+    nbytes = lib.ph_prefill_workspace_bytes(T, H, D, tables.max_kv_len)
+    ws = _workspace(nbytes, query.device)
+    rc = lib.ph_prefill_attention(
+        _ptr(out), _ptr(query), _ptr(key_cache), _ptr(value_cache), T, tables.num_chunks, H, D, _dtype_code(query),
+        query.stride(0), out.stride(0), key_cache.stride(0), float(scale), _ptr(tables.q_cu), _ptr(tables.kv_cu),
+        _ptr(tables.ctx_slots), tables.max_kv_len, _ptr(ws), ws.numel(), _stream())
+    check(rc, "prefill_attention")
+    return out

@@ -1,0 +1,74 @@
+"""The C-ABI library loads and exports every symbol include/parrot_hip.h declares
+(no compute calls: this runs without a GPU)."""
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "parrot_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ph_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_bound_and_exported():
+    from parrotserve_amd import _lib
+
+    declared = _declared_symbols()
+    assert len(declared) >= 12
+    assert sorted(_lib.SIGNATURES) == declared, "ctypes table and header disagree"
+    lib = _lib.load()
+    for name in declared:
+        assert hasattr(lib, name), f"{name} not exported"
+
+
+def test_status_strings_and_version():
+    from parrotserve_amd import _lib
+
+    lib = _lib.load()
+    assert lib.ph_abi_version() >= 1
+    assert _lib.status_string(0) == "ok"
+    assert "head size" in _lib.status_string(_lib.PH_ERR_HEAD_DIM)
+    with pytest.raises(RuntimeError):
+        _lib.check(_lib.PH_ERR_DTYPE, "x")
+    with pytest.raises(ValueError):
+        _lib.check(_lib.PH_ERR_ARG, "x")
+
+
+def test_workspace_queries_are_host_only():
+    from parrotserve_amd import _lib
+
+    lib = _lib.load()
+    # C2 shape: B 64, H 32, D 128, one group, prefix 4096, suffix <= 512
+    n = lib.ph_decode_workspace_bytes(64, 32, 128, 1, 4096, 512, 32)
+    assert n > 0 and n % 256 == 0
+    assert lib.ph_decode_workspace_bytes(0, 32, 128, 1, 4096, 512, 32) == 0
+    assert lib.ph_prefill_workspace_bytes(1000, 40, 128, 3000) > 0
+
+
+def test_argument_validation_needs_no_gpu():
+    """Bad arguments are rejected before any launch."""
+    from parrotserve_amd import _lib
+
+    lib = _lib.load()
+    assert lib.ph_move_tokens(None, None, None, None, 0, 4, 2, 8, 3, 16, 8, 1, 16, 8, 1, None) == _lib.PH_ERR_DTYPE
+    assert lib.ph_move_tokens(None, None, None, None, 0, 4, 2, 8, 2, 16, 8, 1, 16, 8, 1, None) == _lib.PH_ERR_ARG
+    assert lib.ph_move_tokens(None, None, None, None, 0, 0, 2, 8, 2, 16, 8, 1, 16, 8, 1, None) == _lib.PH_OK
+    assert lib.ph_rms_norm(None, None, None, 1e-6, 4, 64, 64, 64, 7, 1, None) == _lib.PH_ERR_DTYPE
+    # unsupported head size mirrors the reference's "Unsupported head size" check
+    rc = lib.ph_decode_attention(1, 1, 1, 1, 4, 2, 80, 0, 160, 160, 160, 1.0, 0, None, None, None, None, 0,
+                                 None, None, 0, None, 0, 0, None, 0, None)
+    assert rc == _lib.PH_ERR_HEAD_DIM
+
+
+def test_cpu_tensors_are_refused_loudly():
+    import torch
+
+    from parrotserve_amd import kernels
+
+    x = torch.zeros(4, 64, dtype=torch.float16)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        kernels.vllm_rms_norm(x, torch.ones(64, dtype=torch.float16), 1e-6)

@@ -1,0 +1,198 @@
+"""GPU parity: token move / KV append (bit-exact), RoPE, RMSNorm vs the CPU oracle."""
+import pytest
+import torch
+
+from oracle.ref_ops import (ref_cos_sin_cache, ref_kv_append, ref_move_tokens, ref_rms_norm, ref_rope_neox,
+                            ref_rotary_embedding)
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float16: dict(atol=2e-3, rtol=1e-2), torch.bfloat16: dict(atol=1e-2, rtol=2e-2)}
+
+
+def _bits(t):
+    return t.contiguous().view(torch.int16) if t.element_size() == 2 else t.contiguous().view(torch.int32)
+
+
+@pytest.mark.parametrize("idx_dtype", [torch.int64, torch.int32])
+@pytest.mark.parametrize("H,D,dtype", [(32, 128, torch.float16), (40, 128, torch.bfloat16), (3, 20, torch.float16),
+                                        (2, 8, torch.float32)])
+def test_move_tokens_bit_exact(dev, idx_dtype, H, D, dtype):
+    from parrotserve_amd import kernels
+
+    g = torch.Generator().manual_seed(11)
+    n_src, n_dst, n = 300, 500, 257
+    src = torch.randn(n_src, H, D, generator=g).to(dtype)
+    dst0 = torch.randn(n_dst, H, D, generator=g).to(dtype)
+    si = torch.randint(0, n_src, (n,), generator=g).to(idx_dtype)
+    di = torch.randperm(n_dst, generator=g)[:n].to(idx_dtype)
+    want = dst0.clone()
+    ref_move_tokens(src, want, si, di)
+    d = dst0.to(dev)
+    kernels.discontinuous_move_tokens(src.to(dev), d, si.to(dev), di.to(dev))
+    assert torch.equal(_bits(d.cpu()), _bits(want))
+
+
+def test_move_tokens_strided_storages(dev):
+    """Free strides on all three axes (tokens_moving.py:88-93): a head-sliced, dim-strided view."""
+    from parrotserve_amd import kernels
+
+    g = torch.Generator().manual_seed(12)
+    big_src = torch.randn(64, 6, 32, generator=g).half()
+    big_dst = torch.randn(80, 4, 48, generator=g).half()
+    src_view = lambda t: t[:, 1:5, ::2]  # [64, 4, 16], strides (192, 32, 2)
+    dst_view = lambda t: t[:, :, 16:32]  # [80, 4, 16], strides (192, 48, 1)
+    si = torch.randperm(64, generator=g)[:40]
+    di = torch.randperm(80, generator=g)[:40]
+    want = big_dst.clone()
+    ref_move_tokens(src_view(big_src), dst_view(want), si, di)
+    s, d = big_src.to(dev), big_dst.to(dev)
+    kernels.discontinuous_move_tokens(src_view(s), dst_view(d), si.to(dev), di.to(dev))
+    assert torch.equal(_bits(d.cpu()), _bits(want))
+
+
+def test_move_tokens_reference_selftest_shape(dev):
+    """tokens_moving.py:316-362: H 96 x D 128 fp16, random src rows to every second dest row (scaled-down count)."""
+    from parrotserve_amd import kernels
+
+    g = torch.Generator().manual_seed(13)
+    n = 4096
+    src = torch.randn(n, 96, 128, generator=g).half()
+    si = torch.randperm(n, generator=g)
+    di = torch.arange(0, 2 * n, 2)
+    d = torch.zeros(2 * n, 96, 128, dtype=torch.float16, device=dev)
+    kernels.discontinuous_move_tokens(src.to(dev), d, si.to(dev), di.to(dev))
+    out = d.cpu()
+    assert torch.equal(_bits(out[::2]), _bits(src[si])) and (out[1::2] == 0).all()
+
+
+def test_move_empty_and_blocked_names(dev):
+    from parrotserve_amd import kernels
+
+    src = torch.randn(8, 2, 16).half().to(dev)
+    dst = torch.zeros(8, 2, 16).half().to(dev)
+    e = torch.empty(0, dtype=torch.int64, device=dev)
+    kernels.discontinuous_move_tokens(src, dst, e, e)
+    assert (dst == 0).all()
+    idx = torch.arange(8, device=dev)
+    kernels.move_tokens_from_blocked_k_cache(src, dst, idx.flip(0), idx)
+    assert torch.equal(dst.cpu(), src.cpu().flip(0))
+    kernels.move_tokens_from_blocked_v_cache(src, dst, idx, idx)
+    assert torch.equal(dst.cpu(), src.cpu())
+    with pytest.raises(ValueError):
+        kernels.move_tokens_from_blocked_k_cache(torch.zeros(2, 2, 2, 4, 8, device=dev).half(), dst, idx, idx)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("idx_dtype", [torch.int32, torch.int64])
+def test_kv_append_bit_exact_from_qkv_views(dev, dtype, idx_dtype):
+    from parrotserve_amd import kernels
+
+    g = torch.Generator().manual_seed(14)
+    T, H, D, slots = 77, 40, 128, 1000
+    qkv = torch.randn(T, 3 * H * D, generator=g).to(dtype)
+    kc0 = torch.randn(slots, H, D, generator=g).to(dtype)
+    vc0 = torch.randn(slots, H, D, generator=g).to(dtype)
+    sm = torch.randperm(slots, generator=g)[:T].to(idx_dtype)
+    _, k, v = qkv.chunk(3, dim=-1)
+    kc, vc = kc0.clone(), vc0.clone()
+    ref_kv_append(k.view(T, H, D), v.view(T, H, D), kc, vc, sm)
+    dq = qkv.to(dev)
+    _, dk, dv = dq.chunk(3, dim=-1)
+    dkc, dvc = kc0.to(dev), vc0.to(dev)
+    kernels.vllm_reshape_and_cache(dk.view(T, H, D), dv.view(T, H, D), dkc, dvc, sm.to(dev))
+    assert torch.equal(_bits(dkc.cpu()), _bits(kc)) and torch.equal(_bits(dvc.cpu()), _bits(vc))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("rows,n", [(128, 5120), (33, 4096), (5, 8192), (7, 1000), (3, 130)])
+def test_rms_norm(dev, dtype, rows, n):
+    from parrotserve_amd import kernels
+
+    g = torch.Generator().manual_seed(15)
+    x = (torch.randn(rows, n, generator=g) * 2 - 0.5).to(dtype)
+    w = (torch.rand(n, generator=g) + 0.5).to(dtype)
+    for fn, first in ((kernels.vllm_rms_norm, True), (kernels.rmsnorm_forward, False)):
+        y = fn(x.to(dev), w.to(dev), 1e-6).cpu()
+        ref = ref_rms_norm(x, w, 1e-6, round_before_weight=first)
+        torch.testing.assert_close(y.float(), ref.float(), **TOL[dtype])
+
+
+def test_rms_norm_reference_selftest_distribution(dev):
+    """kernels/rms_norm.py:85-99: x ~ -2.3 + 0.5 N(0,1), w ~ U[0,1), atol 1e-2 rtol 0."""
+    from parrotserve_amd import kernels
+
+    g = torch.Generator().manual_seed(16)
+    x = (-2.3 + 0.5 * torch.randn(1151, 8192, generator=g)).half()
+    w = torch.rand(8192, generator=g).half()
+    y = kernels.rmsnorm_forward(x.to(dev), w.to(dev), 1e-5).cpu()
+    ref = ref_rms_norm(x, w, 1e-5, round_before_weight=False)
+    assert torch.allclose(y.float(), ref.float(), atol=1e-2, rtol=0)
+    torch.testing.assert_close(y.float(), ref.float(), **TOL[torch.float16])
+
+
+def test_rms_norm_3d_input_keeps_shape(dev):
+    from parrotserve_amd import kernels
+
+    x = torch.randn(2, 5, 256).half()
+    w = torch.ones(256).half()
+    y = kernels.vllm_rms_norm(x.to(dev), w.to(dev), 1e-6)
+    assert y.shape == x.shape
+    torch.testing.assert_close(y.cpu().float(), ref_rms_norm(x, w, 1e-6).float(), **TOL[torch.float16])
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("T,H,D", [(129, 40, 128), (17, 32, 64), (5, 3, 80)])
+def test_rope_neox_on_qkv_views(dev, dtype, T, H, D):
+    from parrotserve_amd import kernels
+
+    g = torch.Generator().manual_seed(17)
+    qkv = torch.randn(T, 3 * H * D, generator=g).to(dtype)
+    pos = torch.randint(0, 4096, (T,), generator=g)
+    cache = ref_cos_sin_cache(4096, D, 10000.0, dtype)
+    q, k, v = qkv.chunk(3, dim=-1)
+    rq, rk = ref_rope_neox(pos, q, k, cache, D, elem_rounding=True)
+    rq32, rk32 = ref_rope_neox(pos, q, k, cache, D, elem_rounding=False)
+    d = qkv.to(dev)
+    dq, dk, dv = d.chunk(3, dim=-1)
+    kernels.vllm_rotary_emb(pos.to(dev), dq, dk, cache.to(dev), D)
+    out = d.cpu()
+    oq, ok, ov = out.chunk(3, dim=-1)
+    assert torch.equal(_bits(ov), _bits(v)), "v must be untouched"
+    # same arithmetic as the reference kernel (every product rounded to the element type): bit-exact
+    assert torch.equal(_bits(oq), _bits(rq)) and torch.equal(_bits(ok), _bits(rk))
+    torch.testing.assert_close(oq.float(), rq32.float(), **TOL[dtype])
+    torch.testing.assert_close(ok.float(), rk32.float(), **TOL[dtype])
+
+
+def test_rotary_embedding_reference_selftest(dev):
+    """kernels/rotary_embedding.py:155-174: T 256, H 96, D 128, cos ~ -1.2+0.5N, sin ~ -2.0+0.5N, atol 1e-2."""
+    from parrotserve_amd import kernels
+
+    g = torch.Generator().manual_seed(18)
+    T, H, D = 256, 96, 128
+    state = torch.randn(T, H, D, generator=g).half()
+    cos = (-1.2 + 0.5 * torch.randn(T, 1, D // 2, generator=g)).half()
+    sin = (-2.0 + 0.5 * torch.randn(T, 1, D // 2, generator=g)).half()
+    ref = ref_rotary_embedding(state, cos, sin)
+    d = state.to(dev)
+    kernels.rotary_embedding(d, cos.to(dev), sin.to(dev))
+    assert torch.allclose(d.cpu().float(), ref.float(), atol=1e-2, rtol=0)
+    assert torch.equal(_bits(d.cpu()), _bits(ref_rotary_embedding(state, cos, sin, elem_rounding=True)))
+
+
+def test_rope_round_trip_property(dev):
+    """rotate by +angle then -angle restores the input (within two roundings)."""
+    from parrotserve_amd import kernels
+
+    g = torch.Generator().manual_seed(19)
+    T, H, D = 64, 8, 128
+    x = torch.randn(T, H, D, generator=g).half()
+    cache = ref_cos_sin_cache(512, D, 10000.0, torch.float16)
+    pos = torch.randint(0, 512, (T,), generator=g)
+    cs = cache[pos]
+    cos, sin = cs[:, None, : D // 2].contiguous(), cs[:, None, D // 2 :].contiguous()
+    d = x.to(dev)
+    kernels.rotary_embedding(d, cos.to(dev), sin.to(dev))
+    kernels.rotary_embedding(d, cos.to(dev), (-sin).to(dev))
+    torch.testing.assert_close(d.cpu().float(), x.float(), atol=8e-3, rtol=1e-2)
