@@ -218,6 +218,16 @@ int ph_prefill_attention(void* out, const void* q, const void* k_cache, const vo
                          const int32_t* ctx_slots, int64_t max_kv_len,
                          void* workspace, size_t workspace_bytes, void* stream);
 
+/* ------------------------------------------------------------------------ */
+/* Instrumentation (no counterpart in the reference, which times whole
+ * iterations from Python, parrot/engine/builtin/builtin_runner.py:158-175).
+ * Arms the NEXT ph_decode_attention call on this thread's library state: it
+ * records events[0] before the prefix kernel, events[1] before the suffix
+ * kernel, events[2] before the merge kernel and events[3] after it, on the
+ * call's stream (hipEvent_t handles owned by the caller).  One call consumes
+ * the arming.  Pass NULL to disarm. */
+int ph_arm_phase_events(void* const* events4);
+
 #ifdef __cplusplus
 }
 #endif

@@ -150,6 +150,20 @@ extern "C" const char* ph_status_string(int status) {
 
 extern "C" int ph_abi_version(void) { return 1; }
 
+static hipEvent_t g_phase_events[4];
+static bool g_phase_armed = false;
+
+extern "C" int ph_arm_phase_events(void* const* events4) {
+  g_phase_armed = events4 != nullptr;
+  if (events4)
+    for (int i = 0; i < 4; ++i) g_phase_events[i] = (hipEvent_t)events4[i];
+  return PH_OK;
+}
+
+static inline void phase_mark(bool armed, int i, hipStream_t st) {
+  if (armed) (void)hipEventRecord(g_phase_events[i], st);
+}
+
 extern "C" size_t ph_decode_workspace_bytes(int64_t num_reqs, int64_t num_heads, int64_t head_dim,
                                             int64_t num_groups, int64_t max_prefix_len, int64_t max_suffix_len,
                                             int64_t chunk_tokens) {
@@ -183,7 +197,10 @@ extern "C" int ph_decode_attention(void* out, const void* q, const void* k_cache
   const Carve ws = carve(workspace, p, B, H, D);
   hipStream_t st = (hipStream_t)stream;
   const float sl2 = scale * kLog2e;
+  const bool armed = g_phase_armed;
+  g_phase_armed = false;
 
+  phase_mark(armed, 0, st);
   if (has_prefix) {
     int covered = 0, max_group_reqs = 0;
     for (int g = 0; g < num_groups; ++g) {
@@ -216,6 +233,7 @@ extern "C" int ph_decode_attention(void* out, const void* q, const void* k_cache
     rc = run_prefix(pa, dtype, D, (int)num_groups, group_req_cu_host, max_group_reqs, st);
     if (rc != PH_OK) return rc;
   }
+  phase_mark(armed, 1, st);
   if (has_suffix) {
     PartialArgs sa{};
     sa.q = (const uint16_t*)q;
@@ -253,7 +271,10 @@ extern "C" int ph_decode_attention(void* out, const void* q, const void* k_cache
   ma.baseB = p.n_splits;
   ma.lens = has_suffix ? suffix_lens : nullptr;
   ma.chunk = p.chunk;
-  return launch_merge(ma, dtype, D, st);
+  phase_mark(armed, 2, st);
+  rc = launch_merge(ma, dtype, D, st);
+  phase_mark(armed, 3, st);
+  return rc;
 }
 
 extern "C" int ph_prefix_attention(void* out, float* m_out, float* l_out, const void* q, const void* k_cache,
