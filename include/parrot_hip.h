@@ -145,6 +145,9 @@ int ph_rotary_embedding(void* state, const void* cos, const void* sin,
  *   suffix_offsets == NULL: suffix_slots is a padded 2-D table, request b's
  *                 list starts at b * suffix_table_stride (the reference's
  *                 paged_block_tables [B, max]).
+ *   suffix_slots_count: number of int32 entries readable behind suffix_slots
+ *                 (the kernel prefetches slot ids before it knows a list's
+ *                 length and clamps those reads to this bound);
  *   suffix_lens:  int32 [B] (DEVICE); max_suffix_len: host upper bound.
  * chunk_tokens: suffix split size (multiple of 16), 0 = choose.
  * workspace: at least ph_decode_workspace_bytes(...) bytes, 256-byte aligned.
@@ -161,7 +164,8 @@ int ph_decode_attention(void* out, const void* q, const void* k_cache, const voi
                         const int32_t* group_req_cu, const int32_t* group_req_cu_host,
                         int64_t max_prefix_len,
                         const int32_t* suffix_slots, const int64_t* suffix_offsets,
-                        int64_t suffix_table_stride, const int32_t* suffix_lens,
+                        int64_t suffix_table_stride, int64_t suffix_slots_count,
+                        const int32_t* suffix_lens,
                         int64_t max_suffix_len, int64_t chunk_tokens,
                         void* workspace, size_t workspace_bytes, void* stream);
 
@@ -188,7 +192,8 @@ int ph_suffix_post_attention(void* out, const float* prev_m, const float* prev_l
                              int64_t num_reqs, int64_t num_heads, int64_t head_dim, int dtype,
                              int64_t q_stride, int64_t out_stride, int64_t cache_stride_n, float scale,
                              const int32_t* suffix_slots, const int64_t* suffix_offsets,
-                             int64_t suffix_table_stride, const int32_t* suffix_lens,
+                             int64_t suffix_table_stride, int64_t suffix_slots_count,
+                             const int32_t* suffix_lens,
                              int64_t max_suffix_len, int64_t chunk_tokens,
                              void* workspace, size_t workspace_bytes, void* stream);
 
@@ -203,7 +208,7 @@ int ph_suffix_post_attention(void* out, const float* prev_m, const float* prev_l
  * q, out: [T, H, D] packed chunk after chunk, row strides q_stride/out_stride.
  * q_cu:  int32 [num_chunks+1] query offsets (DEVICE);
  * kv_cu: int32 [num_chunks+1] offsets into ctx_slots (DEVICE);
- * ctx_slots: int32, every chunk's whole context (ancestors || own), in order.
+ * ctx_slots: int32 [ctx_slots_count], every chunk's whole context (ancestors || own), in order.
  * Query r of chunk c sees key j iff j <= r + (kv_len_c - q_len_c).
  * The new tokens' K/V must already be in the cache (append first).
  * max_kv_len: host upper bound of any chunk's context length.
@@ -215,7 +220,7 @@ int ph_prefill_attention(void* out, const void* q, const void* k_cache, const vo
                          int64_t num_tokens, int64_t num_chunks, int64_t num_heads, int64_t head_dim,
                          int dtype, int64_t q_stride, int64_t out_stride, int64_t cache_stride_n,
                          float scale, const int32_t* q_cu, const int32_t* kv_cu,
-                         const int32_t* ctx_slots, int64_t max_kv_len,
+                         const int32_t* ctx_slots, int64_t ctx_slots_count, int64_t max_kv_len,
                          void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------ */

@@ -38,13 +38,22 @@ static DecodePlan plan_decode(int64_t B, int64_t H, int64_t groups, int64_t max_
     p.n_chunks = 0;
   }
   if (groups > 0 && max_prefix > 0) {
-    // About 512 workgroups over (group, head, query tile, split).
+    // One workgroup per CU at a time (the kernel uses most of the register file), so pick the
+    // split count whose workgroup total wastes the least of a whole number of 256-wide rounds.
+    // Cost model: rounds x (tokens per split + a fixed prologue/epilogue worth ~96 tokens).
     const int64_t mtiles = cdiv(cdiv(B, groups), kPrefixQueryTile);
-    int64_t splits = cdiv(512, groups * H * (mtiles > 0 ? mtiles : 1));
-    const int64_t max_splits = cdiv(max_prefix, 2 * kPrefixTile);
-    if (splits > max_splits) splits = max_splits;
-    if (splits < 1) splits = 1;
-    const int64_t st = round_up(cdiv(max_prefix, splits), kPrefixTile);
+    const int64_t base = groups * H * (mtiles > 0 ? mtiles : 1);
+    const int64_t max_splits = cdiv(max_prefix, 4 * kPrefixTile);
+    int64_t splits = 1, best = -1;
+    for (int64_t s = 1; s <= 64 && s <= (max_splits > 0 ? max_splits : 1); ++s) {
+      const int64_t tok = round_up(cdiv(max_prefix, s), 2 * kPrefixTile);
+      const int64_t cost = cdiv(base * s, 256) * (tok + 96);
+      if (best < 0 || cost < best) {
+        best = cost;
+        splits = s;
+      }
+    }
+    const int64_t st = round_up(cdiv(max_prefix, splits), 2 * kPrefixTile);
     p.split_tokens = (int)st;
     p.n_splits = (int)cdiv(max_prefix, st);
   }
@@ -179,7 +188,7 @@ extern "C" int ph_decode_attention(void* out, const void* q, const void* k_cache
                                    const int32_t* group_req_cu, const int32_t* group_req_cu_host,
                                    int64_t max_prefix_len, const int32_t* suffix_slots,
                                    const int64_t* suffix_offsets, int64_t suffix_table_stride,
-                                   const int32_t* suffix_lens, int64_t max_suffix_len, int64_t chunk_tokens,
+                                   int64_t suffix_slots_count, const int32_t* suffix_lens, int64_t max_suffix_len, int64_t chunk_tokens,
                                    void* workspace, size_t workspace_bytes, void* stream) {
   const int B = (int)num_reqs, H = (int)num_heads, D = (int)head_dim;
   int rc = check_common(out, q, k_cache, v_cache, num_reqs, num_heads, head_dim, dtype, q_stride, out_stride,
@@ -189,7 +198,7 @@ extern "C" int ph_decode_attention(void* out, const void* q, const void* k_cache
   const bool has_prefix = num_groups > 0 && max_prefix_len > 0;
   const bool has_suffix = max_suffix_len > 0;
   if (has_prefix && (!prefix_slots || !prefix_cu || !group_req_cu || !group_req_cu_host)) return PH_ERR_ARG;
-  if (has_suffix && (!suffix_slots || !suffix_lens)) return PH_ERR_ARG;
+  if (has_suffix && (!suffix_slots || !suffix_lens || suffix_slots_count <= 0)) return PH_ERR_ARG;
   const DecodePlan p =
       plan_decode(num_reqs, num_heads, has_prefix ? num_groups : 0, max_prefix_len, max_suffix_len, chunk_tokens);
   if (plan_bytes(p, B, H, D) > workspace_bytes || (p.parts() > 0 && !workspace)) return PH_ERR_WORKSPACE;
@@ -242,6 +251,7 @@ extern "C" int ph_decode_attention(void* out, const void* q, const void* k_cache
     sa.vc = (const uint16_t*)v_cache;
     sa.row_stride = cache_stride_n;
     sa.slots = suffix_slots;
+    sa.slots_total = suffix_slots_count;
     sa.offsets = suffix_offsets;
     sa.table_stride = suffix_table_stride;
     sa.lens = suffix_lens;
@@ -334,7 +344,8 @@ extern "C" int ph_suffix_post_attention(void* out, const float* prev_m, const fl
                                         int64_t num_heads, int64_t head_dim, int dtype, int64_t q_stride,
                                         int64_t out_stride, int64_t cache_stride_n, float scale,
                                         const int32_t* suffix_slots, const int64_t* suffix_offsets,
-                                        int64_t suffix_table_stride, const int32_t* suffix_lens,
+                                        int64_t suffix_table_stride, int64_t suffix_slots_count,
+                                        const int32_t* suffix_lens,
                                         int64_t max_suffix_len, int64_t chunk_tokens, void* workspace,
                                         size_t workspace_bytes, void* stream) {
   const int B = (int)num_reqs, H = (int)num_heads, D = (int)head_dim;
@@ -343,7 +354,7 @@ extern "C" int ph_suffix_post_attention(void* out, const float* prev_m, const fl
   if (rc != PH_OK || num_reqs == 0) return rc;
   if (max_suffix_len < 0 || !prev_m || !prev_l) return PH_ERR_ARG;
   const bool has_suffix = max_suffix_len > 0;
-  if (has_suffix && (!suffix_slots || !suffix_lens)) return PH_ERR_ARG;
+  if (has_suffix && (!suffix_slots || !suffix_lens || suffix_slots_count <= 0)) return PH_ERR_ARG;
   const DecodePlan p = plan_decode(num_reqs, num_heads, 0, 0, max_suffix_len, chunk_tokens);
   if (plan_bytes(p, B, H, D) > workspace_bytes || (p.parts() > 0 && !workspace)) return PH_ERR_WORKSPACE;
   if (((uintptr_t)workspace & 255u) != 0) return PH_ERR_ALIGN;
@@ -357,6 +368,7 @@ extern "C" int ph_suffix_post_attention(void* out, const float* prev_m, const fl
     sa.vc = (const uint16_t*)v_cache;
     sa.row_stride = cache_stride_n;
     sa.slots = suffix_slots;
+    sa.slots_total = suffix_slots_count;
     sa.offsets = suffix_offsets;
     sa.table_stride = suffix_table_stride;
     sa.lens = suffix_lens;
@@ -403,13 +415,14 @@ extern "C" int ph_prefill_attention(void* out, const void* q, const void* k_cach
                                     int64_t num_tokens, int64_t num_chunks, int64_t num_heads, int64_t head_dim,
                                     int dtype, int64_t q_stride, int64_t out_stride, int64_t cache_stride_n,
                                     float scale, const int32_t* q_cu, const int32_t* kv_cu,
-                                    const int32_t* ctx_slots, int64_t max_kv_len, void* workspace,
+                                    const int32_t* ctx_slots, int64_t ctx_slots_count, int64_t max_kv_len,
+                                    void* workspace,
                                     size_t workspace_bytes, void* stream) {
   const int T = (int)num_tokens, H = (int)num_heads, D = (int)head_dim;
   int rc = check_common(out, q, k_cache, v_cache, num_tokens, num_heads, head_dim, dtype, q_stride, out_stride,
                         cache_stride_n);
   if (rc != PH_OK || num_tokens == 0) return rc;
-  if (num_chunks <= 0 || max_kv_len <= 0 || !q_cu || !kv_cu || !ctx_slots) return PH_ERR_ARG;
+  if (num_chunks <= 0 || max_kv_len <= 0 || !q_cu || !kv_cu || !ctx_slots || ctx_slots_count <= 0) return PH_ERR_ARG;
   if (ph_prefill_workspace_bytes(num_tokens, num_heads, head_dim, max_kv_len) > workspace_bytes || !workspace)
     return PH_ERR_WORKSPACE;
   if (((uintptr_t)workspace & 255u) != 0) return PH_ERR_ALIGN;
@@ -429,6 +442,7 @@ extern "C" int ph_prefill_attention(void* out, const void* q, const void* k_cach
   sa.vc = (const uint16_t*)v_cache;
   sa.row_stride = cache_stride_n;
   sa.slots = ctx_slots;
+  sa.slots_total = ctx_slots_count;
   sa.offsets = offsets;
   sa.lens = lens;
   sa.shared_len = -1;

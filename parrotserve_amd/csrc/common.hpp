@@ -80,12 +80,25 @@ __device__ __forceinline__ void st16_nt(void* p, u32x4 v) {
   __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
 }
 
-// Butterfly sum over aligned groups of W lanes (W a power of two <= 64); every
-// lane of the group ends with the group's sum.
+// v + (v of the lane selected by a DPP control): one v_add_f32_dpp, no LDS round trip.
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+  const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true);
+  return v + __builtin_bit_cast(float, moved);
+}
+
+// Sum over aligned groups of W lanes (W a power of two <= 64); every lane of
+// the group ends with the group's sum.  Up to 16 lanes the exchange stays inside
+// a DPP row: quad_perm [1,0,3,2], quad_perm [2,3,0,1], row_half_mirror,
+// row_mirror (pairing lanes, not an xor butterfly, which is all a sum needs).
 template <int W>
 __device__ __forceinline__ float group_sum(float v) {
-#pragma unroll
-  for (int s = W / 2; s >= 1; s >>= 1) v += __shfl_xor(v, s, kWave);
+  if (W >= 2) v = dpp_add<0xB1>(v);
+  if (W >= 4) v = dpp_add<0x4E>(v);
+  if (W >= 8) v = dpp_add<0x141>(v);
+  if (W >= 16) v = dpp_add<0x140>(v);
+  if (W >= 32) v += __shfl_xor(v, 16, kWave);
+  if (W >= 64) v += __shfl_xor(v, 32, kWave);
   return v;
 }
 template <int W>

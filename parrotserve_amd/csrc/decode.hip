@@ -15,9 +15,11 @@
 // parrot/engine/builtin/kernels/shared_flash_decoding.py:137-199 (n-way reduce).
 #include "decode.hpp"
 
+#include <cstdlib>
+
 namespace ph {
 
-template <typename E, int D, int TB>
+template <typename E, int D, int TB, int STAGES, int DBG = 0>
 __global__ __launch_bounds__(256) void decode_partial_kernel(PartialArgs a) {
   constexpr int LPH = D / 8;       // lanes per head
   constexpr int HPW = kWave / LPH;  // heads per wave
@@ -31,47 +33,74 @@ __global__ __launch_bounds__(256) void decode_partial_kernel(PartialArgs a) {
   if (rb >= a.num_reqs) return;
   const int b = a.req_begin + rb;
 
-  int64_t off;
+  // The first block's slot ids are fetched before the length is known (clamped to the table's
+  // end), so the chain of dependent loads in front of the K/V stream is two deep, not three.
+  const int t0 = c * a.chunk;
+  int64_t off, last;  // last = highest readable index behind this list's start
   int len;
   if (a.shared_cu) {
     off = a.shared_cu[0];
     len = a.shared_cu[1] - a.shared_cu[0];
+    last = len - 1;
   } else if (a.shared_len >= 0) {
     off = 0;
     len = a.shared_len;
+    last = len - 1;
   } else {
     off = a.offsets ? a.offsets[b] : (int64_t)b * a.table_stride;
-    len = a.lens[b];
+    len = -1;
+    last = a.slots_total - 1 - off;
   }
-  const int t0 = c * a.chunk;
-  if (t0 >= len) return;
-  const int t1 = min(len, t0 + a.chunk);
+  if (last < 0) return;  // an empty shared list, or an offset at the very end of the table
+  const int32_t* slots = a.slots + off;
+  int myslot = slots[min((int64_t)(t0 + lane), last)];
+  if (len < 0) len = a.lens[b];
 
   const int head = hg * HPW + lane / LPH;
   const bool head_ok = head < a.H;
   const int hclamp = head_ok ? head : a.H - 1;
-  const int64_t lane_off = (int64_t)hclamp * D + (lane % LPH) * 8;
-
+  const uint32_t lane_off = (uint32_t)(hclamp * D + (lane % LPH) * 8);  // elements inside a token row
   const u32x4 qv = ld16(a.q + (int64_t)b * a.q_stride + lane_off);
-  const int32_t* slots = a.slots + off;
+
+  if (t0 >= len) return;
+  const int t1 = min(len, t0 + a.chunk);
 
   float m = -INFINITY, l = 0.f;
   float o[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) o[i] = 0.f;
 
+  u32x4 kb[STAGES][TB], vb[STAGES][TB];
+
   for (int tb = t0; tb < t1; tb += kWave) {
-    const int mine = min(tb + lane, t1 - 1);
-    const int myslot = slots[mine];
+    if (tb > t0) myslot = slots[min(tb + lane, t1 - 1)];
     const int nb = min(kWave, t1 - tb);
-    for (int j0 = 0; j0 < nb; j0 += TB) {
-      u32x4 kk[TB], vv[TB];
+
+    // TB token rows (K and V) in flight per stage; row bases are wave-uniform (SGPR)
+    auto load = [&](u32x4(&kk)[TB], u32x4(&vv)[TB], int j0) {
 #pragma unroll
       for (int j = 0; j < TB; ++j) {
-        const int64_t slot = __builtin_amdgcn_readlane(myslot, j0 + j);
-        const int64_t ro = slot * a.row_stride + lane_off;
-        kk[j] = ld16(a.kc + ro);
-        vv[j] = ld16(a.vc + ro);
+        const int64_t slot = __builtin_amdgcn_readlane(myslot, min(j0 + j, nb - 1));
+        const uint16_t* kr = a.kc + slot * a.row_stride;
+        const uint16_t* vr = a.vc + slot * a.row_stride;
+        if (DBG == 1) {
+          kk[j] = qv;
+          vv[j] = qv;
+        } else {
+          kk[j] = ld16(kr + lane_off);
+          vv[j] = ld16(vr + lane_off);
+        }
+      }
+    };
+    auto compute = [&](const u32x4(&kk)[TB], const u32x4(&vv)[TB], int j0) {
+      if (DBG == 2) {
+#pragma unroll
+        for (int j = 0; j < TB; ++j) {
+          o[0] += __builtin_bit_cast(float, kk[j][0] ^ kk[j][1] ^ kk[j][2] ^ kk[j][3]);
+          o[1] += __builtin_bit_cast(float, vv[j][0] ^ vv[j][1] ^ vv[j][2] ^ vv[j][3]);
+        }
+        l = 1.f;
+        return;
       }
       float s[TB];
       float mb = -INFINITY;
@@ -95,11 +124,28 @@ __global__ __launch_bounds__(256) void decode_partial_kernel(PartialArgs a) {
         l += p;
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
-          o[2 * w] += p * Elem<E>::lo(vv[j][w]);
-          o[2 * w + 1] += p * Elem<E>::hi(vv[j][w]);
+          o[2 * w] = __builtin_fmaf(p, Elem<E>::lo(vv[j][w]), o[2 * w]);
+          o[2 * w + 1] = __builtin_fmaf(p, Elem<E>::hi(vv[j][w]), o[2 * w + 1]);
         }
       }
       m = mn;
+    };
+
+    // two-stage software pipeline: the next batch's rows are in flight while this one is reduced
+    if (STAGES == 2) {
+      load(kb[0], vb[0], 0);
+      for (int j0 = 0; j0 < nb; j0 += 2 * TB) {
+        const bool more1 = j0 + TB < nb;
+        if (more1) load(kb[STAGES - 1], vb[STAGES - 1], j0 + TB);
+        compute(kb[0], vb[0], j0);
+        if (j0 + 2 * TB < nb) load(kb[0], vb[0], j0 + 2 * TB);
+        if (more1) compute(kb[STAGES - 1], vb[STAGES - 1], j0 + TB);
+      }
+    } else {
+      for (int j0 = 0; j0 < nb; j0 += TB) {
+        load(kb[0], vb[0], j0);
+        compute(kb[0], vb[0], j0);
+      }
     }
   }
 
@@ -117,19 +163,22 @@ __global__ __launch_bounds__(256) void decode_partial_kernel(PartialArgs a) {
   }
 }
 
-// One wave per (request, HPW heads): fold every valid partial.
+// One workgroup per (request, HPW heads); its four waves fold every fourth part each
+// (loads are unconditional and independent, so several parts are in flight per wave),
+// then wave 0 folds the four running results through LDS and writes the output row.
 template <typename E, int D>
 __global__ __launch_bounds__(256) void merge_kernel(MergeArgs a) {
   constexpr int LPH = D / 8;
   constexpr int HPW = kWave / LPH;
+  __shared__ float sh[3][10][kWave];
   const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(blockIdx.x * 4 + (threadIdx.x >> 6));
+  const int w = threadIdx.x >> 6;
   const int hgroups = (a.H + HPW - 1) / HPW;
-  const int b = wave / hgroups;
-  const int hg = wave - b * hgroups;
-  if (b >= a.B) return;
-  const int head = hg * HPW + lane / LPH;
-  if (head >= a.H) return;
+  const int b = blockIdx.x / hgroups;
+  const int hg = blockIdx.x - b * hgroups;
+  const int head_raw = hg * HPW + lane / LPH;
+  const bool head_ok = head_raw < a.H;
+  const int head = head_ok ? head_raw : a.H - 1;
   const int dl = (lane % LPH) * 8;
 
   float M = -INFINITY, L = 0.f;
@@ -137,47 +186,68 @@ __global__ __launch_bounds__(256) void merge_kernel(MergeArgs a) {
 #pragma unroll
   for (int i = 0; i < 8; ++i) acc[i] = 0.f;
 
-  if (a.prev_m) {  // a partial already sitting in out / prev_m / prev_l
+  if (a.prev_m && w == 0) {  // a partial already sitting in out / prev_m / prev_l
     const float lp = a.prev_l[(int64_t)b * a.H + head];
     if (lp > 0.f) {
       const u32x4 ov = ld16(a.out + (int64_t)b * a.out_stride + (int64_t)head * D + dl);
       M = a.prev_m[(int64_t)b * a.H + head];
       L = lp;
 #pragma unroll
-      for (int w = 0; w < 4; ++w) {
-        acc[2 * w] = lp * Elem<E>::lo(ov[w]);
-        acc[2 * w + 1] = lp * Elem<E>::hi(ov[w]);
+      for (int k = 0; k < 4; ++k) {
+        acc[2 * k] = lp * Elem<E>::lo(ov[k]);
+        acc[2 * k + 1] = lp * Elem<E>::hi(ov[k]);
       }
     }
   }
 
   const int nB = a.lens ? (a.lens[b] + a.chunk - 1) / a.chunk : 0;
   const int total = a.nA + nB;
-  for (int i = 0; i < total; ++i) {
+#pragma unroll 2
+  for (int i = w; i < total; i += 4) {
     const int part = i < a.nA ? i : a.baseB + (i - a.nA);
     const int64_t pr = ((int64_t)part * a.B + b) * a.H + head;
-    const float lp = a.ml[pr * 2 + 1];
-    if (lp > 0.f) {
-      const float mp = a.ml[pr * 2];
-      const float* op = a.opart + pr * D + dl;
-      const float4_t o0 = *reinterpret_cast<const float4_t*>(op);
-      const float4_t o1 = *reinterpret_cast<const float4_t*>(op + 4);
-      const float Mn = fmaxf(M, mp);
-      const float sc = __builtin_amdgcn_exp2f(M - Mn);
-      const float w = __builtin_amdgcn_exp2f(mp - Mn) * lp;
-      L = L * sc + w;
+    const float2 mlp = *reinterpret_cast<const float2*>(a.ml + pr * 2);
+    const float* op = a.opart + pr * D + dl;
+    const float4_t o0 = *reinterpret_cast<const float4_t*>(op);
+    const float4_t o1 = *reinterpret_cast<const float4_t*>(op + 4);
+    const bool live = mlp.y > 0.f;  // l == 0 marks an empty part (its O may be garbage)
+    const float mp = live ? mlp.x : -INFINITY;
+    const float Mn = fmaxf(M, mp);
+    const float sc = (M == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(M - Mn);
+    const float wgt = live ? __builtin_amdgcn_exp2f(mp - Mn) * mlp.y : 0.f;
+    L = L * sc + wgt;
 #pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        acc[k] = acc[k] * sc + w * o0[k];
-        acc[4 + k] = acc[4 + k] * sc + w * o1[k];
-      }
-      M = Mn;
+    for (int k = 0; k < 4; ++k) {
+      acc[k] = acc[k] * sc + (live ? wgt * o0[k] : 0.f);
+      acc[4 + k] = acc[4 + k] * sc + (live ? wgt * o1[k] : 0.f);
     }
+    M = Mn;
   }
+
+  if (w > 0) {
+    sh[w - 1][0][lane] = M;
+    sh[w - 1][1][lane] = L;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) sh[w - 1][2 + k][lane] = acc[k];
+  }
+  __syncthreads();
+  if (w != 0) return;
+#pragma unroll
+  for (int o = 0; o < 3; ++o) {
+    const float mo = sh[o][0][lane], lo = sh[o][1][lane];
+    const float Mn = fmaxf(M, mo);
+    const float sa = (M == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(M - Mn);
+    const float sb = (mo == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mo - Mn);
+    L = L * sa + lo * sb;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) acc[k] = acc[k] * sa + sh[o][2 + k][lane] * sb;
+    M = Mn;
+  }
+  if (!head_ok) return;
   const float inv = L > 0.f ? 1.f / L : 0.f;
   u32x4 r;
 #pragma unroll
-  for (int w = 0; w < 4; ++w) r[w] = pack2<E>(acc[2 * w] * inv, acc[2 * w + 1] * inv);
+  for (int k = 0; k < 4; ++k) r[k] = pack2<E>(acc[2 * k] * inv, acc[2 * k + 1] * inv);
   st16(a.out + (int64_t)b * a.out_stride + (int64_t)head * D + dl, r);
   if (a.m_out && dl == 0) {
     a.m_out[(int64_t)b * a.H + head] = M;
@@ -198,7 +268,16 @@ static int launch_partial_t(const PartialArgs& a, hipStream_t st) {
   const int64_t waves = (int64_t)a.num_reqs * a.n_chunks * hgroups;
   if (waves == 0) return PH_OK;
   dim3 grid((unsigned)((waves + 3) / 4)), block(256);
-  hipLaunchKernelGGL((decode_partial_kernel<E, D, 8>), grid, block, 0, st, a);
+  static const int variant = getenv("PH_DECODE_VARIANT") ? atoi(getenv("PH_DECODE_VARIANT")) : 0;
+  switch (variant) {
+    case 1: hipLaunchKernelGGL((decode_partial_kernel<E, D, 4, 1>), grid, block, 0, st, a); break;
+    case 5: hipLaunchKernelGGL((decode_partial_kernel<E, D, 4, 1, 1>), grid, block, 0, st, a); break;
+    case 6: hipLaunchKernelGGL((decode_partial_kernel<E, D, 4, 1, 2>), grid, block, 0, st, a); break;
+    case 2: hipLaunchKernelGGL((decode_partial_kernel<E, D, 2, 2>), grid, block, 0, st, a); break;
+    case 3: hipLaunchKernelGGL((decode_partial_kernel<E, D, 8, 1>), grid, block, 0, st, a); break;
+    case 4: hipLaunchKernelGGL((decode_partial_kernel<E, D, 2, 1>), grid, block, 0, st, a); break;
+    default: hipLaunchKernelGGL((decode_partial_kernel<E, D, 4, 2>), grid, block, 0, st, a); break;
+  }
   return launch_status();
 }
 
@@ -206,9 +285,9 @@ template <typename E, int D>
 static int launch_merge_t(const MergeArgs& a, hipStream_t st) {
   constexpr int HPW = kWave / (D / 8);
   const int64_t hgroups = (a.H + HPW - 1) / HPW;
-  const int64_t waves = (int64_t)a.B * hgroups;
-  if (waves == 0) return PH_OK;
-  dim3 grid((unsigned)((waves + 3) / 4)), block(256);
+  const int64_t groups = (int64_t)a.B * hgroups;
+  if (groups == 0) return PH_OK;
+  dim3 grid((unsigned)groups), block(256);
   hipLaunchKernelGGL((merge_kernel<E, D>), grid, block, 0, st, a);
   return launch_status();
 }

@@ -15,6 +15,7 @@ struct PartialArgs {
   const uint16_t* vc;
   int64_t row_stride;       // elements between consecutive slots
   const int32_t* slots;     // slot table base
+  int64_t slots_total;      // entries readable behind `slots` (speculative reads are clamped to it)
   const int64_t* offsets;   // per-request start inside `slots`, or null
   int64_t table_stride;     // start = b * table_stride when offsets is null
   const int32_t* lens;      // per-request list length

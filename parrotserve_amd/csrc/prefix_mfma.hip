@@ -17,7 +17,12 @@
 //   C (32 x 32): lane holds column r, rows 8*j + 4*h + i at register 4*j + i
 // The contraction index is a free permutation as long as A and B agree, which
 // lets the fp32 S^T registers feed the second product as its B operand with no
-// cross-lane movement: V^T is stored in LDS with tokens permuted to match.
+// cross-lane movement.  V stays row-major [token][dim] in LDS; its transposed A
+// operand comes from ds_read_b64_tr_b16, which hands lane j of each 16-lane
+// group column j of a 4-row x 16-column block whose row addresses the lanes
+// supply (source lane s -> row s/4, columns 4*(s%4)..+3).  Both tiles are
+// XOR-swizzled in 16-byte chunks so that the 128-bit K reads and the
+// transposing V reads are free of bank conflicts.
 //
 // Math restated from parrot/engine/builtin/kernels/shared_flash_decoding.py:34-134.
 #include "decode.hpp"
@@ -48,11 +53,11 @@ constexpr int kVtOff = 8192;
 
 __device__ __forceinline__ u32x4 lds_ld16(const char* p) { return *reinterpret_cast<const u32x4*>(p); }
 
-// position of token t (0..31) inside a V^T row so that the 8 tokens a lane
-// needs for contraction step u sit in one 16-byte chunk
-__device__ __forceinline__ int vt_pos(int t) {
-  const int i = t & 3, hh = (t >> 2) & 1, j = t >> 3;
-  return (j >> 1) * 16 + hh * 8 + (j & 1) * 4 + i;
+typedef short short4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ u32x2 lds_tr16(const char* p) {
+  const short4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      (short4_t __attribute__((address_space(3)))*)(const_cast<char*>(p)));
+  return __builtin_bit_cast(u32x2, v);
 }
 
 template <typename E, int NQB>
@@ -118,42 +123,39 @@ __global__ __launch_bounds__(256, 1) void prefix_mfma_kernel(PrefixArgs a, int m
   const int tl = lane >> 4, c = lane & 15;
   const int64_t col = (int64_t)head * kPD + c * 8;
   u32x4 kreg[8], vreg[8];
-  int tb = s0 + kTile * w;
-  if (tb < s1) {
+  int snext[8];  // slot ids one tile ahead of the K/V rows in flight, so no load waits on a fresh slot fetch
+  auto fetch_slots = [&](int t0) {
+#pragma unroll
+    for (int r = 0; r < 8; ++r) snext[r] = slots[min(t0 + 4 * r + tl, s1 - 1)];
+  };
+  auto fetch_rows = [&]() {
 #pragma unroll
     for (int r = 0; r < 8; ++r) {
-      const int tok = min(tb + 4 * r + tl, s1 - 1);
-      const int64_t ro = (int64_t)slots[tok] * a.row_stride + col;
+      const int64_t ro = (int64_t)snext[r] * a.row_stride + col;
       kreg[r] = ld16(a.kc + ro);
       vreg[r] = ld16(a.vc + ro);
     }
+  };
+  int tb = s0 + kTile * w;
+  if (tb < s1) {
+    fetch_slots(tb);
+    fetch_rows();
+    if (tb + 4 * kTile < s1) fetch_slots(tb + 4 * kTile);
   }
 
   for (; tb < s1; tb += 4 * kTile) {
-    // registers -> LDS: K row-major with XOR-swizzled 16-byte chunks, V transposed
+    // registers -> LDS, both tiles row-major [token][dim] with XOR-swizzled 16-byte chunks
 #pragma unroll
     for (int r = 0; r < 8; ++r) {
       const int t = 4 * r + tl;
       *reinterpret_cast<u32x4*>(wl + t * 256 + ((c ^ (t & 15)) * 16)) = kreg[r];
-      const int pos = vt_pos(t);
-#pragma unroll
-      for (int k = 0; k < 8; ++k) {
-        const int d = 8 * c + k;
-        const uint16_t val = (uint16_t)(vreg[r][k >> 1] >> ((k & 1) * 16));
-        *reinterpret_cast<uint16_t*>(wl + kVtOff + d * 64 + (((pos >> 3) ^ ((d >> 2) & 3)) * 16) + (pos & 7) * 2) =
-            val;
-      }
+      *reinterpret_cast<u32x4*>(wl + kVtOff + t * 256 + ((c ^ (4 * (t & 3))) * 16)) = vreg[r];
     }
-    // prefetch the wave's next tile while this one is consumed
-    const int nt = tb + 4 * kTile;
-    if (nt < s1) {
-#pragma unroll
-      for (int r = 0; r < 8; ++r) {
-        const int tok = min(nt + 4 * r + tl, s1 - 1);
-        const int64_t ro = (int64_t)slots[tok] * a.row_stride + col;
-        kreg[r] = ld16(a.kc + ro);
-        vreg[r] = ld16(a.vc + ro);
-      }
+    // next tile's rows go in flight now (their slot ids arrived during the previous tile);
+    // then the slot ids of the tile after that
+    if (tb + 4 * kTile < s1) {
+      fetch_rows();
+      if (tb + 8 * kTile < s1) fetch_slots(tb + 8 * kTile);
     }
 
     // S^T = K Q^T
@@ -202,15 +204,25 @@ __global__ __launch_bounds__(256, 1) void prefix_mfma_kernel(PrefixArgs a, int m
         for (int e = 0; e < 4; ++e) pop[nb][u][e] = pack2<E>(x[8 * u + 2 * e], x[8 * u + 2 * e + 1]);
     }
 
-    // O^T += V^T P^T
+    // O^T += V^T P^T.  A operand (row = dim 32db + ql, contraction = the 8 tokens of (h, u)):
+    // two transposing reads, tokens 16u + 4h + {0..3} and 16u + 8 + 4h + {0..3}.
+    {
+      const int sl = lane & 15, rh = (lane >> 4) & 1;
+      const int trow = 4 * h + (sl >> 2);                       // + 16u + 8x
+      const int tcol = 2 * rh + ((sl & 3) >> 1);                // + 4db, in 16-byte chunks
+      const int tswz = 4 * (sl >> 2);                           // = 4 * (row & 3)
+      const char* vbase = wl + kVtOff + trow * 256 + (sl & 1) * 8;
 #pragma unroll
-    for (int db = 0; db < 4; ++db) {
-      const int d = 32 * db + ql;
+      for (int db = 0; db < 4; ++db) {
+        const int chunk = ((4 * db + tcol) ^ tswz) * 16;
 #pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        const u32x4 va = lds_ld16(wl + kVtOff + d * 64 + (((2 * u + h) ^ ((d >> 2) & 3)) * 16));
+        for (int u = 0; u < 2; ++u) {
+          const u32x2 lo = lds_tr16(vbase + (16 * u) * 256 + chunk);
+          const u32x2 hi = lds_tr16(vbase + (16 * u + 8) * 256 + chunk);
+          const u32x4 va = {lo[0], lo[1], hi[0], hi[1]};
 #pragma unroll
-        for (int nb = 0; nb < NQB; ++nb) oacc[db][nb] = Mfma32<E>::run(va, pop[nb][u], oacc[db][nb]);
+          for (int nb = 0; nb < NQB; ++nb) oacc[db][nb] = Mfma32<E>::run(va, pop[nb][u], oacc[db][nb]);
+        }
       }
     }
   }

@@ -15,6 +15,7 @@ from __future__ import annotations
 import dataclasses
 from typing import Dict, List, Optional, Sequence, Tuple
 
+import numpy as np
 import torch
 
 from . import _lib
@@ -255,6 +256,14 @@ class DecodeTables:
     max_suffix_len: int = 0
     chunk_tokens: int = 0  # 0 = let the library choose
 
+    def suffix_slots_count(self) -> int:
+        """Entries readable behind ``suffix_slots`` (bound for the kernel's early slot fetch)."""
+        if self.suffix_slots is None:
+            return 0
+        if self.suffix_offsets is None:
+            return (self.num_reqs - 1) * self.suffix_table_stride + self.suffix_slots.shape[-1]
+        return self.suffix_slots.numel()
+
     @staticmethod
     def build(prefix_lists: Sequence[Sequence[int]], group_req_cu: Sequence[int],
               suffix_lists: Sequence[Sequence[int]], device) -> "DecodeTables":
@@ -281,14 +290,15 @@ class DecodeTables:
         t.max_suffix_len = max(lens) if lens else 0
         total = sum(lens)
         if t.max_suffix_len > 0:
-            flat = [x for s in suffix_lists for x in s]
-            offs = [0] * B
-            acc = 0
-            for i, n in enumerate(lens):
-                offs[i] = acc
-                acc += n
-            t.suffix_slots = torch.tensor(flat, dtype=torch.int32, device=device)
-            t.suffix_offsets = torch.tensor(offs, dtype=torch.int64, device=device)
+            # padded [B, max] table: a request's list start needs no lookup, so the kernel can fetch
+            # slot ids and the length at the same time
+            width = (t.max_suffix_len + 15) // 16 * 16
+            table = np.zeros((B, width), dtype=np.int32)
+            for i, sl in enumerate(suffix_lists):
+                table[i, : len(sl)] = np.asarray(sl, dtype=np.int32)
+            t.suffix_slots = torch.from_numpy(table).to(device)
+            t.suffix_offsets = None
+            t.suffix_table_stride = width
             t.suffix_lens = torch.tensor(lens, dtype=torch.int32, device=device)
             # parts of about 1/2048 of the batch's tokens, 32 .. 1024 tokens each
             chunk = 32
@@ -325,7 +335,8 @@ def decode_attention(query: torch.Tensor, key_cache: torch.Tensor, value_cache: 
         query.stride(0), out.stride(0), key_cache.stride(0), float(scale),
         tables.num_groups, _ptr(tables.prefix_slots), _ptr(tables.prefix_cu), _ptr(tables.group_req_cu),
         _ptr(tables.group_req_cu_host), tables.max_prefix_len,
-        _ptr(tables.suffix_slots), _ptr(tables.suffix_offsets), tables.suffix_table_stride, _ptr(tables.suffix_lens),
+        _ptr(tables.suffix_slots), _ptr(tables.suffix_offsets), tables.suffix_table_stride,
+        tables.suffix_slots_count(), _ptr(tables.suffix_lens),
         tables.max_suffix_len, tables.chunk_tokens, _ptr(ws), ws.numel(), _stream())
     check(rc, "decode_attention")
     return out
@@ -451,6 +462,6 @@ def prefill_attention(query, key_cache, value_cache, tables: PrefillTables, scal
     rc = lib.ph_prefill_attention(
         _ptr(out), _ptr(query), _ptr(key_cache), _ptr(value_cache), T, tables.num_chunks, H, D, _dtype_code(query),
         query.stride(0), out.stride(0), key_cache.stride(0), float(scale), _ptr(tables.q_cu), _ptr(tables.kv_cu),
-        _ptr(tables.ctx_slots), tables.max_kv_len, _ptr(ws), ws.numel(), _stream())
+        _ptr(tables.ctx_slots), tables.ctx_slots.numel(), tables.max_kv_len, _ptr(ws), ws.numel(), _stream())
     check(rc, "prefill_attention")
     return out
