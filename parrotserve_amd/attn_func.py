@@ -1,0 +1,269 @@
+"""Attention plug-in of the builtin engine on the HIP kernels.
+
+Same contract as the reference's ``AttnFunc`` classes
+(parrot/engine/builtin/attn_func.py:31-55): ``__init__(layer_idx, scaling,
+num_heads, head_dim)``, a static ``init_iteration_state(iteration_state,
+builtin_config, jobs, num_heads, head_size)`` that turns the jobs' context trees
+into index tensors once per iteration, and ``forward(q, k, v, iteration_state)
+-> [T, H*D]`` with Fill tokens first, then one token per Generate job.
+
+``forward`` = KV append by slot, prefill-with-parent-context for the Fill
+tokens, shared-prefix decode (prefix phase + suffix phase + merge) for the
+Generate tokens.  The three reference selector strings all resolve to this
+class (the KV layout is token-granular for all of them here).
+"""
+from __future__ import annotations
+
+import dataclasses
+from typing import Any, Dict, List, Optional, Sequence, Tuple
+
+import torch
+from torch import nn
+
+from . import kernels
+from .mem import get_k_cache, get_v_cache
+from .primitive_job import Fill, Generate
+
+ATTN_FUNCS = [
+    "xformers_with_buffer",
+    "xformers_fill_vllm_paged_attention_generate",
+    "xformers_fill_shared_prompts_generate",
+    "hip_shared_prefix",
+]
+
+
+# --------------------------------------------------------------------------- #
+# host-side index tables (pure python, no device)
+# --------------------------------------------------------------------------- #
+def _lca(context1, context2):
+    """Lowest common ancestor of two context nodes, ``None`` if the trees differ
+    (attn_func.py:412-439)."""
+    if context1 is context2:
+        return context1
+    if context1 is None or context2 is None:
+        return None
+    while context1 is not None:
+        if context1 is context2:
+            return context1
+        if context1.depth > context2.depth:
+            context1 = context1.parent_context
+        elif context1.depth < context2.depth:
+            context2 = context2.parent_context
+        else:
+            context1 = context1.parent_context
+            context2 = context2.parent_context
+    return None
+
+
+def get_shared_context_len(jobs: Sequence[Any]) -> int:
+    """Length of the context shared by ALL jobs (attn_func.py:441-459)."""
+    assert len(jobs) > 0
+    if len(jobs) == 1:
+        return jobs[0].context.get_context_len()
+    lca = _lca(jobs[0].context, jobs[1].context)
+    for job in jobs[2:]:
+        if lca is None:
+            break
+        lca = _lca(lca, job.context)
+    return lca.get_context_len() if lca is not None else 0
+
+
+@dataclasses.dataclass
+class IterationTables:
+    """Index tables of one iteration as python lists (what the reference uploads
+    as tensors, attn_func.py:462-599, at block_size 1)."""
+
+    flash_context_len: int
+    flash_block_table: List[int]
+    paged_block_tables: List[List[int]]  # ragged; the reference pads with 0
+    paged_context_lens: List[int]
+    slot_mapping: List[int]  # flat [T]
+    fill_q_lens: List[int]
+    fill_kv_lens: List[int]
+    fill_slots: List[int]
+    fill_slot_lists: List[List[int]]
+    # prefix groups over the Generate jobs: (prefix slot list, generate indices)
+    groups: List[Tuple[List[int], List[int]]]
+    num_fill_tokens: List[int]
+    num_generates: int
+
+
+def build_iteration_tables(jobs: Sequence[Any], grouping: str = "lca") -> IterationTables:
+    """``grouping="lca"``: one prefix shared by every job of the iteration, the
+    reference's rule.  ``grouping="parent"``: Generate jobs forked from the same
+    parent context form a group whose prefix is that parent's whole context, so
+    several prompt groups can share the iteration."""
+    assert grouping in ("lca", "parent")
+    P = get_shared_context_len(jobs) if grouping == "lca" else 0
+    slots0 = jobs[0].context.get_context_slot_ids()
+    t = IterationTables(P, slots0[:P], [], [], [], [], [], [], [], [], [], 0)
+    gen_full: List[List[int]] = []
+    gen_parent: List[Any] = []
+    for job in jobs:
+        slots = job.context.get_context_slot_ids()
+        if isinstance(job, Fill):
+            n = len(job.token_ids)
+            t.num_fill_tokens.append(n)
+            t.fill_q_lens.append(n)
+            t.fill_kv_lens.append(len(slots))
+            t.fill_slots.extend(slots)
+            t.fill_slot_lists.append(slots)
+        elif isinstance(job, Generate):
+            n = 1
+            t.num_generates += 1
+            gen_full.append(slots)
+            gen_parent.append(job.context.parent_context)
+        else:
+            raise TypeError(f"unknown job type {type(job)}")
+        t.slot_mapping.extend(slots[-n:])
+    if grouping == "lca":
+        for slots in gen_full:
+            t.paged_block_tables.append(slots[P:])
+            t.paged_context_lens.append(len(slots) - P)
+        if P > 0 and gen_full:
+            t.groups.append((t.flash_block_table, list(range(len(gen_full)))))
+    else:
+        by_parent: Dict[int, int] = {}
+        for i, (slots, parent) in enumerate(zip(gen_full, gen_parent)):
+            plen = parent.get_context_len() if parent is not None else 0
+            t.paged_block_tables.append(slots[plen:])
+            t.paged_context_lens.append(len(slots) - plen)
+            if plen == 0:
+                continue
+            g = by_parent.get(id(parent))
+            if g is None:
+                by_parent[id(parent)] = len(t.groups)
+                t.groups.append((slots[:plen], [i]))
+            else:
+                t.groups[g][1].append(i)
+    return t
+
+
+# --------------------------------------------------------------------------- #
+# the plug-in
+# --------------------------------------------------------------------------- #
+class AttnFunc(nn.Module):
+    """Base class (attn_func.py:31-55)."""
+
+    def __init__(self, layer_idx: int, scaling: float, num_heads: int, head_dim: int):
+        super().__init__()
+        self.layer_idx = layer_idx
+        self.scaling = scaling
+        self.num_heads = num_heads
+        self.head_dim = head_dim
+
+    @staticmethod
+    def init_iteration_state(iteration_state, builtin_config, jobs, num_heads: int, head_size: int):
+        raise NotImplementedError
+
+
+class HipSharedPrefixAttn(AttnFunc):
+    """Fill: prefill with parent context.  Generate: shared-prefix decode."""
+
+    grouping = "lca"
+
+    @classmethod
+    def _init(cls, iteration_state, builtin_config, jobs, num_heads, head_size):
+        tabs = build_iteration_tables(jobs, cls.grouping)
+        device = builtin_config.device
+        st = iteration_state
+        st.num_fill_tokens.extend(tabs.num_fill_tokens)
+        st.generation_sampling_config.extend(j.sampling_config for j in jobs if isinstance(j, Generate))
+        st.tables = tabs
+        # names the reference attaches (attn_func.py:571-599)
+        st.flash_context_len = tabs.flash_context_len
+        st.slot_mapping = torch.tensor(tabs.slot_mapping, dtype=torch.int32, device=device)
+        st.fill_tables = None
+        if tabs.fill_q_lens:
+            st.fill_tables = kernels.PrefillTables.build(tabs.fill_q_lens, tabs.fill_slot_lists, device)
+        st.decode_tables = None
+        st.decode_perm = None
+        if tabs.num_generates:
+            # requests of one prefix group must be adjacent: order = groups first, ungrouped last
+            order: List[int] = []
+            gcu = [0]
+            for _, members in tabs.groups:
+                order.extend(members)
+                gcu.append(len(order))
+            grouped = set(order)
+            order.extend(i for i in range(tabs.num_generates) if i not in grouped)
+            suffix = [tabs.paged_block_tables[i] for i in order]
+            st.decode_tables = kernels.DecodeTables.build([p for p, _ in tabs.groups], gcu if tabs.groups else [],
+                                                          suffix, device)
+            if order != list(range(tabs.num_generates)):
+                perm = torch.tensor(order, dtype=torch.int64, device=device)
+                inv = torch.empty_like(perm)
+                inv[perm] = torch.arange(len(order), dtype=torch.int64, device=device)
+                st.decode_perm = (perm, inv)
+
+    @staticmethod
+    def init_iteration_state(iteration_state, builtin_config, jobs, num_heads: int, head_size: int):
+        HipSharedPrefixAttn._init(iteration_state, builtin_config, jobs, num_heads, head_size)
+
+    def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, iteration_state) -> torch.Tensor:
+        st = iteration_state
+        k_cache = get_k_cache(self.layer_idx)
+        v_cache = get_v_cache(self.layer_idx)
+        kernels.kv_append(k, v, k_cache, v_cache, st.slot_mapping)
+        T = q.shape[0]
+        if q.stride(1) != self.head_dim or q.stride(2) != 1:
+            q = q.contiguous()
+        output = torch.empty((T, self.num_heads, self.head_dim), dtype=q.dtype, device=q.device)
+        nf = st.num_total_fill_tokens
+        if nf > 0:
+            kernels.prefill_attention(q[:nf], k_cache, v_cache, st.fill_tables, scale=self.scaling, out=output[:nf])
+        if st.num_generation_jobs > 0:
+            q_gen = q[nf:]
+            if st.decode_perm is None:
+                kernels.decode_attention(q_gen, k_cache, v_cache, st.decode_tables, scale=self.scaling, out=output[nf:])
+            else:
+                perm, inv = st.decode_perm
+                o = kernels.decode_attention(q_gen.index_select(0, perm), k_cache, v_cache, st.decode_tables,
+                                             scale=self.scaling)
+                output[nf:] = o.index_select(0, inv)
+        return output.view(-1, self.num_heads * self.head_dim)
+
+
+class HipGroupedPrefixAttn(HipSharedPrefixAttn):
+    """Same kernels; prefix groups are detected per fork parent, so several prompt
+    groups in one batch each keep their shared-prefix phase."""
+
+    grouping = "parent"
+
+    @staticmethod
+    def init_iteration_state(iteration_state, builtin_config, jobs, num_heads: int, head_size: int):
+        HipGroupedPrefixAttn._init(iteration_state, builtin_config, jobs, num_heads, head_size)
+
+
+def get_attn_func(attn_func_name: str):
+    """Selector of ``instance.attn_func`` (attn_func.py:711-737): unknown names raise ValueError."""
+    if attn_func_name in ("xformers_with_buffer", "xformers_fill_vllm_paged_attention_generate",
+                          "xformers_fill_shared_prompts_generate"):
+        return HipSharedPrefixAttn
+    if attn_func_name == "hip_shared_prefix":
+        return HipGroupedPrefixAttn
+    raise ValueError(f"Unknown attention function name: {attn_func_name}. Supported attetion functions: {ATTN_FUNCS}")
+
+
+@dataclasses.dataclass
+class BuiltinConfig:
+    """The fields of ``BuiltinConfig`` the attention path reads (parrot/engine/config.py:28-60)."""
+
+    num_kv_cache_blocks: int
+    attn_func: Any = "xformers_fill_shared_prompts_generate"
+    dtype: Any = torch.float16
+    device: Any = "cuda"
+    block_size: int = 1
+    max_seq_len: Optional[int] = None
+
+    def __post_init__(self):
+        if isinstance(self.dtype, str):
+            table = {"float16": torch.float16, "bfloat16": torch.bfloat16}
+            if self.dtype not in table:
+                raise ValueError(f"Unknown dtype {self.dtype}")
+            self.dtype = table[self.dtype]
+        if self.block_size != 1:
+            raise ValueError("block_size must be 1: the KV pool is token-granular")
+        self.attn_func_name = self.attn_func if isinstance(self.attn_func, str) else self.attn_func.__name__
+        if isinstance(self.attn_func, str):
+            self.attn_func = get_attn_func(self.attn_func)

@@ -92,21 +92,6 @@ __global__ __launch_bounds__(256, 1) void prefix_mfma_kernel(PrefixArgs a, int m
   char* wl = smem + w * kWaveLds;
   const int32_t* slots = a.slots + poff;
 
-  // Q as the B operand: column = query ql (+32 nb), contraction chunk (h, s) = dims 64h + 8s .. +8
-  u32x4 qop[NQB][8];
-#pragma unroll
-  for (int nb = 0; nb < NQB; ++nb) {
-    const int q = 32 * nb + ql;
-    const bool ok = q < nq;
-    const uint16_t* qp = a.q + (int64_t)(qbase + (ok ? q : 0)) * a.q_stride + head * kPD + 64 * h;
-#pragma unroll
-    for (int s = 0; s < 8; ++s) {
-      u32x4 v = ld16(qp + 8 * s);
-      if (!ok) v = u32x4{0, 0, 0, 0};
-      qop[nb][s] = v;
-    }
-  }
-
   float16_t oacc[4][NQB];
   float m[NQB], lsum[NQB];
 #pragma unroll
@@ -142,6 +127,23 @@ __global__ __launch_bounds__(256, 1) void prefix_mfma_kernel(PrefixArgs a, int m
     fetch_rows();
     if (tb + 4 * kTile < s1) fetch_slots(tb + 4 * kTile);
   }
+
+  // (issued after the first K/V rows so the two latencies overlap)
+  // Q as the B operand: column = query ql (+32 nb), contraction chunk (h, s) = dims 64h + 8s .. +8
+  u32x4 qop[NQB][8];
+#pragma unroll
+  for (int nb = 0; nb < NQB; ++nb) {
+    const int q = 32 * nb + ql;
+    const bool ok = q < nq;
+    const uint16_t* qp = a.q + (int64_t)(qbase + (ok ? q : 0)) * a.q_stride + head * kPD + 64 * h;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      u32x4 v = ld16(qp + 8 * s);
+      if (!ok) v = u32x4{0, 0, 0, 0};
+      qop[nb][s] = v;
+    }
+  }
+
 
   for (; tb < s1; tb += 4 * kTile) {
     // registers -> LDS, both tiles row-major [token][dim] with XOR-swizzled 16-byte chunks

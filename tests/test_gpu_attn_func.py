@@ -1,0 +1,206 @@
+"""GPU parity of the AttnFunc plug-in and the decoder-layer wiring against the CPU oracle."""
+import pytest
+import torch
+
+from oracle.ref_ops import (ref_cos_sin_cache, ref_decode_attention, ref_prefill_with_parent, ref_rms_norm,
+                            ref_rope_neox)
+
+pytestmark = pytest.mark.gpu
+
+TOL = dict(atol=2e-3, rtol=1e-2)
+
+
+class _Cfg:
+    def __init__(self, heads, hidden):
+        self.num_attention_heads = heads
+        self.hidden_size = hidden
+
+
+def _build_forest(pool, rng_seed, n_groups, branches, prefix, with_fills):
+    """parents (already filled) -> forked children; returns jobs in engine order (Fill first)."""
+    from parrotserve_amd.context import BlockContext
+    from parrotserve_amd.primitive_job import Fill, Generate
+
+    g = torch.Generator().manual_seed(rng_seed)
+    cid = 0
+    fills, gens = [], []
+    for gi in range(n_groups):
+        parent = BlockContext(cid, None, pool, 1)
+        cid += 1
+        parent.allocate(prefix + 7 * gi)
+        for b in range(branches):
+            child = BlockContext(cid, parent, pool, 1)
+            cid += 1
+            child.allocate(int(torch.randint(1, 30, (1,), generator=g)))
+            job = Generate(0, cid, child.context_id, parent.context_id, sampling_config=None)
+            job.context = child
+            gens.append(job)
+        if with_fills:
+            child = BlockContext(cid, parent, pool, 1)
+            cid += 1
+            n = int(torch.randint(1, 50, (1,), generator=g))
+            child.allocate(n)
+            job = Fill(0, cid, child.context_id, parent.context_id, token_ids=list(range(n)))
+            job.context = child
+            fills.append(job)
+    # interleave groups among the generates so that grouping has to reorder them
+    perm = torch.randperm(len(gens), generator=g).tolist()
+    return fills + [gens[i] for i in perm]
+
+
+@pytest.mark.parametrize("name", ["xformers_fill_shared_prompts_generate", "hip_shared_prefix"])
+@pytest.mark.parametrize("n_groups,with_fills", [(1, False), (1, True), (3, True)])
+def test_attn_func_forward_matches_oracle(dev, name, n_groups, with_fills):
+    from parrotserve_amd import mem
+    from parrotserve_amd.attn_func import BuiltinConfig
+    from parrotserve_amd.context import RecyclePool
+    from parrotserve_amd.iter_state import IterationState
+    from parrotserve_amd.primitive_job import Fill
+
+    H, D, slots = 8, 128, 4096
+    pool = RecyclePool(pool_size=slots)
+    jobs = _build_forest(pool, 5 + n_groups, n_groups, 6, 150, with_fills)
+    cfg = BuiltinConfig(num_kv_cache_blocks=slots, attn_func=name, dtype=torch.float16, device=dev)
+    store = mem.init_model_cache_storage(2, slots, H, D, torch.float16, dev)
+    g = torch.Generator().manual_seed(3)
+    kc_cpu = torch.randn(slots, H, D, generator=g).half()
+    vc_cpu = torch.randn(slots, H, D, generator=g).half()
+    store.k_cache[1].copy_(kc_cpu)
+    store.v_cache[1].copy_(vc_cpu)
+
+    st = IterationState(jobs, _Cfg(H, H * D), cfg)
+    n_new = [len(j.token_ids) if isinstance(j, Fill) else 1 for j in jobs]
+    T = sum(n_new)
+    assert st.num_total_fill_tokens + st.num_generation_jobs == T
+    qkv = torch.randn(T, 3 * H * D, generator=g).half()
+    q, k, v = (t.view(T, H, D) for t in qkv.chunk(3, dim=-1))  # strided views, as the model passes them
+
+    # oracle: append, then per job attention over its whole context
+    kc_ref, vc_ref = kc_cpu.clone(), vc_cpu.clone()
+    pos = 0
+    ref = torch.zeros(T, H, D, dtype=torch.float16)
+    for j, n in zip(jobs, n_new):
+        sl = torch.tensor(j.context.get_context_slot_ids())
+        kc_ref[sl[-n:]] = k[pos : pos + n]
+        vc_ref[sl[-n:]] = v[pos : pos + n]
+        pos += n
+    pos = 0
+    for j, n in zip(jobs, n_new):
+        sl = torch.tensor(j.context.get_context_slot_ids())
+        if isinstance(j, Fill):
+            ref[pos : pos + n] = ref_prefill_with_parent(q[pos : pos + n], kc_ref, vc_ref, [n], [sl])
+        else:
+            ref[pos : pos + 1] = ref_decode_attention(q[pos : pos + 1], kc_ref, vc_ref, [sl])
+        pos += n
+
+    attn = cfg.attn_func(layer_idx=1, scaling=D ** -0.5, num_heads=H, head_dim=D)
+    dq = qkv.to(dev)
+    q_d, k_d, v_d = (t.view(T, H, D) for t in dq.chunk(3, dim=-1))
+    out = attn(q_d, k_d, v_d, st)
+    assert out.shape == (T, H * D)
+    torch.testing.assert_close(out.cpu().view(T, H, D).float(), ref.float(), **TOL)
+    # the append really happened, bit-exact, and only at the new tokens' slots
+    assert torch.equal(store.k_cache[1].cpu().view(torch.int16), kc_ref.view(torch.int16))
+    assert torch.equal(store.v_cache[1].cpu().view(torch.int16), vc_ref.view(torch.int16))
+
+
+def test_decoder_layer_config5_scaled(dev):
+    """Config 5's recipe scaled down (fp16, weights N(0, 0.02), RMSNorm -> QKV -> RoPE -> prefix groups x
+    branches -> shared-prefix + suffix attention -> O-proj -> MLP): hidden 640, 5 heads x 128, FFN 1728,
+    2 groups x 8 branches, prefix 300, suffix U[4,40], seed 4."""
+    from parrotserve_amd import mem, synth
+    from parrotserve_amd.attn_func import BuiltinConfig
+    from parrotserve_amd.context import BlockContext, RecyclePool
+    from parrotserve_amd.iter_state import IterationState
+    from parrotserve_amd.llama_layer import LlamaDecoderLayer
+    from parrotserve_amd.primitive_job import Generate
+
+    case = synth.config5(groups=2, branches=8, prefix=300, s_lo=4, s_hi=40, hidden=640, heads=5, ffn=1728,
+                         pool_slots=1 << 12)
+    dec = case.decode
+    B, H, D, hidden = dec.num_reqs, 5, 128, 640
+    slots = dec.pool_slots
+    store = mem.init_model_cache_storage(1, slots, H, D, torch.float16, dev, max_seq_len=1024, rope_theta=case.theta)
+    kc, vc = synth.pool_to_device(dec.k_rows, dec.v_rows, dec.used_slots, slots, dev)
+    store.k_cache[0].copy_(kc)
+    store.v_cache[0].copy_(vc)
+
+    # contexts whose slot lists are exactly the synthetic case's (ids handed out through a scripted pool)
+    class _Scripted(RecyclePool):
+        def __init__(self, ids):
+            super().__init__(pool_size=None)
+            self._ids = list(ids)
+
+        def allocate(self):
+            return self._ids.pop(0)
+
+    jobs = []
+    for gi in range(2):
+        parent = BlockContext(gi, None, _Scripted(dec.used_slots[dec.prefix_lists[gi]].tolist()), 1)
+        parent.allocate(300)
+        for b in range(8):
+            r = gi * 8 + b
+            ids = dec.used_slots[dec.suffix_lists[r]].tolist()
+            child = BlockContext(100 + r, parent, _Scripted(ids), 1)
+            child.allocate(len(ids))
+            j = Generate(0, r, child.context_id, parent.context_id)
+            j.context = child
+            jobs.append(j)
+    cfg = BuiltinConfig(num_kv_cache_blocks=slots, attn_func="hip_shared_prefix", dtype=torch.float16, device=dev)
+    st = IterationState(jobs, type("C", (), dict(num_attention_heads=H, hidden_size=hidden))(), cfg)
+    assert st.decode_tables.num_groups == 2 and st.decode_perm is None
+
+    layer = LlamaDecoderLayer(hidden, H, 1728, case.eps, 0, cfg.attn_func).half().to(dev)
+    w = case.weights
+    with torch.no_grad():
+        layer.self_attn.qkv_proj.weight.copy_(w["qkv_proj"])
+        layer.self_attn.o_proj.weight.copy_(w["o_proj"])
+        layer.mlp.gate_proj.weight.copy_(w["gate_proj"])
+        layer.mlp.up_proj.weight.copy_(w["up_proj"])
+        layer.mlp.down_proj.weight.copy_(w["down_proj"])
+    x = case.x.to(dev)
+    pos = case.positions.to(dev)
+
+    # GPU, stage by stage (same calls LlamaDecoderLayer.forward makes), so each HIP op is checked on the
+    # inputs it really saw
+    with torch.inference_mode():
+        h1 = layer.input_layernorm(x)
+        qkv = layer.self_attn.qkv_proj(h1)
+        qkv_before = qkv.clone()
+        q, k, v = torch.chunk(qkv, 3, dim=-1)
+        from parrotserve_amd.kernels import vllm_rotary_emb
+        vllm_rotary_emb(pos, q, k, mem.get_cos_sin_cache(), head_size=D)
+        attn_out = layer.self_attn.attn_func(q.view(B, H, D), k.view(B, H, D), v.view(B, H, D), st)
+        mem.Model_Cache.k_cache[0].copy_(kc)  # undo the append, then run the whole layer in one go
+        mem.Model_Cache.v_cache[0].copy_(vc)
+        y = layer(x, pos, st)
+
+    # 1. RMSNorm
+    ref_h1 = ref_rms_norm(case.x, w["input_layernorm"], case.eps)
+    torch.testing.assert_close(h1.cpu().float(), ref_h1.float(), **TOL)
+    # 2. RoPE on the GPU's own qkv (bit-exact with the reference kernel's arithmetic)
+    cache = ref_cos_sin_cache(1024, D, case.theta, torch.float16)
+    torch.testing.assert_close(mem.get_cos_sin_cache().cpu().float(), cache.float(), atol=1e-3, rtol=0)
+    qb, kb, vb = qkv_before.cpu().chunk(3, dim=-1)
+    rq, rk = ref_rope_neox(case.positions, qb, kb, mem.get_cos_sin_cache().cpu(), D, elem_rounding=True)
+    assert torch.equal(q.cpu().view(torch.int16), rq.contiguous().view(torch.int16))
+    assert torch.equal(k.cpu().view(torch.int16), rk.contiguous().view(torch.int16))
+    # 3. append + shared-prefix attention on those q/k/v
+    k_rows, v_rows = dec.k_rows.clone(), dec.v_rows.clone()
+    for r in range(B):
+        last = int(dec.suffix_lists[r][-1])
+        k_rows[last] = rk.view(B, H, D)[r]
+        v_rows[last] = vb.reshape(B, H, D)[r]
+    ref_attn = ref_decode_attention(rq.view(B, H, D), k_rows, v_rows, dec.full_lists())
+    torch.testing.assert_close(attn_out.cpu().view(B, H, D).float(), ref_attn.float(), **TOL)
+    # 4. whole layer vs an fp32 CPU evaluation that takes the checked attention output
+    a = attn_out.cpu().float()
+    hcpu = case.x.float() + (a @ w["o_proj"].float().t()).half().float()
+    hcpu = hcpu.half()
+    h2 = ref_rms_norm(hcpu, w["post_attention_layernorm"], case.eps).float()
+    gate = (h2 @ w["gate_proj"].float().t()).half().float()
+    up = (h2 @ w["up_proj"].float().t()).half().float()
+    act = (torch.nn.functional.silu(gate).half().float() * up).half().float()
+    mlp = (act @ w["down_proj"].float().t()).half().float()
+    ref_y = (hcpu.float() + mlp).half()
+    torch.testing.assert_close(y.cpu().float(), ref_y.float(), atol=2e-2, rtol=2e-2)

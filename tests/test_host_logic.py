@@ -1,0 +1,179 @@
+"""Host-side slot indexing of the product package against the list-based oracle model (bit-exact integers)."""
+import random
+
+import pytest
+
+from oracle.ref_context import RefContext, RefPoolError, RefRecyclePool, ref_iteration_tables, ref_shared_context_len
+from parrotserve_amd.attn_func import (BuiltinConfig, HipGroupedPrefixAttn, HipSharedPrefixAttn,
+                                       build_iteration_tables, get_attn_func, get_shared_context_len)
+from parrotserve_amd.context import BlockContext, ParrotError, RecyclePool
+from parrotserve_amd.primitive_job import Fill, Generate
+
+
+def test_pool_random_trace_matches_oracle():
+    rng = random.Random(0)
+    a, b = RecyclePool(pool_size=64), RefRecyclePool(pool_size=64)
+    live = []
+    for _ in range(3000):
+        if live and rng.random() < 0.45:
+            i = live.pop(rng.randrange(len(live)))
+            a.free(i)
+            b.free(i)
+        else:
+            try:
+                x = a.allocate()
+            except ParrotError:
+                with pytest.raises(RefPoolError):
+                    b.allocate()
+                a.allocated_num -= 1  # the reference counts the failed attempt too; keep both models aligned
+                b.allocated_num -= 1
+                continue
+            assert x == b.allocate()
+            live.append(x)
+        assert a.get_allocated_num() == b.allocated_num
+    with pytest.raises(ValueError):
+        i = live.pop()
+        a.free(i)
+        a.free(i)
+
+
+def test_pool_never_issues_last_id():
+    p = RecyclePool(pool_size=3)
+    assert [p.allocate(), p.allocate()] == [0, 1]
+    with pytest.raises(ParrotError):
+        p.allocate()
+
+
+def _random_forest(seed, n_ctx=40):
+    """The same random fork/allocate/destroy script applied to the product and the oracle models."""
+    rng = random.Random(seed)
+    pa, pb = RecyclePool(pool_size=100000), RefRecyclePool(pool_size=100000)
+    A, B = {}, {}
+    next_id = 0
+    for _ in range(n_ctx * 3):
+        r = rng.random()
+        if r < 0.5 or not A:
+            parent = rng.choice(list(A)) if A and rng.random() < 0.8 else None
+            A[next_id] = BlockContext(next_id, A.get(parent), pa, 1)
+            B[next_id] = RefContext(next_id, B.get(parent), pb)
+            n = rng.randrange(0, 9)
+            A[next_id].allocate(n)
+            B[next_id].allocate(n)
+            next_id += 1
+        elif r < 0.85:
+            c = rng.choice(list(A))
+            n = rng.randrange(1, 5)
+            A[c].allocate(n)
+            B[c].allocate(n)
+        else:
+            leaves = [c for c in A if not A[c].sub_context_ids]
+            c = rng.choice(leaves)
+            A.pop(c).destruction()
+            B.pop(c).destroy()
+    return A, B
+
+
+@pytest.mark.parametrize("seed", range(5))
+def test_context_tree_matches_oracle(seed):
+    A, B = _random_forest(seed)
+    assert A.keys() == B.keys()
+    for c in A:
+        assert A[c].get_context_slot_ids() == B[c].context_slot_ids()
+        assert A[c].get_context_block_ids() == B[c].context_slot_ids()
+        assert A[c].get_context_len() == B[c].context_len()
+        assert A[c].get_this_context_len() == B[c].this_len()
+        assert A[c].depth == B[c].depth
+    root = next(iter(A.values()))
+    if root.sub_context_ids:
+        with pytest.raises(AssertionError):
+            root.destruction()
+
+
+def _jobs_for(A, B, seed):
+    rng = random.Random(seed)
+    ids = [c for c in A if A[c].get_this_context_len() > 0]
+    rng.shuffle(ids)
+    ids = ids[: max(2, len(ids) // 2)]
+    fills = ids[: len(ids) // 3]
+    gens = ids[len(ids) // 3 :]
+    ja, jb = [], []
+    for c in fills:  # Fill jobs first (builtin_runner.py:76)
+        n = rng.randrange(1, A[c].get_this_context_len() + 1)
+        f = Fill(0, 0, c, -1, token_ids=list(range(n)))
+        f.context = A[c]
+        ja.append(f)
+        jb.append(dict(kind="fill", context=B[c], num_tokens=n))
+    for c in gens:
+        g = Generate(0, 0, c, -1, sampling_config=None)
+        g.context = A[c]
+        ja.append(g)
+        jb.append(dict(kind="generate", context=B[c], num_tokens=1))
+    return ja, jb
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_iteration_tables_match_oracle(seed):
+    A, B = _random_forest(seed + 10)
+    ja, jb = _jobs_for(A, B, seed)
+    t = build_iteration_tables(ja, "lca")
+    ref = ref_iteration_tables(jb)
+    assert get_shared_context_len(ja) == ref_shared_context_len([j["context"] for j in jb])
+    for key in ("flash_context_len", "flash_block_table", "paged_block_tables", "paged_context_lens", "slot_mapping",
+                "fill_q_lens", "fill_kv_lens", "fill_slots"):
+        assert getattr(t, key) == ref[key], key
+
+
+def test_shared_prefix_scenario_tables():
+    """The reference's shared-prefix scenario: one parent Fill context, children fork and generate
+    (tests/engine/builtin/test_shared_prefix.py:7-54 in the reference drives this shape)."""
+    pool = RecyclePool(pool_size=10000)
+    parent = BlockContext(0, None, pool, 1)
+    parent.allocate(100)
+    kids = []
+    for i in range(8):
+        c = BlockContext(1 + i, parent, pool, 1)
+        c.allocate(3 + i)
+        g = Generate(0, i, 1 + i, 0)
+        g.context = c
+        kids.append(g)
+    t = build_iteration_tables(kids, "lca")
+    assert t.flash_context_len == 100 and t.flash_block_table == list(range(100))
+    assert t.paged_context_lens == [3 + i for i in range(8)]
+    assert t.slot_mapping == [k.context.token_kv_slot_ids[-1] for k in kids]
+    assert t.groups == [(list(range(100)), list(range(8)))]
+    tp = build_iteration_tables(kids, "parent")
+    assert tp.groups == t.groups and tp.paged_block_tables == t.paged_block_tables
+
+
+def test_parent_grouping_two_prompt_groups_and_a_loner():
+    pool = RecyclePool(pool_size=10000)
+    p1 = BlockContext(0, None, pool, 1); p1.allocate(10)
+    p2 = BlockContext(1, None, pool, 1); p2.allocate(20)
+    jobs = []
+    for i, par in enumerate([p1, p2, p1, None, p2]):
+        c = BlockContext(10 + i, par, pool, 1)
+        c.allocate(2)
+        g = Generate(0, i, 10 + i, -1)
+        g.context = c
+        jobs.append(g)
+    lca = build_iteration_tables(jobs, "lca")
+    assert lca.flash_context_len == 0 and lca.groups == []  # the reference's single-LCA rule finds nothing shared
+    assert [len(x) for x in lca.paged_block_tables] == [12, 22, 12, 2, 22]
+    par = build_iteration_tables(jobs, "parent")
+    assert par.groups == [(p1.token_kv_slot_ids, [0, 2]), (p2.token_kv_slot_ids, [1, 4])]
+    assert par.paged_context_lens == [2, 2, 2, 2, 2]
+
+
+def test_selector_and_config():
+    for name in ("xformers_with_buffer", "xformers_fill_vllm_paged_attention_generate",
+                 "xformers_fill_shared_prompts_generate"):
+        assert get_attn_func(name) is HipSharedPrefixAttn
+    assert get_attn_func("hip_shared_prefix") is HipGroupedPrefixAttn
+    with pytest.raises(ValueError):
+        get_attn_func("flash_attn_3")
+    cfg = BuiltinConfig(num_kv_cache_blocks=16, attn_func="hip_shared_prefix", dtype="float16", device="cpu")
+    assert cfg.attn_func is HipGroupedPrefixAttn and cfg.attn_func_name == "hip_shared_prefix"
+    with pytest.raises(ValueError):
+        BuiltinConfig(num_kv_cache_blocks=16, block_size=16)
+    with pytest.raises(ValueError):
+        BlockContext(0, None, RecyclePool(), block_size=16)
