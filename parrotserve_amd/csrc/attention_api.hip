@@ -407,6 +407,7 @@ extern "C" size_t ph_prefill_workspace_bytes(int64_t num_tokens, int64_t num_hea
                                              int64_t max_kv_len) {
   if (num_tokens <= 0 || num_heads <= 0 || head_dim <= 0) return 0;
   const DecodePlan p = plan_decode(num_tokens, num_heads, 0, 0, max_kv_len, 0);
+  if (prefix_mfma_supported(PH_F16, (int)head_dim)) return 256 + (size_t)round_up((num_tokens + 2) * 4, 256);
   return (size_t)round_up(num_tokens * 8, 256) + (size_t)round_up(num_tokens * 4, 256) +
          plan_bytes(p, num_tokens, num_heads, head_dim);
 }
@@ -427,6 +428,26 @@ extern "C" int ph_prefill_attention(void* out, const void* q, const void* k_cach
     return PH_ERR_WORKSPACE;
   if (((uintptr_t)workspace & 255u) != 0) return PH_ERR_ALIGN;
   hipStream_t st = (hipStream_t)stream;
+  if (prefix_mfma_supported(dtype, D)) {
+    if (num_chunks > num_tokens) return PH_ERR_ARG;  // every chunk holds at least one query (tile_cu fits the workspace)
+    PrefillArgs pa{};
+    pa.q = (const uint16_t*)q;
+    pa.q_stride = q_stride;
+    pa.kc = (const uint16_t*)k_cache;
+    pa.vc = (const uint16_t*)v_cache;
+    pa.row_stride = cache_stride_n;
+    pa.out = (uint16_t*)out;
+    pa.out_stride = out_stride;
+    pa.q_cu = q_cu;
+    pa.kv_cu = kv_cu;
+    pa.ctx_slots = ctx_slots;
+    pa.tile_cu = (int32_t*)workspace;
+    pa.num_chunks = (int)num_chunks;
+    pa.H = H;
+    pa.scale_log2e = scale * kLog2e;
+    const int64_t max_tiles = num_tokens / 64 + num_chunks;
+    return launch_prefill_mfma(pa, dtype, D, (int)max_tiles, st);
+  }
   int64_t* offsets = (int64_t*)workspace;
   int32_t* lens = (int32_t*)((char*)workspace + round_up(num_tokens * 8, 256));
   void* dws = (char*)lens + round_up(num_tokens * 4, 256);

@@ -65,7 +65,26 @@ struct PrefixArgs {
   float scale_log2e;
 };
 
+struct PrefillArgs {
+  const uint16_t* q;
+  int64_t q_stride;
+  const uint16_t* kc;
+  const uint16_t* vc;
+  int64_t row_stride;
+  uint16_t* out;
+  int64_t out_stride;
+  const int32_t* q_cu;       // [C+1] device
+  const int32_t* kv_cu;      // [C+1] device
+  const int32_t* ctx_slots;
+  int32_t* tile_cu;          // [C+1] scratch: 64-query tiles before each chunk
+  int num_chunks;
+  int H;
+  float scale_log2e;
+};
+
 int launch_partial(const PartialArgs& a, int dtype, int D, hipStream_t st);
+// MFMA prefill: grid (head, query tile); max_tiles bounds the tile count (sum of ceil(n_c / 64)).
+int launch_prefill_mfma(const PrefillArgs& a, int dtype, int D, int max_tiles, hipStream_t st);
 int launch_merge(const MergeArgs& a, int dtype, int D, hipStream_t st);
 int launch_clear_ml(float* ml, int64_t entries, hipStream_t st);
 // MFMA shared-prefix kernel: grid (split, head, group x m-tile).

@@ -60,40 +60,30 @@ __device__ __forceinline__ u32x2 lds_tr16(const char* p) {
   return __builtin_bit_cast(u32x2, v);
 }
 
-template <typename E, int NQB>
-__global__ __launch_bounds__(256, 1) void prefix_mfma_kernel(PrefixArgs a, int mtiles) {
-  extern __shared__ __attribute__((aligned(16))) char smem[];
-  const int split = blockIdx.x, head = blockIdx.y;
-  const int g = blockIdx.z / mtiles, mt = blockIdx.z - g * mtiles;
-  int r0 = 0, r1 = a.B, poff = 0, plen = a.fixed_prefix_len;
-  if (a.prefix_cu) {
-    r0 = a.group_req_cu[g];
-    r1 = a.group_req_cu[g + 1];
-    poff = a.prefix_cu[g];
-    plen = a.prefix_cu[g + 1] - poff;
-  }
-  const int qbase = r0 + mt * 32 * NQB;
-  const int nq = min(32 * NQB, r1 - qbase);
-  if (nq <= 0) return;
-  const int s0 = split * a.split_tokens;
-  const int s1 = min(plen, s0 + a.split_tokens);
-  if (s0 >= plen) {  // this group's prefix ends before the split: mark the part empty
-    for (int q = threadIdx.x; q < nq; q += 256) {
-      const int64_t pr = ((int64_t)split * a.B + qbase + q) * a.H + head;
-      a.ml[pr * 2] = -INFINITY;
-      a.ml[pr * 2 + 1] = 0.f;
-    }
-    return;
-  }
+// One 64-query (NQB = 2) or 32-query (NQB = 1) tile against the slot list [s0, s1).
+struct TileWork {
+  const uint16_t* qrow0;  // first query row of the tile, already offset to the head
+  int64_t q_stride;
+  int nq;                 // live queries in the tile
+  const int32_t* slots;   // slot list base
+  int s0, s1;             // token range of this workgroup
+  int causal_off;         // CAUSAL: query i sees token t iff t <= causal_off + i
+};
 
+// Runs the tile on all four waves; on return wave 0 holds the folded (unnormalised) accumulators,
+// the running maxima and per-lane partial sums of the softmax denominators.
+template <typename E, int NQB, bool CAUSAL>
+__device__ __forceinline__ void attn_tile(const TileWork& wk, const uint16_t* __restrict__ kc,
+                                          const uint16_t* __restrict__ vc, int64_t row_stride, int head,
+                                          float scale_log2e, char* smem, float16_t (&oacc)[4][NQB], float (&m)[NQB],
+                                          float (&lsum)[NQB]) {
   const int lane = threadIdx.x & 63;
   const int w = threadIdx.x >> 6;
   const int h = lane >> 5, ql = lane & 31;
   char* wl = smem + w * kWaveLds;
-  const int32_t* slots = a.slots + poff;
+  const int32_t* slots = wk.slots;
+  const int s1 = wk.s1;
 
-  float16_t oacc[4][NQB];
-  float m[NQB], lsum[NQB];
 #pragma unroll
   for (int nb = 0; nb < NQB; ++nb) {
     m[nb] = -INFINITY;
@@ -116,12 +106,12 @@ __global__ __launch_bounds__(256, 1) void prefix_mfma_kernel(PrefixArgs a, int m
   auto fetch_rows = [&]() {
 #pragma unroll
     for (int r = 0; r < 8; ++r) {
-      const int64_t ro = (int64_t)snext[r] * a.row_stride + col;
-      kreg[r] = ld16(a.kc + ro);
-      vreg[r] = ld16(a.vc + ro);
+      const int64_t ro = (int64_t)snext[r] * row_stride + col;
+      kreg[r] = ld16(kc + ro);
+      vreg[r] = ld16(vc + ro);
     }
   };
-  int tb = s0 + kTile * w;
+  int tb = wk.s0 + kTile * w;
   if (tb < s1) {
     fetch_slots(tb);
     fetch_rows();
@@ -134,8 +124,8 @@ __global__ __launch_bounds__(256, 1) void prefix_mfma_kernel(PrefixArgs a, int m
 #pragma unroll
   for (int nb = 0; nb < NQB; ++nb) {
     const int q = 32 * nb + ql;
-    const bool ok = q < nq;
-    const uint16_t* qp = a.q + (int64_t)(qbase + (ok ? q : 0)) * a.q_stride + head * kPD + 64 * h;
+    const bool ok = q < wk.nq;
+    const uint16_t* qp = wk.qrow0 + (int64_t)(ok ? q : 0) * wk.q_stride + 64 * h;
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
       u32x4 v = ld16(qp + 8 * s);
@@ -143,7 +133,6 @@ __global__ __launch_bounds__(256, 1) void prefix_mfma_kernel(PrefixArgs a, int m
       qop[nb][s] = v;
     }
   }
-
 
   for (; tb < s1; tb += 4 * kTile) {
     // registers -> LDS, both tiles row-major [token][dim] with XOR-swizzled 16-byte chunks
@@ -179,20 +168,22 @@ __global__ __launch_bounds__(256, 1) void prefix_mfma_kernel(PrefixArgs a, int m
     for (int nb = 0; nb < NQB; ++nb) {
       float x[16];
       float mloc = -INFINITY;
+      const int tmax = CAUSAL ? min(s1 - 1, wk.causal_off + 32 * nb + ql) : s1 - 1;  // last visible token
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int t = 8 * (r >> 2) + 4 * h + (r & 3);
-        x[r] = (tb + t < s1) ? sacc[nb][r] * a.scale_log2e : -INFINITY;
+        x[r] = (tb + t <= tmax) ? sacc[nb][r] * scale_log2e : -INFINITY;
         mloc = fmaxf(mloc, x[r]);
       }
       mloc = fmaxf(mloc, __shfl_xor(mloc, 32, kWave));
       const float mn = fmaxf(m[nb], mloc);
-      const float alpha = __builtin_amdgcn_exp2f(m[nb] - mn);
+      const float mref = (CAUSAL && mn == -INFINITY) ? 0.f : mn;  // a row with nothing visible yet
+      const float alpha = __builtin_amdgcn_exp2f(m[nb] - mref);
       m[nb] = mn;
       float ps = 0.f;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        x[r] = __builtin_amdgcn_exp2f(x[r] - mn);
+        x[r] = __builtin_amdgcn_exp2f(x[r] - mref);
         ps += x[r];
       }
       lsum[nb] = lsum[nb] * alpha + ps;
@@ -270,9 +261,53 @@ __global__ __launch_bounds__(256, 1) void prefix_mfma_kernel(PrefixArgs a, int m
   __syncthreads();
   if (w == 1) dump(smem);
   __syncthreads();
-  if (w != 0) return;
-  fold(smem);
+  if (w == 0) fold(smem);
+}
 
+template <int NQB>
+constexpr int tile_lds_bytes() {
+  return 4 * kWaveLds > 2 * (4 * NQB * 16 + 2 * NQB) * 256 ? 4 * kWaveLds : 2 * (4 * NQB * 16 + 2 * NQB) * 256;
+}
+
+// Shared-prefix phase: workgroup = (split, head, group x query tile); writes one (O, m, l) part.
+template <typename E, int NQB>
+__global__ __launch_bounds__(256, 1) void prefix_mfma_kernel(PrefixArgs a, int mtiles) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int split = blockIdx.x, head = blockIdx.y;
+  const int g = blockIdx.z / mtiles, mt = blockIdx.z - g * mtiles;
+  int r0 = 0, r1 = a.B, poff = 0, plen = a.fixed_prefix_len;
+  if (a.prefix_cu) {
+    r0 = a.group_req_cu[g];
+    r1 = a.group_req_cu[g + 1];
+    poff = a.prefix_cu[g];
+    plen = a.prefix_cu[g + 1] - poff;
+  }
+  const int qbase = r0 + mt * 32 * NQB;
+  const int nq = min(32 * NQB, r1 - qbase);
+  if (nq <= 0) return;
+  const int s0 = split * a.split_tokens;
+  const int s1 = min(plen, s0 + a.split_tokens);
+  if (s0 >= plen) {  // this group's prefix ends before the split: mark the part empty
+    for (int q = threadIdx.x; q < nq; q += 256) {
+      const int64_t pr = ((int64_t)split * a.B + qbase + q) * a.H + head;
+      a.ml[pr * 2] = -INFINITY;
+      a.ml[pr * 2 + 1] = 0.f;
+    }
+    return;
+  }
+  TileWork wk;
+  wk.qrow0 = a.q + (int64_t)qbase * a.q_stride + head * kPD;
+  wk.q_stride = a.q_stride;
+  wk.nq = nq;
+  wk.slots = a.slots + poff;
+  wk.s0 = s0;
+  wk.s1 = s1;
+  wk.causal_off = 0;
+  float16_t oacc[4][NQB];
+  float m[NQB], lsum[NQB];
+  attn_tile<E, NQB, false>(wk, a.kc, a.vc, a.row_stride, head, a.scale_log2e, smem, oacc, m, lsum);
+  if (threadIdx.x >= 64) return;
+  const int lane = threadIdx.x, h = lane >> 5, ql = lane & 31;
 #pragma unroll
   for (int nb = 0; nb < NQB; ++nb) {
     const float L = lsum[nb] + __shfl_xor(lsum[nb], 32, kWave);
@@ -297,24 +332,91 @@ __global__ __launch_bounds__(256, 1) void prefix_mfma_kernel(PrefixArgs a, int m
   }
 }
 
+// Prefill with parent context: workgroup = (head, 64-query tile of one chunk), all of the tile's
+// visible keys (ancestors, then the chunk's own tokens up to the diagonal); writes the final rows.
+// blockIdx.x is the head so that the query tiles of one (chunk, head), which stream the same K/V,
+// land on the same XCD (workgroups go round-robin over the 8 XCDs in linear order) and share its L2.
+template <typename E>
+__global__ __launch_bounds__(256, 1) void prefill_mfma_kernel(PrefillArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int head = blockIdx.x;
+  const int ti = blockIdx.y;
+  if (head >= a.H) return;
+  if (ti >= a.tile_cu[a.num_chunks]) return;
+  int lo = 0, hi = a.num_chunks;  // chunk with tile_cu[c] <= ti < tile_cu[c+1]
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (a.tile_cu[mid] <= ti) lo = mid; else hi = mid;
+  }
+  const int cq0 = a.q_cu[lo], n = a.q_cu[lo + 1] - cq0;
+  const int kv0 = a.kv_cu[lo], kvn = a.kv_cu[lo + 1] - kv0;
+  const int q0 = (ti - a.tile_cu[lo]) * 64;
+  const int nq = min(64, n - q0);
+  TileWork wk;
+  wk.qrow0 = a.q + (int64_t)(cq0 + q0) * a.q_stride + head * kPD;
+  wk.q_stride = a.q_stride;
+  wk.nq = nq;
+  wk.slots = a.ctx_slots + kv0;
+  wk.s0 = 0;
+  wk.causal_off = kvn - n + q0;
+  wk.s1 = min(kvn, wk.causal_off + nq);  // the last live query sees tokens up to causal_off + nq - 1
+  float16_t oacc[4][2];
+  float m[2], lsum[2];
+  attn_tile<E, 2, true>(wk, a.kc, a.vc, a.row_stride, head, a.scale_log2e, smem, oacc, m, lsum);
+  if (threadIdx.x >= 64) return;
+  const int lane = threadIdx.x, h = lane >> 5, ql = lane & 31;
+#pragma unroll
+  for (int nb = 0; nb < 2; ++nb) {
+    const float L = lsum[nb] + __shfl_xor(lsum[nb], 32, kWave);
+    const int q = 32 * nb + ql;
+    if (q < nq) {
+      const float inv = L > 0.f ? 1.f / L : 0.f;
+      uint16_t* op = a.out + (int64_t)(cq0 + q0 + q) * a.out_stride + head * kPD;
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          u32x2 v = {pack2<E>(oacc[db][nb][4 * j] * inv, oacc[db][nb][4 * j + 1] * inv),
+                     pack2<E>(oacc[db][nb][4 * j + 2] * inv, oacc[db][nb][4 * j + 3] * inv)};
+          *reinterpret_cast<u32x2*>(op + 32 * db + 8 * j + 4 * h) = v;
+        }
+    }
+  }
+}
+
+// tile_cu[c] = number of 64-query tiles before chunk c (serial scan; chunk counts are small)
+__global__ void prefill_tiles_kernel(const int32_t* q_cu, int num_chunks, int32_t* tile_cu) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  int acc = 0;
+  for (int c = 0; c < num_chunks; ++c) {
+    tile_cu[c] = acc;
+    acc += (q_cu[c + 1] - q_cu[c] + 63) / 64;
+  }
+  tile_cu[num_chunks] = acc;
+}
+
 template <typename E>
 static int launch_prefix_t(const PrefixArgs& a, int num_groups, int max_group_reqs, hipStream_t st) {
   const int nqb = max_group_reqs <= 32 ? 1 : 2;
   const int mtiles = (max_group_reqs + 32 * nqb - 1) / (32 * nqb);
   dim3 grid(a.n_splits, a.H, num_groups * mtiles), block(256);
   if (nqb == 1) {
-    constexpr int lds = 4 * kWaveLds > 2 * (4 * 1 * 16 + 2) * 256 ? 4 * kWaveLds : 2 * (4 * 1 * 16 + 2) * 256;
-    hipLaunchKernelGGL((prefix_mfma_kernel<E, 1>), grid, block, lds, st, a, mtiles);
+    hipLaunchKernelGGL((prefix_mfma_kernel<E, 1>), grid, block, tile_lds_bytes<1>(), st, a, mtiles);
   } else {
-    constexpr int lds = 4 * kWaveLds > 2 * (4 * 2 * 16 + 4) * 256 ? 4 * kWaveLds : 2 * (4 * 2 * 16 + 4) * 256;
-    static bool attr_set = false;
-    if (!attr_set) {
-      hipFuncSetAttribute(reinterpret_cast<const void*>(&prefix_mfma_kernel<E, 2>),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-      attr_set = true;
-    }
-    hipLaunchKernelGGL((prefix_mfma_kernel<E, 2>), grid, block, lds, st, a, mtiles);
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefix_mfma_kernel<E, 2>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, tile_lds_bytes<2>());
+    hipLaunchKernelGGL((prefix_mfma_kernel<E, 2>), grid, block, tile_lds_bytes<2>(), st, a, mtiles);
   }
+  return launch_status();
+}
+
+template <typename E>
+static int launch_prefill_t(const PrefillArgs& a, int max_tiles, hipStream_t st) {
+  hipLaunchKernelGGL(prefill_tiles_kernel, dim3(1), dim3(64), 0, st, a.q_cu, a.num_chunks, a.tile_cu);
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_mfma_kernel<E>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, tile_lds_bytes<2>());
+  const int hx = (a.H + 7) / 8 * 8;  // keeps head == linear id mod 8 for every tile row
+  hipLaunchKernelGGL((prefill_mfma_kernel<E>), dim3(hx, max_tiles), dim3(256), tile_lds_bytes<2>(), st, a);
   return launch_status();
 }
 
@@ -325,6 +427,12 @@ int launch_prefix_mfma(const PrefixArgs& a, int dtype, int D, int num_groups, in
   if (num_groups <= 0 || max_group_reqs <= 0 || a.n_splits <= 0) return PH_OK;
   return dtype == PH_F16 ? launch_prefix_t<F16>(a, num_groups, max_group_reqs, st)
                          : launch_prefix_t<BF16>(a, num_groups, max_group_reqs, st);
+}
+
+int launch_prefill_mfma(const PrefillArgs& a, int dtype, int D, int max_tiles, hipStream_t st) {
+  if (D != kPD) return PH_ERR_HEAD_DIM;
+  if (max_tiles <= 0) return PH_OK;
+  return dtype == PH_F16 ? launch_prefill_t<F16>(a, max_tiles, st) : launch_prefill_t<BF16>(a, max_tiles, st);
 }
 
 }  // namespace ph

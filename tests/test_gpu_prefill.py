@@ -56,3 +56,59 @@ def test_config4_scaled(dev):
     assert case.dtype == torch.bfloat16 and case.q.shape[1:] == (40, 128)
     out, ref = run_prefill_case(case, dev)
     torch.testing.assert_close(out.float(), ref.float(), **TOL[torch.bfloat16])
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_prefill_tile_boundaries(dev, dtype):
+    """Chunk lengths around the 64-query tile and 32-token KV tile sizes, with and without parents."""
+    from parrotserve_amd import synth
+
+    for parent, q_lens in ((0, [63, 64, 65, 1, 129]), (31, [64, 33]), (96, [2, 127, 128]), (1, [300])):
+        case = synth.make_prefill_case("b", 77 + parent, dtype, q_lens, parent, 3, 128, 1 << 12)
+        out, ref = run_prefill_case(case, dev)
+        torch.testing.assert_close(out.float(), ref.float(), **TOL[dtype])
+
+
+def test_config4_full_size_property(dev):
+    """Config 4 at full size (16 chunks U[64,1024] over 2048-token parents, 40x128, bf16, seed 3): a query
+    row of the prefill equals a decode request over exactly the keys it may see (q_len == 1 reduction),
+    checked on the GPU for 512 sampled rows, plus oracle parity on the first chunk."""
+    from parrotserve_amd import kernels, synth
+
+    case = synth.config4()
+    T, H, D = case.q.shape
+    assert len(case.q_lens) == 16 and H == 40 and case.dtype == torch.bfloat16
+    kc, vc = synth.pool_to_device(case.k_rows, case.v_rows, case.used_slots, case.pool_slots, dev)
+    cache = ref_cos_sin_cache(int(case.positions.max()) + 1, D, case.theta, case.dtype)
+    q, k, v = case.q.to(dev), case.k_new.to(dev), case.v_new.to(dev)
+    kernels.vllm_rotary_emb(case.positions.to(dev), q.view(T, -1), k.view(T, -1), cache.to(dev), D)
+    new_slots = torch.cat([case.used_slots[n] for n in case.new_lists]).to(torch.int32).to(dev)
+    kernels.vllm_reshape_and_cache(k, v, kc, vc, new_slots)
+    ctx = [case.used_slots[torch.cat([p, n])].tolist() for p, n in zip(case.parent_lists, case.new_lists)]
+    tables = kernels.PrefillTables.build(case.q_lens, ctx, dev)
+    out = kernels.prefill_attention(q, kc, vc, tables)
+
+    g = torch.Generator().manual_seed(0)
+    rows = torch.randperm(T, generator=g)[:512].sort().values.tolist()
+    starts = [0]
+    for n in case.q_lens:
+        starts.append(starts[-1] + n)
+    lists = []
+    for r in rows:
+        c = max(i for i in range(16) if starts[i] <= r)
+        n = case.q_lens[c]
+        vis = len(ctx[c]) - n + (r - starts[c]) + 1
+        lists.append(ctx[c][:vis])
+    dt = kernels.DecodeTables.build([], [], lists, dev)
+    ridx = torch.tensor(rows, device=dev)
+    dec = kernels.decode_attention(q[ridx].contiguous(), kc, vc, dt)
+    torch.testing.assert_close(out[ridx].float(), dec.float(), **TOL[torch.bfloat16])
+
+    # oracle parity on chunk 0 (its queries and keys only)
+    n0 = case.q_lens[0]
+    rq, rk = ref_rope_neox(case.positions[:n0], case.q[:n0].reshape(n0, -1), case.k_new[:n0].reshape(n0, -1), cache, D,
+                           elem_rounding=True)
+    k_all = torch.cat([case.k_rows[case.parent_lists[0]], rk.view(n0, H, D)])
+    v_all = torch.cat([case.v_rows[case.parent_lists[0]], case.v_new[:n0]])
+    ref0 = ref_prefill_with_parent(rq.view(n0, H, D), k_all, v_all, [n0], [torch.arange(k_all.shape[0])])
+    torch.testing.assert_close(out[:n0].cpu().float(), ref0.float(), **TOL[torch.bfloat16])
