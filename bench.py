@@ -87,6 +87,97 @@ def cpu_baseline(case, sample_reqs: int):
     }
 
 
+def _time_gpu(torch, fn, iters=20, warmup=3):
+    for _ in range(warmup):
+        fn()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ts = []
+    for _ in range(iters):
+        a.record()
+        fn()
+        b.record()
+        b.synchronize()
+        ts.append(a.elapsed_time(b) * 1e-3)
+    ts.sort()
+    return ts[len(ts) // 2]
+
+
+def extras(torch, dev):
+    """The other configurations' kernels, each against its own roofline (median launch time, torch events
+    on the launch stream).  Data is synthetic of the configured shapes; parity for these shapes is in tests/."""
+    from parrotserve_amd import kernels, synth
+
+    out = {}
+    H, D = 32, 128
+    # --- config 3: token move, 65,536 random rows of 8 KB inside a 4M-slot pool (one tensor) ---------------
+    pool = 1 << 22
+    kc = torch.empty((pool, H, D), dtype=torch.float16, device=dev)
+    kc.normal_()
+    src, dst = synth.config3_move()
+    src, dst = src.to(dev), dst.to(dev)
+    t = _time_gpu(torch, lambda: kernels.discontinuous_move_tokens(kc, kc, src, dst))
+    nbytes = 2 * src.numel() * H * D * 2
+    out["c3_token_move"] = {"rows": src.numel(), "row_bytes": H * D * 2, "us": t * 1e6, "GB/s": nbytes / t / 1e9,
+                            "frac_hbm": nbytes / t / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": nbytes}
+    # --- config 3: ragged non-shared decode, B 256, ctx log-uniform[128, 8192] ------------------------------
+    vc = torch.empty_like(kc)
+    vc.normal_()
+    case = synth.config3(batch=256, pool_slots=pool)
+    lens = [l.numel() for l in case.suffix_lists]
+    tabs = kernels.DecodeTables.build([], [], case.pool_lists(case.suffix_lists), dev)
+    q = case.q.to(dev)
+    o = torch.empty_like(q)
+    t = _time_gpu(torch, lambda: kernels.decode_attention(q, kc, vc, tabs, out=o), iters=10)
+    nbytes = 2 * sum(lens) * H * D * 2
+    out["c3_ragged_decode"] = {"batch": 256, "sum_ctx": sum(lens), "ms": t * 1e3, "GB/s": nbytes / t / 1e9,
+                               "frac_hbm": nbytes / t / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": nbytes,
+                               "tokens/s/layer": 256 / t}
+    del kc, vc, tabs
+    # --- config 4: RoPE + append + prefill with parent context, bf16 40x128 ---------------------------------
+    c4 = synth.config4()
+    T, H4, _ = c4.q.shape
+    kc4, vc4 = synth.pool_to_device(c4.k_rows, c4.v_rows, c4.used_slots, c4.pool_slots, dev)
+    cache = kernels_cos_sin(torch, int(c4.positions.max()) + 1, D, c4.theta, torch.bfloat16, dev)
+    qkv = torch.randn((T, 3 * H4 * D), device=dev, dtype=torch.bfloat16)
+    q4, k4, v4 = qkv.chunk(3, dim=-1)
+    pos = c4.positions.to(dev)
+    t_rope = _time_gpu(torch, lambda: kernels.vllm_rotary_emb(pos, q4, k4, cache, D))
+    rope_bytes = 2 * T * 2 * H4 * D * 2 + T * D * 2
+    new_slots = torch.cat([c4.used_slots[n] for n in c4.new_lists]).to(torch.int32).to(dev)
+    k3, v3 = k4.view(T, H4, D), v4.view(T, H4, D)
+    t_app = _time_gpu(torch, lambda: kernels.vllm_reshape_and_cache(k3, v3, kc4, vc4, new_slots))
+    ctx = [c4.used_slots[torch.cat([p, n])].tolist() for p, n in zip(c4.parent_lists, c4.new_lists)]
+    ptab = kernels.PrefillTables.build(c4.q_lens, ctx, dev)
+    qc = q4.reshape(T, H4, D).contiguous()
+    o4 = torch.empty_like(qc)
+    t_pre = _time_gpu(torch, lambda: kernels.prefill_attention(qc, kc4, vc4, ptab, out=o4), iters=10)
+    par = c4.parent_lists[0].numel()
+    flops = 4 * H4 * D * sum(n * par + n * (n + 1) // 2 for n in c4.q_lens)
+    out["c4_rope"] = {"tokens": T, "us": t_rope * 1e6, "GB/s": rope_bytes / t_rope / 1e9,
+                      "frac_hbm": rope_bytes / t_rope / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": rope_bytes}
+    app_bytes = 2 * 2 * T * H4 * D * 2
+    out["c4_kv_append"] = {"tokens": T, "us": t_app * 1e6, "GB/s": app_bytes / t_app / 1e9,
+                           "frac_hbm": app_bytes / t_app / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": app_bytes}
+    out["c4_prefill"] = {"tokens": T, "chunks": len(c4.q_lens), "ms": t_pre * 1e3, "flops": flops,
+                         "TFLOP/s": flops / t_pre / 1e12, "frac_mfma_peak": flops / t_pre / 1e12 / MFMA_F16_PEAK_TFLOPS,
+                         "tokens/s/layer": T / t_pre}
+    del kc4, vc4
+    # --- RMSNorm at a bandwidth-sized row count (LLaMA-13B hidden) -----------------------------------------
+    x = torch.randn((8192, 5120), device=dev, dtype=torch.float16)
+    w = torch.ones(5120, device=dev, dtype=torch.float16)
+    t = _time_gpu(torch, lambda: kernels.vllm_rms_norm(x, w, 1e-6))
+    nbytes = 2 * x.numel() * 2 + 5120 * 2
+    out["rms_norm_8192x5120"] = {"us": t * 1e6, "GB/s": nbytes / t / 1e9, "frac_hbm": nbytes / t / 1e9 / HBM_PEAK_GBS,
+                                 "algorithmic_bytes": nbytes}
+    return out
+
+
+def kernels_cos_sin(torch, n, d, theta, dtype, dev):
+    from parrotserve_amd.mem import make_cos_sin_cache
+
+    return make_cos_sin_cache(n, d, theta, dtype, dev)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -95,6 +186,7 @@ def main():
     ap.add_argument("--layers", type=int, default=8, help="distinct KV sets the steps rotate over")
     ap.add_argument("--cpu-sample", type=int, default=16)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-extras", action="store_true", help="skip the other configurations' kernel rooflines")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs the hot path on ONE GPU; --gpus must be 1 "
@@ -213,6 +305,10 @@ def main():
         "merge_us": t_merge * 1e6,
         "warm_single_kv_set": {"value": B / t_warm, "ms_per_step": t_warm * 1e3},
     }
+    if not args.no_extras:
+        del kc, vc, tables, qs
+        torch.cuda.empty_cache()
+        result["extras"] = extras(torch, dev)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(case, min(args.cpu_sample, B))
     print(json.dumps(result))

@@ -269,6 +269,11 @@ static int launch_partial_t(const PartialArgs& a, hipStream_t st) {
   if (waves == 0) return PH_OK;
   dim3 grid((unsigned)((waves + 3) / 4)), block(256);
   static const int variant = getenv("PH_DECODE_VARIANT") ? atoi(getenv("PH_DECODE_VARIANT")) : 0;
+  static const int lds_cap = getenv("PH_DECODE_LDS") ? atoi(getenv("PH_DECODE_LDS")) : 0;
+  if (lds_cap) {
+    hipLaunchKernelGGL((decode_partial_kernel<E, D, 4, 2>), grid, block, lds_cap, st, a);
+    return launch_status();
+  }
   switch (variant) {
     case 1: hipLaunchKernelGGL((decode_partial_kernel<E, D, 4, 1>), grid, block, 0, st, a); break;
     case 5: hipLaunchKernelGGL((decode_partial_kernel<E, D, 4, 1, 1>), grid, block, 0, st, a); break;
