@@ -150,11 +150,33 @@ int ph_rotary_embedding(void* state, const void* cos, const void* sin,
  *                 length and clamps those reads to this bound);
  *   suffix_lens:  int32 [B] (DEVICE); max_suffix_len: host upper bound.
  * chunk_tokens: suffix split size (multiple of 16), 0 = choose.
- * workspace: at least ph_decode_workspace_bytes(...) bytes, 256-byte aligned.
+ * plan (HOST struct of DEVICE pointers, may be NULL): a caller that knows the
+ *   suffix lengths on the host (the reference builds them from Python lists,
+ *   attn_func.py:523-531) cuts the batch's suffix token stream into num_lanes
+ *   near-equal pieces; a piece is one or more items (request, first token,
+ *   token count).  The suffix phase then runs one wave set per piece, every wave
+ *   moving the same number of bytes, instead of one per fixed-size chunk.
+ *   items:        int32 [num_items][4] = request, first token, count, 0, in
+ *                 request order (a request's items are consecutive, its tokens
+ *                 ascending and covered exactly once);
+ *   lane_rec:     int32 [num_lanes][8], piece j = (first item, item count,
+ *                 then a copy of its first item's request, first token, count,
+ *                 0, 0, 0) -- one record read starts a piece;
+ *   req_item_cu:  int32 [B+1], request b owns items [cu[b], cu[b+1]).
+ * workspace: at least ph_decode_workspace_bytes(...) bytes, 256-byte aligned
+ *   (num_items = plan->num_items, or 0 without a plan).
  */
+typedef struct {
+  const int32_t* items;
+  int64_t num_items;
+  const int32_t* lane_rec;
+  int64_t num_lanes;
+  const int32_t* req_item_cu;
+} ph_suffix_plan;
+
 size_t ph_decode_workspace_bytes(int64_t num_reqs, int64_t num_heads, int64_t head_dim,
                                  int64_t num_groups, int64_t max_prefix_len,
-                                 int64_t max_suffix_len, int64_t chunk_tokens);
+                                 int64_t max_suffix_len, int64_t chunk_tokens, int64_t num_items);
 
 int ph_decode_attention(void* out, const void* q, const void* k_cache, const void* v_cache,
                         int64_t num_reqs, int64_t num_heads, int64_t head_dim, int dtype,
@@ -167,6 +189,7 @@ int ph_decode_attention(void* out, const void* q, const void* k_cache, const voi
                         int64_t suffix_table_stride, int64_t suffix_slots_count,
                         const int32_t* suffix_lens,
                         int64_t max_suffix_len, int64_t chunk_tokens,
+                        const ph_suffix_plan* plan,
                         void* workspace, size_t workspace_bytes, void* stream);
 
 /* The two halves of the shared-prefix op, exposed separately because the

@@ -29,14 +29,23 @@ SIGNATURES: Dict[str, Tuple[object, List[object]]] = {
     "ph_rms_norm": (I, [P, P, P, F, L, L, L, L, I, I, P]),
     "ph_rope_neox": (I, [P, P, P, P, L, L, L, L, L, L, L, I, P]),
     "ph_rotary_embedding": (I, [P, P, P, L, L, L, L, L, L, I, P]),
-    "ph_decode_workspace_bytes": (Z, [L, L, L, L, L, L, L]),
-    "ph_decode_attention": (I, [P, P, P, P, L, L, L, I, L, L, L, F, L, P, P, P, P, L, P, P, L, L, P, L, L, P, Z, P]),
+    "ph_decode_workspace_bytes": (Z, [L, L, L, L, L, L, L, L]),
+    "ph_decode_attention": (I, [P, P, P, P, L, L, L, I, L, L, L, F, L, P, P, P, P, L, P, P, L, L, P, L, L, P, P, Z, P]),
     "ph_prefix_attention": (I, [P, P, P, P, P, P, L, L, L, I, L, L, L, F, P, L, P, Z, P]),
     "ph_suffix_post_attention": (I, [P, P, P, P, P, P, L, L, L, I, L, L, L, F, P, P, L, L, P, L, L, P, Z, P]),
     "ph_arm_phase_events": (I, [P]),
     "ph_prefill_workspace_bytes": (Z, [L, L, L, L]),
     "ph_prefill_attention": (I, [P, P, P, P, L, L, L, L, I, L, L, L, F, P, P, P, L, L, P, Z, P]),
 }
+
+
+
+class SuffixPlan(ctypes.Structure):
+    """ph_suffix_plan: host struct of device pointers."""
+
+    _fields_ = [("items", c_void_p), ("num_items", c_int64), ("lane_rec", c_void_p), ("num_lanes", c_int64),
+                ("req_item_cu", c_void_p)]
+
 
 _lib = None
 

@@ -189,7 +189,7 @@ class HipSharedPrefixAttn(AttnFunc):
             order.extend(i for i in range(tabs.num_generates) if i not in grouped)
             suffix = [tabs.paged_block_tables[i] for i in order]
             st.decode_tables = kernels.DecodeTables.build([p for p, _ in tabs.groups], gcu if tabs.groups else [],
-                                                          suffix, device)
+                                                          suffix, device, num_heads=num_heads, head_dim=head_size)
             if order != list(range(tabs.num_generates)):
                 perm = torch.tensor(order, dtype=torch.int64, device=device)
                 inv = torch.empty_like(perm)

@@ -6,11 +6,14 @@
 namespace ph {
 
 struct DecodePlan {
-  int chunk;         // suffix tokens per part
-  int n_chunks;      // suffix parts per request
+  int chunk;         // suffix tokens per part (grid form)
+  int n_chunks;      // suffix parts per request (grid form)
   int split_tokens;  // prefix tokens per part
   int n_splits;      // prefix parts
+  int64_t items;     // suffix items (balanced form), 0 in the grid form
   int parts() const { return n_chunks + n_splits; }
+  // partial rows (one row = one head's (O, m, l)): [parts][B][H] then [items][H]
+  size_t rows(int64_t B, int64_t H) const { return (size_t)parts() * B * H + (size_t)items * H; }
 };
 
 static int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
@@ -20,9 +23,13 @@ constexpr int kPrefixTile = 64;        // tokens per LDS tile of the MFMA kernel
 constexpr int kPrefixQueryTile = 64;   // queries per workgroup of the MFMA kernel
 
 static DecodePlan plan_decode(int64_t B, int64_t H, int64_t groups, int64_t max_prefix, int64_t max_suffix,
-                              int64_t chunk_tokens) {
+                              int64_t chunk_tokens, int64_t num_items = 0) {
   DecodePlan p{};
-  if (max_suffix > 0) {
+  p.items = num_items;
+  if (num_items > 0) {
+    p.chunk = 32;
+    p.n_chunks = 0;
+  } else if (max_suffix > 0) {
     int64_t chunk = chunk_tokens;
     if (chunk <= 0) {
       // Aim for about 2048 (request, chunk) items assuming mean length = max/2.
@@ -61,7 +68,7 @@ static DecodePlan plan_decode(int64_t B, int64_t H, int64_t groups, int64_t max_
 }
 
 static size_t plan_bytes(const DecodePlan& p, int64_t B, int64_t H, int64_t D) {
-  const size_t rows = (size_t)p.parts() * B * H;
+  const size_t rows = p.rows(B, H);
   return round_up((int64_t)(rows * D * sizeof(float)), 256) + round_up((int64_t)(rows * 2 * sizeof(float)), 256);
 }
 
@@ -70,7 +77,7 @@ struct Carve {
   float* ml;
 };
 static Carve carve(void* ws, const DecodePlan& p, int64_t B, int64_t H, int64_t D) {
-  const size_t rows = (size_t)p.parts() * B * H;
+  const size_t rows = p.rows(B, H);
   Carve c;
   c.opart = (float*)ws;
   c.ml = (float*)((char*)ws + round_up((int64_t)(rows * D * sizeof(float)), 256));
@@ -175,9 +182,10 @@ static inline void phase_mark(bool armed, int i, hipStream_t st) {
 
 extern "C" size_t ph_decode_workspace_bytes(int64_t num_reqs, int64_t num_heads, int64_t head_dim,
                                             int64_t num_groups, int64_t max_prefix_len, int64_t max_suffix_len,
-                                            int64_t chunk_tokens) {
+                                            int64_t chunk_tokens, int64_t num_items) {
   if (num_reqs <= 0 || num_heads <= 0 || head_dim <= 0) return 0;
-  const DecodePlan p = plan_decode(num_reqs, num_heads, num_groups, max_prefix_len, max_suffix_len, chunk_tokens);
+  const DecodePlan p =
+      plan_decode(num_reqs, num_heads, num_groups, max_prefix_len, max_suffix_len, chunk_tokens, num_items);
   return plan_bytes(p, num_reqs, num_heads, head_dim);
 }
 
@@ -188,8 +196,9 @@ extern "C" int ph_decode_attention(void* out, const void* q, const void* k_cache
                                    const int32_t* group_req_cu, const int32_t* group_req_cu_host,
                                    int64_t max_prefix_len, const int32_t* suffix_slots,
                                    const int64_t* suffix_offsets, int64_t suffix_table_stride,
-                                   int64_t suffix_slots_count, const int32_t* suffix_lens, int64_t max_suffix_len, int64_t chunk_tokens,
-                                   void* workspace, size_t workspace_bytes, void* stream) {
+                                   int64_t suffix_slots_count, const int32_t* suffix_lens, int64_t max_suffix_len,
+                                   int64_t chunk_tokens, const ph_suffix_plan* plan, void* workspace,
+                                   size_t workspace_bytes, void* stream) {
   const int B = (int)num_reqs, H = (int)num_heads, D = (int)head_dim;
   int rc = check_common(out, q, k_cache, v_cache, num_reqs, num_heads, head_dim, dtype, q_stride, out_stride,
                         cache_stride_n);
@@ -199,8 +208,12 @@ extern "C" int ph_decode_attention(void* out, const void* q, const void* k_cache
   const bool has_suffix = max_suffix_len > 0;
   if (has_prefix && (!prefix_slots || !prefix_cu || !group_req_cu || !group_req_cu_host)) return PH_ERR_ARG;
   if (has_suffix && (!suffix_slots || !suffix_lens || suffix_slots_count <= 0)) return PH_ERR_ARG;
-  const DecodePlan p =
-      plan_decode(num_reqs, num_heads, has_prefix ? num_groups : 0, max_prefix_len, max_suffix_len, chunk_tokens);
+  const bool planned = has_suffix && plan != nullptr && plan->num_items > 0;
+  if (planned && (!plan->items || !plan->lane_rec || !plan->req_item_cu || plan->num_lanes <= 0 ||
+                  plan->num_items > (int64_t)1 << 30))
+    return PH_ERR_ARG;
+  const DecodePlan p = plan_decode(num_reqs, num_heads, has_prefix ? num_groups : 0, max_prefix_len, max_suffix_len,
+                                   chunk_tokens, planned ? plan->num_items : 0);
   if (plan_bytes(p, B, H, D) > workspace_bytes || (p.parts() > 0 && !workspace)) return PH_ERR_WORKSPACE;
   if (((uintptr_t)workspace & 255u) != 0) return PH_ERR_ALIGN;
   const Carve ws = carve(workspace, p, B, H, D);
@@ -243,7 +256,27 @@ extern "C" int ph_decode_attention(void* out, const void* q, const void* k_cache
     if (rc != PH_OK) return rc;
   }
   phase_mark(armed, 1, st);
-  if (has_suffix) {
+  const int64_t item_base = (int64_t)p.n_splits * B * H;  // first partial row of the balanced form's items
+  if (planned) {
+    ItemArgs ia{};
+    ia.q = (const uint16_t*)q;
+    ia.q_stride = q_stride;
+    ia.kc = (const uint16_t*)k_cache;
+    ia.vc = (const uint16_t*)v_cache;
+    ia.row_stride = cache_stride_n;
+    ia.slots = suffix_slots;
+    ia.offsets = suffix_offsets;
+    ia.table_stride = suffix_table_stride;
+    ia.items = reinterpret_cast<const int4*>(plan->items);
+    ia.lane_rec = reinterpret_cast<const int4*>(plan->lane_rec);
+    ia.num_lanes = (int)plan->num_lanes;
+    ia.opart = ws.opart + item_base * D;
+    ia.ml = ws.ml + item_base * 2;
+    ia.H = H;
+    ia.scale_log2e = sl2;
+    rc = launch_items(ia, dtype, D, st);
+    if (rc != PH_OK) return rc;
+  } else if (has_suffix) {
     PartialArgs sa{};
     sa.q = (const uint16_t*)q;
     sa.q_stride = q_stride;
@@ -281,6 +314,8 @@ extern "C" int ph_decode_attention(void* out, const void* q, const void* k_cache
   ma.baseB = p.n_splits;
   ma.lens = has_suffix ? suffix_lens : nullptr;
   ma.chunk = p.chunk;
+  ma.req_item_cu = planned ? plan->req_item_cu : nullptr;
+  ma.item_base = item_base;
   phase_mark(armed, 2, st);
   rc = launch_merge(ma, dtype, D, st);
   phase_mark(armed, 3, st);

@@ -31,6 +31,25 @@ struct PartialArgs {
   float scale_log2e;
 };
 
+// Balanced (host-planned) suffix phase; partial rows are [item][H].
+struct ItemArgs {
+  const uint16_t* q;
+  int64_t q_stride;
+  const uint16_t* kc;
+  const uint16_t* vc;
+  int64_t row_stride;
+  const int32_t* slots;
+  const int64_t* offsets;      // per-request start inside `slots`, or null
+  int64_t table_stride;
+  const int4* items;           // (request, first token, token count, 0)
+  const int4* lane_rec;        // [num_lanes][2]: (first item, item count, request, first token), (count, 0, 0, 0)
+  int num_lanes;
+  float* opart;                // already offset to the items' first row
+  float* ml;
+  int H;
+  float scale_log2e;
+};
+
 struct MergeArgs {
   const float* opart;
   const float* ml;
@@ -41,6 +60,8 @@ struct MergeArgs {
   int baseB;                // parts [baseB, baseB + ceil(lens[b]/chunk)) likewise
   const int32_t* lens;      // may be null (no B range)
   int chunk;
+  const int32_t* req_item_cu; // balanced form: request b owns items [cu[b], cu[b+1]) ...
+  int64_t item_base;          // ... whose partial rows start at item_base (rows of H)
   const float* prev_m;      // optional partial already in out/prev_m/prev_l
   const float* prev_l;
   float* m_out;             // optional export of the merged m / l
@@ -85,6 +106,7 @@ struct PrefillArgs {
 int launch_partial(const PartialArgs& a, int dtype, int D, hipStream_t st);
 // MFMA prefill: grid (head, query tile); max_tiles bounds the tile count (sum of ceil(n_c / 64)).
 int launch_prefill_mfma(const PrefillArgs& a, int dtype, int D, int max_tiles, hipStream_t st);
+int launch_items(const ItemArgs& a, int dtype, int D, hipStream_t st);
 int launch_merge(const MergeArgs& a, int dtype, int D, hipStream_t st);
 int launch_clear_ml(float* ml, int64_t entries, hipStream_t st);
 // MFMA shared-prefix kernel: grid (split, head, group x m-tile).

@@ -12,6 +12,7 @@ is no PyTorch fallback.
 """
 from __future__ import annotations
 
+import ctypes
 import dataclasses
 from typing import Dict, List, Optional, Sequence, Tuple
 
@@ -255,6 +256,11 @@ class DecodeTables:
     suffix_lens: Optional[torch.Tensor] = None  # [B] device
     max_suffix_len: int = 0
     chunk_tokens: int = 0  # 0 = let the library choose
+    # balanced suffix plan (needs the lengths on the host): device int32 arrays + the host struct
+    plan_items: Optional[torch.Tensor] = None  # [num_items, 4]
+    plan_lane_item_cu: Optional[torch.Tensor] = None  # lane records [num_lanes, 8]
+    plan_req_item_cu: Optional[torch.Tensor] = None  # [B + 1]
+    plan: Optional[_lib.SuffixPlan] = None
 
     def suffix_slots_count(self) -> int:
         """Entries readable behind ``suffix_slots`` (bound for the kernel's early slot fetch)."""
@@ -264,12 +270,31 @@ class DecodeTables:
             return (self.num_reqs - 1) * self.suffix_table_stride + self.suffix_slots.shape[-1]
         return self.suffix_slots.numel()
 
+    def set_plan(self, lens: Sequence[int], num_lanes: int, device) -> None:
+        """Cut the batch's suffix token stream into ``num_lanes`` near-equal pieces (see ph_suffix_plan)."""
+        items, lane_cu, req_cu = plan_suffix_items(lens, num_lanes)
+        if items.shape[0] == 0:
+            return
+        lanes = lane_cu.shape[0] - 1
+        rec = np.zeros((lanes, 8), dtype=np.int32)
+        rec[:, 0] = lane_cu[:-1]
+        rec[:, 1] = lane_cu[1:] - lane_cu[:-1]
+        first = np.minimum(lane_cu[:-1], items.shape[0] - 1)
+        rec[:, 2:5] = items[first, 0:3]
+        self.plan_items = torch.from_numpy(items).to(device)
+        self.plan_lane_item_cu = torch.from_numpy(rec).to(device)
+        self.plan_req_item_cu = torch.from_numpy(req_cu).to(device)
+        self.plan = _lib.SuffixPlan(self.plan_items.data_ptr(), items.shape[0], self.plan_lane_item_cu.data_ptr(),
+                                    lane_cu.shape[0] - 1, self.plan_req_item_cu.data_ptr())
+
     @staticmethod
     def build(prefix_lists: Sequence[Sequence[int]], group_req_cu: Sequence[int],
-              suffix_lists: Sequence[Sequence[int]], device) -> "DecodeTables":
+              suffix_lists: Sequence[Sequence[int]], device, num_heads: int = 32, head_dim: int = 128,
+              balanced: bool = True) -> "DecodeTables":
         """From python lists: ``prefix_lists[g]`` is group g's slot list shared by
         requests ``group_req_cu[g] .. group_req_cu[g+1]-1``; ``suffix_lists[b]`` is
-        request b's own slot list."""
+        request b's own slot list.  ``balanced`` adds the host-planned item list of the
+        suffix phase, sized for ``num_heads x head_dim``."""
         B = len(suffix_lists)
         t = DecodeTables(num_reqs=B)
         G = len(prefix_lists)
@@ -305,7 +330,48 @@ class DecodeTables:
             while chunk < total // 2048 and chunk < 1024:
                 chunk *= 2
             t.chunk_tokens = chunk
+            if balanced:
+                t.set_plan(lens, suffix_lanes(device, num_heads, head_dim, total), device)
         return t
+
+
+def suffix_lanes(device, num_heads: int, head_dim: int, total_tokens: int) -> int:
+    """Pieces of the balanced suffix phase: one launch-wide round of waves at three waves per SIMD
+    (a piece is streamed by one wave per 64/(head_dim/8) heads), and no piece under 16 tokens."""
+    heads_per_wave = max(1, 64 // max(1, head_dim // 8))
+    hgroups = (num_heads + heads_per_wave - 1) // heads_per_wave
+    cus = 256
+    if torch.cuda.is_available() and str(device) != "cpu":
+        cus = torch.cuda.get_device_properties(device).multi_processor_count
+    lanes = max(1, cus * 4 * 3 // hgroups)
+    return max(1, min(lanes, (total_tokens + 15) // 16))
+
+
+def plan_suffix_items(lens: Sequence[int], num_lanes: int):
+    """(items [n, 4] int32, lane_item_cu [lanes+1] int32, req_item_cu [B+1] int32): the token stream of
+    all requests back to back is cut at the request boundaries and at ``num_lanes`` near-equal marks."""
+    lens_a = np.asarray(lens, dtype=np.int64)
+    B = lens_a.shape[0]
+    cu = np.zeros(B + 1, dtype=np.int64)
+    np.cumsum(lens_a, out=cu[1:])
+    total = int(cu[-1])
+    if total == 0:
+        return np.zeros((0, 4), np.int32), np.zeros(1, np.int32), np.zeros(B + 1, np.int32)
+    num_lanes = max(1, min(num_lanes, total))
+    cuts = (np.arange(num_lanes + 1, dtype=np.int64) * total) // num_lanes
+    pts = np.unique(np.concatenate([cu, cuts]))
+    a, b = pts[:-1], pts[1:]
+    req = np.searchsorted(cu, a, side="right") - 1
+    lane = np.searchsorted(cuts, a, side="right") - 1
+    items = np.zeros((a.shape[0], 4), dtype=np.int32)
+    items[:, 0] = req
+    items[:, 1] = a - cu[req]
+    items[:, 2] = b - a
+    lane_cu = np.zeros(num_lanes + 1, dtype=np.int32)
+    np.cumsum(np.bincount(lane, minlength=num_lanes), out=lane_cu[1:])
+    req_cu = np.zeros(B + 1, dtype=np.int32)
+    np.cumsum(np.bincount(req, minlength=B), out=req_cu[1:])
+    return items, lane_cu, req_cu
 
 
 @torch.inference_mode()
@@ -327,8 +393,9 @@ def decode_attention(query: torch.Tensor, key_cache: torch.Tensor, value_cache: 
         return out
     scale = D ** -0.5 if scale is None else scale
     lib = _lib.load()
+    plan = tables.plan
     nbytes = lib.ph_decode_workspace_bytes(B, H, D, tables.num_groups, tables.max_prefix_len, tables.max_suffix_len,
-                                           tables.chunk_tokens)
+                                           tables.chunk_tokens, 0 if plan is None else plan.num_items)
     ws = _workspace(nbytes, query.device)
     rc = lib.ph_decode_attention(
         _ptr(out), _ptr(query), _ptr(key_cache), _ptr(value_cache), B, H, D, _dtype_code(query),
@@ -337,7 +404,8 @@ def decode_attention(query: torch.Tensor, key_cache: torch.Tensor, value_cache: 
         _ptr(tables.group_req_cu_host), tables.max_prefix_len,
         _ptr(tables.suffix_slots), _ptr(tables.suffix_offsets), tables.suffix_table_stride,
         tables.suffix_slots_count(), _ptr(tables.suffix_lens),
-        tables.max_suffix_len, tables.chunk_tokens, _ptr(ws), ws.numel(), _stream())
+        tables.max_suffix_len, tables.chunk_tokens, None if plan is None else ctypes.byref(plan),
+        _ptr(ws), ws.numel(), _stream())
     check(rc, "decode_attention")
     return out
 

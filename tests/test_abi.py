@@ -43,9 +43,10 @@ def test_workspace_queries_are_host_only():
 
     lib = _lib.load()
     # C2 shape: B 64, H 32, D 128, one group, prefix 4096, suffix <= 512
-    n = lib.ph_decode_workspace_bytes(64, 32, 128, 1, 4096, 512, 32)
+    n = lib.ph_decode_workspace_bytes(64, 32, 128, 1, 4096, 512, 32, 0)
     assert n > 0 and n % 256 == 0
-    assert lib.ph_decode_workspace_bytes(0, 32, 128, 1, 4096, 512, 32) == 0
+    assert lib.ph_decode_workspace_bytes(0, 32, 128, 1, 4096, 512, 32, 0) == 0
+    assert lib.ph_decode_workspace_bytes(64, 32, 128, 1, 4096, 512, 0, 448) < n  # balanced form: fewer partial rows
     assert lib.ph_prefill_workspace_bytes(1000, 40, 128, 3000) > 0
 
 
@@ -60,7 +61,7 @@ def test_argument_validation_needs_no_gpu():
     assert lib.ph_rms_norm(None, None, None, 1e-6, 4, 64, 64, 64, 7, 1, None) == _lib.PH_ERR_DTYPE
     # unsupported head size mirrors the reference's "Unsupported head size" check
     rc = lib.ph_decode_attention(1, 1, 1, 1, 4, 2, 80, 0, 160, 160, 160, 1.0, 0, None, None, None, None, 0,
-                                 None, None, 0, 0, None, 0, 0, None, 0, None)
+                                 None, None, 0, 0, None, 0, 0, None, None, 0, None)
     assert rc == _lib.PH_ERR_HEAD_DIM
 
 

@@ -194,3 +194,25 @@ def test_unsupported_inputs_raise(dev):
     q32 = torch.zeros(2, 2, 128, dtype=torch.float32, device=dev)
     with pytest.raises(RuntimeError, match="data type"):
         kernels.decode_attention(q32, q32.new_zeros(8, 2, 128), q32.new_zeros(8, 2, 128), t)
+
+
+def test_balanced_and_grid_suffix_forms_agree(dev):
+    """The host-planned balanced suffix phase and the grid-of-chunks form give the same result (and both
+    match the oracle) on ragged lengths including empty and one-token suffixes."""
+    from parrotserve_amd import kernels, synth
+
+    g = torch.Generator().manual_seed(21)
+    s = [0, 1, 2, 700, 33, 64, 65, 0, 511, 5] + torch.randint(1, 300, (40,), generator=g).tolist()
+    case = synth.make_decode_case("bg", 21, torch.float16, 1, len(s), 300, s, 8, 128, 1 << 14)
+    kc, vc = synth.pool_to_device(case.k_rows, case.v_rows, case.used_slots, case.pool_slots, dev)
+    pre, suf = case.pool_lists(case.prefix_lists), case.pool_lists(case.suffix_lists)
+    ta = kernels.DecodeTables.build(pre, case.group_req_cu, suf, dev, num_heads=8, balanced=True)
+    tb = kernels.DecodeTables.build(pre, case.group_req_cu, suf, dev, num_heads=8, balanced=False)
+    assert ta.plan is not None and tb.plan is None
+    q = case.q.to(dev)
+    a = kernels.decode_attention(q, kc, vc, ta).cpu()
+    b = kernels.decode_attention(q, kc, vc, tb).cpu()
+    ref = ref_decode_attention(case.q, case.k_rows, case.v_rows, case.full_lists())
+    torch.testing.assert_close(a.float(), ref.float(), **TOL[torch.float16])
+    torch.testing.assert_close(b.float(), ref.float(), **TOL[torch.float16])
+    torch.testing.assert_close(a.float(), b.float(), atol=1e-3, rtol=1e-2)

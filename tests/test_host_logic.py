@@ -177,3 +177,32 @@ def test_selector_and_config():
         BuiltinConfig(num_kv_cache_blocks=16, block_size=16)
     with pytest.raises(ValueError):
         BlockContext(0, None, RecyclePool(), block_size=16)
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_suffix_plan_covers_every_token_once_and_balances(seed):
+    import numpy as np
+
+    from parrotserve_amd.kernels import plan_suffix_items
+
+    rng = random.Random(seed)
+    lens = [rng.choice([0, 1, 3, 17, 64, 500, 2000]) for _ in range(rng.randrange(1, 60))]
+    lanes = rng.choice([1, 7, 64, 384])
+    items, lane_cu, req_cu = plan_suffix_items(lens, lanes)
+    total = sum(lens)
+    if total == 0:
+        assert items.shape[0] == 0
+        return
+    # every request's tokens are covered exactly once, in order, by consecutive items
+    for b, n in enumerate(lens):
+        mine = items[req_cu[b] : req_cu[b + 1]]
+        assert (mine[:, 0] == b).all()
+        pos = 0
+        for _, t0, cnt, _z in mine.tolist():
+            assert t0 == pos and cnt > 0
+            pos += cnt
+        assert pos == n
+    assert req_cu[-1] == items.shape[0] == lane_cu[-1]
+    # pieces differ by at most one token
+    per_lane = [int(items[lane_cu[j] : lane_cu[j + 1], 2].sum()) for j in range(len(lane_cu) - 1)]
+    assert sum(per_lane) == total and max(per_lane) - min(per_lane) <= 1
