@@ -49,19 +49,26 @@ struct Elem<BF16> {
   static __device__ __forceinline__ float hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
   static __device__ __forceinline__ float one(uint16_t b) { return __builtin_bit_cast(float, (uint32_t)b << 16); }
   static __device__ __forceinline__ uint16_t bits(float f) {  // round to nearest even
-    uint32_t u = __builtin_bit_cast(uint32_t, f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);  // quiet NaN
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (uint16_t)(u >> 16);
+    return __builtin_bit_cast(uint16_t, (__bf16)f);
   }
   static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float acc) {
     return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), acc, false);
   }
 };
 
+// Two floats -> one packed pair of elements, round to nearest even (v_cvt_pk_{f16,bf16}_f32).
 template <typename E>
-__device__ __forceinline__ uint32_t pack2(float a, float b) {
-  return (uint32_t)Elem<E>::bits(a) | ((uint32_t)Elem<E>::bits(b) << 16);
+__device__ __forceinline__ uint32_t pack2(float a, float b);
+template <>
+__device__ __forceinline__ uint32_t pack2<F16>(float a, float b) {
+  typedef float float2_t __attribute__((ext_vector_type(2)));
+  const float2_t f = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, half2_t));
+}
+template <>
+__device__ __forceinline__ uint32_t pack2<BF16>(float a, float b) {
+  const bf16x2_t v = {(__bf16)a, (__bf16)b};
+  return __builtin_bit_cast(uint32_t, v);
 }
 
 // Round a float to the element type and back (the "t(.)" of the reference's

@@ -70,13 +70,16 @@ struct TileWork {
   int causal_off;         // CAUSAL: query i sees token t iff t <= causal_off + i
 };
 
-// Runs the tile on all four waves; on return wave 0 holds the folded (unnormalised) accumulators,
-// the running maxima and per-lane partial sums of the softmax denominators.
+// Runs the tile on all four waves.  On return wave w holds, for the 32 dims [32w, 32w+32) of every
+// query, the accumulators folded over the four waves (unnormalised, C layout: register 4j+i = dim
+// 32w + 8j + 4h + i of query 32nb + ql), plus each query's final maximum and softmax denominator.
 template <typename E, int NQB, bool CAUSAL>
 __device__ __forceinline__ void attn_tile(const TileWork& wk, const uint16_t* __restrict__ kc,
                                           const uint16_t* __restrict__ vc, int64_t row_stride, int head,
-                                          float scale_log2e, char* smem, float16_t (&oacc)[4][NQB], float (&m)[NQB],
-                                          float (&lsum)[NQB]) {
+                                          float scale_log2e, char* smem, float16_t (&ofold)[NQB], float (&mfin)[NQB],
+                                          float (&lfin)[NQB]) {
+  float16_t oacc[4][NQB];
+  float m[NQB], lsum[NQB];
   const int lane = threadIdx.x & 63;
   const int w = threadIdx.x >> 6;
   const int h = lane >> 5, ql = lane & 31;
@@ -162,28 +165,36 @@ __device__ __forceinline__ void attn_tile(const TileWork& wk, const uint16_t* __
       for (int nb = 0; nb < NQB; ++nb) sacc[nb] = Mfma32<E>::run(ka, qop[nb][s], sacc[nb]);
     }
 
-    // online softmax; P^T packed straight into B-operand form
+    // online softmax in the exp2 domain (scores are scaled inside the exponent's fma); P^T is packed
+    // straight into B-operand form.  Only a split's last tile and causal tiles need token masks.
     u32x4 pop[NQB][2];
+    const bool full = !CAUSAL && tb + kTile <= s1;
 #pragma unroll
     for (int nb = 0; nb < NQB; ++nb) {
       float x[16];
-      float mloc = -INFINITY;
-      const int tmax = CAUSAL ? min(s1 - 1, wk.causal_off + 32 * nb + ql) : s1 - 1;  // last visible token
+      if (full) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int t = 8 * (r >> 2) + 4 * h + (r & 3);
-        x[r] = (tb + t <= tmax) ? sacc[nb][r] * scale_log2e : -INFINITY;
-        mloc = fmaxf(mloc, x[r]);
+        for (int r = 0; r < 16; ++r) x[r] = sacc[nb][r];
+      } else {
+        const int tmax = CAUSAL ? min(s1 - 1, wk.causal_off + 32 * nb + ql) : s1 - 1;  // last visible token
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int t = 8 * (r >> 2) + 4 * h + (r & 3);
+          x[r] = (tb + t <= tmax) ? sacc[nb][r] : -INFINITY;
+        }
       }
-      mloc = fmaxf(mloc, __shfl_xor(mloc, 32, kWave));
+      float mloc = fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3]));
+#pragma unroll
+      for (int r = 4; r < 16; r += 4) mloc = fmaxf(mloc, fmaxf(fmaxf(x[r], x[r + 1]), fmaxf(x[r + 2], x[r + 3])));
+      mloc = fmaxf(mloc, __shfl_xor(mloc, 32, kWave)) * scale_log2e;  // scale > 0 keeps the order
       const float mn = fmaxf(m[nb], mloc);
-      const float mref = (CAUSAL && mn == -INFINITY) ? 0.f : mn;  // a row with nothing visible yet
+      const float mref = (mn == -INFINITY) ? 0.f : mn;  // a row with nothing visible yet
       const float alpha = __builtin_amdgcn_exp2f(m[nb] - mref);
       m[nb] = mn;
       float ps = 0.f;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        x[r] = __builtin_amdgcn_exp2f(x[r] - mref);
+        x[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(x[r], scale_log2e, -mref));
         ps += x[r];
       }
       lsum[nb] = lsum[nb] * alpha + ps;
@@ -220,53 +231,75 @@ __device__ __forceinline__ void attn_tile(const TileWork& wk, const uint16_t* __
     }
   }
 
-  // fold the four waves: (2,3) -> (0,1), then 1 -> 0
-  constexpr int kDump = (4 * NQB * 16 + 2 * NQB) * 64 * 4;  // bytes per dumped wave
-  auto dump = [&](char* base) {
-    float* f = reinterpret_cast<float*>(base);
+  // Fold the four waves.  Every wave parks the three 32-dim blocks it does not own, and its (m, l);
+  // after one barrier wave w folds block w of all four waves, so the fold and the write-out that
+  // follows run on the whole workgroup.
+  constexpr int kBlk = NQB * 16 * 256;            // bytes of one (source wave, dim block): NQB x 16 floats x 64 lanes
+  char* mlb = smem + 16 * kBlk;                    // [wave][m or l][nb][lane] floats
+  __syncthreads();                                 // the staging tiles are dead from here on
 #pragma unroll
-    for (int db = 0; db < 4; ++db)
+  for (int db = 0; db < 4; ++db) {
+    if (db == w) continue;
+    char* base = smem + (w * 4 + db) * kBlk + lane * 16;
 #pragma unroll
-      for (int nb = 0; nb < NQB; ++nb)
+    for (int nb = 0; nb < NQB; ++nb)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) f[((db * NQB + nb) * 16 + r) * 64 + lane] = oacc[db][nb][r];
+      for (int j = 0; j < 4; ++j) {
+        const float4_t v = {oacc[db][nb][4 * j], oacc[db][nb][4 * j + 1], oacc[db][nb][4 * j + 2],
+                            oacc[db][nb][4 * j + 3]};
+        *reinterpret_cast<float4_t*>(base + (nb * 4 + j) * 1024) = v;
+      }
+  }
 #pragma unroll
-    for (int nb = 0; nb < NQB; ++nb) {
-      f[(4 * NQB * 16 + nb) * 64 + lane] = m[nb];
-      f[(4 * NQB * 16 + NQB + nb) * 64 + lane] = lsum[nb];
+  for (int nb = 0; nb < NQB; ++nb) {
+    *reinterpret_cast<float*>(mlb + ((w * 2 + 0) * NQB + nb) * 256 + lane * 4) = m[nb];
+    *reinterpret_cast<float*>(mlb + ((w * 2 + 1) * NQB + nb) * 256 + lane * 4) = lsum[nb];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int nb = 0; nb < NQB; ++nb) {
+    float ms[4], ls[4];
+    float M = -INFINITY;
+#pragma unroll
+    for (int src = 0; src < 4; ++src) {
+      ms[src] = *reinterpret_cast<const float*>(mlb + ((src * 2 + 0) * NQB + nb) * 256 + lane * 4);
+      ls[src] = *reinterpret_cast<const float*>(mlb + ((src * 2 + 1) * NQB + nb) * 256 + lane * 4);
+      M = fmaxf(M, ms[src]);
     }
-  };
-  auto fold = [&](const char* base) {
-    const float* f = reinterpret_cast<const float*>(base);
+    float L = 0.f;
 #pragma unroll
-    for (int nb = 0; nb < NQB; ++nb) {
-      const float mo = f[(4 * NQB * 16 + nb) * 64 + lane];
-      const float lo = f[(4 * NQB * 16 + NQB + nb) * 64 + lane];
-      const float mn = fmaxf(m[nb], mo);
-      const float sa = (m[nb] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m[nb] - mn);
-      const float sb = (mo == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mo - mn);
-      m[nb] = mn;
-      lsum[nb] = lsum[nb] * sa + lo * sb;
+    for (int r = 0; r < 16; ++r) ofold[nb][r] = 0.f;
 #pragma unroll
-      for (int db = 0; db < 4; ++db)
+    for (int src = 0; src < 4; ++src) {
+      const float sc = (ms[src] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(ms[src] - M);
+      L += ls[src] * sc;
+      if (src == w) {
+        // the block this wave kept in registers (static register index per candidate w)
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-          oacc[db][nb][r] = oacc[db][nb][r] * sa + f[((db * NQB + nb) * 16 + r) * 64 + lane] * sb;
+        for (int db = 0; db < 4; ++db)
+          if (db == w) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) ofold[nb][r] += oacc[db][nb][r] * sc;
+          }
+      } else {
+        const char* base = smem + (src * 4 + w) * kBlk + lane * 16;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float4_t v = *reinterpret_cast<const float4_t*>(base + (nb * 4 + j) * 1024);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) ofold[nb][4 * j + i] += v[i] * sc;
+        }
+      }
     }
-  };
-  __syncthreads();
-  if (w >= 2) dump(smem + (w - 2) * kDump);
-  __syncthreads();
-  if (w < 2) fold(smem + w * kDump);
-  __syncthreads();
-  if (w == 1) dump(smem);
-  __syncthreads();
-  if (w == 0) fold(smem);
+    mfin[nb] = M;
+    lfin[nb] = L + __shfl_xor(L, 32, kWave);
+  }
 }
 
 template <int NQB>
 constexpr int tile_lds_bytes() {
-  return 4 * kWaveLds > 2 * (4 * NQB * 16 + 2 * NQB) * 256 ? 4 * kWaveLds : 2 * (4 * NQB * 16 + 2 * NQB) * 256;
+  constexpr int fold = 16 * NQB * 16 * 256 + 4 * 2 * NQB * 256;  // parked blocks + (m, l) of four waves
+  return 4 * kWaveLds > fold ? 4 * kWaveLds : fold;
 }
 
 // Shared-prefix phase: workgroup = (split, head, group x query tile); writes one (O, m, l) part.
@@ -303,30 +336,25 @@ __global__ __launch_bounds__(256, 1) void prefix_mfma_kernel(PrefixArgs a, int m
   wk.s0 = s0;
   wk.s1 = s1;
   wk.causal_off = 0;
-  float16_t oacc[4][NQB];
-  float m[NQB], lsum[NQB];
-  attn_tile<E, NQB, false>(wk, a.kc, a.vc, a.row_stride, head, a.scale_log2e, smem, oacc, m, lsum);
-  if (threadIdx.x >= 64) return;
-  const int lane = threadIdx.x, h = lane >> 5, ql = lane & 31;
+  float16_t of[NQB];
+  float m[NQB], l[NQB];
+  attn_tile<E, NQB, false>(wk, a.kc, a.vc, a.row_stride, head, a.scale_log2e, smem, of, m, l);
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, h = lane >> 5, ql = lane & 31;
 #pragma unroll
   for (int nb = 0; nb < NQB; ++nb) {
-    const float L = lsum[nb] + __shfl_xor(lsum[nb], 32, kWave);
     const int q = 32 * nb + ql;
     if (q < nq) {
-      const float inv = 1.f / L;
+      const float inv = 1.f / l[nb];
       const int64_t pr = ((int64_t)split * a.B + qbase + q) * a.H + head;
-      float* op = a.opart + pr * kPD;
+      float* op = a.opart + pr * kPD + 32 * w + 4 * h;
 #pragma unroll
-      for (int db = 0; db < 4; ++db)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          float4_t v = {oacc[db][nb][4 * j] * inv, oacc[db][nb][4 * j + 1] * inv, oacc[db][nb][4 * j + 2] * inv,
-                        oacc[db][nb][4 * j + 3] * inv};
-          *reinterpret_cast<float4_t*>(op + 32 * db + 8 * j + 4 * h) = v;
-        }
-      if (h == 0) {
+      for (int j = 0; j < 4; ++j) {
+        float4_t v = {of[nb][4 * j] * inv, of[nb][4 * j + 1] * inv, of[nb][4 * j + 2] * inv, of[nb][4 * j + 3] * inv};
+        *reinterpret_cast<float4_t*>(op + 8 * j) = v;
+      }
+      if (h == 0 && w == 0) {
         a.ml[pr * 2] = m[nb];
-        a.ml[pr * 2 + 1] = L;
+        a.ml[pr * 2 + 1] = l[nb];
       }
     }
   }
@@ -360,26 +388,22 @@ __global__ __launch_bounds__(256, 1) void prefill_mfma_kernel(PrefillArgs a) {
   wk.s0 = 0;
   wk.causal_off = kvn - n + q0;
   wk.s1 = min(kvn, wk.causal_off + nq);  // the last live query sees tokens up to causal_off + nq - 1
-  float16_t oacc[4][2];
-  float m[2], lsum[2];
-  attn_tile<E, 2, true>(wk, a.kc, a.vc, a.row_stride, head, a.scale_log2e, smem, oacc, m, lsum);
-  if (threadIdx.x >= 64) return;
-  const int lane = threadIdx.x, h = lane >> 5, ql = lane & 31;
+  float16_t of[2];
+  float m[2], l[2];
+  attn_tile<E, 2, true>(wk, a.kc, a.vc, a.row_stride, head, a.scale_log2e, smem, of, m, l);
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, h = lane >> 5, ql = lane & 31;
 #pragma unroll
   for (int nb = 0; nb < 2; ++nb) {
-    const float L = lsum[nb] + __shfl_xor(lsum[nb], 32, kWave);
     const int q = 32 * nb + ql;
     if (q < nq) {
-      const float inv = L > 0.f ? 1.f / L : 0.f;
-      uint16_t* op = a.out + (int64_t)(cq0 + q0 + q) * a.out_stride + head * kPD;
+      const float inv = l[nb] > 0.f ? 1.f / l[nb] : 0.f;
+      uint16_t* op = a.out + (int64_t)(cq0 + q0 + q) * a.out_stride + head * kPD + 32 * w + 4 * h;
 #pragma unroll
-      for (int db = 0; db < 4; ++db)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          u32x2 v = {pack2<E>(oacc[db][nb][4 * j] * inv, oacc[db][nb][4 * j + 1] * inv),
-                     pack2<E>(oacc[db][nb][4 * j + 2] * inv, oacc[db][nb][4 * j + 3] * inv)};
-          *reinterpret_cast<u32x2*>(op + 32 * db + 8 * j + 4 * h) = v;
-        }
+      for (int j = 0; j < 4; ++j) {
+        u32x2 v = {pack2<E>(of[nb][4 * j] * inv, of[nb][4 * j + 1] * inv),
+                   pack2<E>(of[nb][4 * j + 2] * inv, of[nb][4 * j + 3] * inv)};
+        *reinterpret_cast<u32x2*>(op + 8 * j) = v;
+      }
     }
   }
 }
@@ -401,6 +425,8 @@ static int launch_prefix_t(const PrefixArgs& a, int num_groups, int max_group_re
   const int mtiles = (max_group_reqs + 32 * nqb - 1) / (32 * nqb);
   dim3 grid(a.n_splits, a.H, num_groups * mtiles), block(256);
   if (nqb == 1) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefix_mfma_kernel<E, 1>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, tile_lds_bytes<1>());
     hipLaunchKernelGGL((prefix_mfma_kernel<E, 1>), grid, block, tile_lds_bytes<1>(), st, a, mtiles);
   } else {
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefix_mfma_kernel<E, 2>),
