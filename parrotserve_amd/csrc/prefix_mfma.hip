@@ -5,8 +5,8 @@
 // Workgroup = (split of the prefix, head, group x 64-query tile), 4 waves.
 // Each wave owns every fourth 32-token tile of the split and ALL queries of
 // the tile, so each K/V byte is fetched from HBM once per (group, query tile)
-// and crosses LDS once: global -> registers (coalesced 128-bit gathers by slot)
-// -> wave-private LDS tile -> MFMA operand layout.  No workgroup barrier in
+// and crosses LDS once: global -> wave-private LDS tile (coalesced 128-bit gathers by slot, written
+// by the load itself, double-buffered) -> MFMA operand layout.  No workgroup barrier in
 // the main loop.  Online softmax in the exp2 domain, fp32 accumulation in
 // v_mfma_f32_32x32x16_{f16,bf16}.  The four waves' partials are folded through
 // LDS at the end and one (O, m, l) part per (split, request, head) is written.
@@ -48,8 +48,19 @@ struct Mfma32<BF16> {
 
 constexpr int kPD = 128;             // head size handled by this kernel
 constexpr int kTile = 32;            // tokens per wave tile
-constexpr int kWaveLds = 16384;      // K tile 8 KB + V^T tile 8 KB
+constexpr int kStage = 16384;        // one staged tile: K 8 KB + V 8 KB
+constexpr int kWaveLds = 2 * kStage; // two stages per wave
 constexpr int kVtOff = 8192;
+
+// 16 bytes per lane from global memory straight into LDS (no VGPR staging): lane i's data lands at
+// lds + 16 * i.  `lds` must be wave-uniform.  Issued as inline assembly on purpose: the compiler then
+// does not tie later LDS reads of the *other* stage to these loads, so a whole tile stays in flight
+// under the matrix work; completion is awaited explicitly (vmcnt) before a stage is read.
+__device__ __forceinline__ void lds_dma16(const void* gptr, const char* lds) {
+  const uint32_t dst =
+      __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)lds);
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(dst) : "memory");
+}
 
 __device__ __forceinline__ u32x4 lds_ld16(const char* p) { return *reinterpret_cast<const u32x4*>(p); }
 
@@ -79,7 +90,8 @@ __device__ __forceinline__ void attn_tile(const TileWork& wk, const uint16_t* __
                                           float scale_log2e, char* smem, float16_t (&ofold)[NQB], float (&mfin)[NQB],
                                           float (&lfin)[NQB]) {
   float16_t oacc[4][NQB];
-  float m[NQB], lsum[NQB];
+  float m[NQB], lsum[NQB], mtrue[NQB];  // exponent reference, denominator relative to it, true running maximum
+  constexpr float kSlack = 8.f;
   const int lane = threadIdx.x & 63;
   const int w = threadIdx.x >> 6;
   const int h = lane >> 5, ql = lane & 31;
@@ -90,6 +102,7 @@ __device__ __forceinline__ void attn_tile(const TileWork& wk, const uint16_t* __
 #pragma unroll
   for (int nb = 0; nb < NQB; ++nb) {
     m[nb] = -INFINITY;
+    mtrue[nb] = -INFINITY;
     lsum[nb] = 0.f;
 #pragma unroll
     for (int db = 0; db < 4; ++db)
@@ -97,27 +110,31 @@ __device__ __forceinline__ void attn_tile(const TileWork& wk, const uint16_t* __
       for (int r = 0; r < 16; ++r) oacc[db][nb][r] = 0.f;
   }
 
-  // global -> register staging: instruction r covers tokens 4r .. 4r+3, 16 lanes per token row
+  // global -> LDS staging without registers: instruction r covers tokens 4r .. 4r+3, 16 lanes per
+  // token row; LDS chunk position c of row t receives global chunk c ^ swizzle(t), so the tiles sit
+  // XOR-swizzled in LDS while every lane's destination stays lane-linear as the DMA requires.
   const int tl = lane >> 4, c = lane & 15;
-  const int64_t col = (int64_t)head * kPD + c * 8;
-  u32x4 kreg[8], vreg[8];
-  int snext[8];  // slot ids one tile ahead of the K/V rows in flight, so no load waits on a fresh slot fetch
+  const uint16_t* kcol = kc + (int64_t)head * kPD;
+  const uint16_t* vcol = vc + (int64_t)head * kPD + ((c ^ (4 * tl)) * 8);
+  int snext[8];  // slot ids one tile ahead of the K/V rows in flight, so no row load waits on a fresh slot fetch
   auto fetch_slots = [&](int t0) {
 #pragma unroll
     for (int r = 0; r < 8; ++r) snext[r] = slots[min(t0 + 4 * r + tl, s1 - 1)];
   };
-  auto fetch_rows = [&]() {
+  auto fetch_rows = [&](int stage) {
+    const char* kb = wl + stage * kStage;
 #pragma unroll
     for (int r = 0; r < 8; ++r) {
-      const int64_t ro = (int64_t)snext[r] * row_stride + col;
-      kreg[r] = ld16(kc + ro);
-      vreg[r] = ld16(vc + ro);
+      const int64_t ro = (int64_t)snext[r] * row_stride;
+      lds_dma16(kcol + ro + ((c ^ ((4 * r + tl) & 15)) * 8), kb + r * 1024);
+      lds_dma16(vcol + ro, kb + kVtOff + r * 1024);
     }
   };
   int tb = wk.s0 + kTile * w;
+  int stage = 0;
   if (tb < s1) {
     fetch_slots(tb);
-    fetch_rows();
+    fetch_rows(0);
     if (tb + 4 * kTile < s1) fetch_slots(tb + 4 * kTile);
   }
 
@@ -137,20 +154,17 @@ __device__ __forceinline__ void attn_tile(const TileWork& wk, const uint16_t* __
     }
   }
 
-  for (; tb < s1; tb += 4 * kTile) {
-    // registers -> LDS, both tiles row-major [token][dim] with XOR-swizzled 16-byte chunks
-#pragma unroll
-    for (int r = 0; r < 8; ++r) {
-      const int t = 4 * r + tl;
-      *reinterpret_cast<u32x4*>(wl + t * 256 + ((c ^ (t & 15)) * 16)) = kreg[r];
-      *reinterpret_cast<u32x4*>(wl + kVtOff + t * 256 + ((c ^ (4 * (t & 3))) * 16)) = vreg[r];
-    }
-    // next tile's rows go in flight now (their slot ids arrived during the previous tile);
+  for (; tb < s1; tb += 4 * kTile, stage ^= 1) {
+    // this tile's rows (and the slot ids fetched behind them) have landed
+    __builtin_amdgcn_s_waitcnt(0);
+    __builtin_amdgcn_sched_barrier(0);
+    // next tile's rows go in flight into the other stage (last read a full iteration ago);
     // then the slot ids of the tile after that
     if (tb + 4 * kTile < s1) {
-      fetch_rows();
+      fetch_rows(stage ^ 1);
       if (tb + 8 * kTile < s1) fetch_slots(tb + 8 * kTile);
     }
+    const char* st = wl + stage * kStage;
 
     // S^T = K Q^T
     float16_t sacc[NQB];
@@ -160,7 +174,7 @@ __device__ __forceinline__ void attn_tile(const TileWork& wk, const uint16_t* __
       for (int r = 0; r < 16; ++r) sacc[nb][r] = 0.f;
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
-      const u32x4 ka = lds_ld16(wl + ql * 256 + (((8 * h + s) ^ (ql & 15)) * 16));
+      const u32x4 ka = lds_ld16(st + ql * 256 + (((8 * h + s) ^ (ql & 15)) * 16));
 #pragma unroll
       for (int nb = 0; nb < NQB; ++nb) sacc[nb] = Mfma32<E>::run(ka, qop[nb][s], sacc[nb]);
     }
@@ -187,10 +201,17 @@ __device__ __forceinline__ void attn_tile(const TileWork& wk, const uint16_t* __
 #pragma unroll
       for (int r = 4; r < 16; r += 4) mloc = fmaxf(mloc, fmaxf(fmaxf(x[r], x[r + 1]), fmaxf(x[r + 2], x[r + 3])));
       mloc = fmaxf(mloc, __shfl_xor(mloc, 32, kWave)) * scale_log2e;  // scale > 0 keeps the order
-      const float mn = fmaxf(m[nb], mloc);
-      const float mref = (mn == -INFINITY) ? 0.f : mn;  // a row with nothing visible yet
-      const float alpha = __builtin_amdgcn_exp2f(m[nb] - mref);
-      m[nb] = mn;
+      mtrue[nb] = fmaxf(mtrue[nb], mloc);
+      // The exponent reference m[nb] follows the running maximum lazily: it moves only when the maximum
+      // has outgrown it by more than kSlack (so P stays below 2^kSlack, well inside fp16/bf16 range).
+      // The 128 accumulators of a lane live in accumulation registers the vector ALU cannot multiply
+      // in place, so skipping the rescale on almost every tile matters.
+      const bool move = mloc > m[nb] + kSlack;
+      const float mnew = move ? mloc : m[nb];
+      const float mref = (mnew == -INFINITY) ? 0.f : mnew;  // a row with nothing visible yet
+      const bool had = m[nb] != -INFINITY;                   // accumulators are still zero otherwise
+      const float alpha = (move && had) ? __builtin_amdgcn_exp2f(m[nb] - mref) : 1.f;
+      m[nb] = mnew;
       float ps = 0.f;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
@@ -198,10 +219,12 @@ __device__ __forceinline__ void attn_tile(const TileWork& wk, const uint16_t* __
         ps += x[r];
       }
       lsum[nb] = lsum[nb] * alpha + ps;
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {  // wave-uniform
 #pragma unroll
-      for (int db = 0; db < 4; ++db)
+        for (int db = 0; db < 4; ++db)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) oacc[db][nb][r] *= alpha;
+          for (int r = 0; r < 16; ++r) oacc[db][nb][r] *= alpha;
+      }
 #pragma unroll
       for (int u = 0; u < 2; ++u)
 #pragma unroll
@@ -215,7 +238,7 @@ __device__ __forceinline__ void attn_tile(const TileWork& wk, const uint16_t* __
       const int trow = 4 * h + (sl >> 2);                       // + 16u + 8x
       const int tcol = 2 * rh + ((sl & 3) >> 1);                // + 4db, in 16-byte chunks
       const int tswz = 4 * (sl >> 2);                           // = 4 * (row & 3)
-      const char* vbase = wl + kVtOff + trow * 256 + (sl & 1) * 8;
+      const char* vbase = st + kVtOff + trow * 256 + (sl & 1) * 8;
 #pragma unroll
       for (int db = 0; db < 4; ++db) {
         const int chunk = ((4 * db + tcol) ^ tswz) * 16;
@@ -254,6 +277,7 @@ __device__ __forceinline__ void attn_tile(const TileWork& wk, const uint16_t* __
   for (int nb = 0; nb < NQB; ++nb) {
     *reinterpret_cast<float*>(mlb + ((w * 2 + 0) * NQB + nb) * 256 + lane * 4) = m[nb];
     *reinterpret_cast<float*>(mlb + ((w * 2 + 1) * NQB + nb) * 256 + lane * 4) = lsum[nb];
+    *reinterpret_cast<float*>(mlb + ((8 + w) * NQB + nb) * 256 + lane * 4) = mtrue[nb];
   }
   __syncthreads();
 #pragma unroll
@@ -291,14 +315,23 @@ __device__ __forceinline__ void attn_tile(const TileWork& wk, const uint16_t* __
         }
       }
     }
-    mfin[nb] = M;
-    lfin[nb] = L + __shfl_xor(L, 32, kWave);
+    // report the true maximum, with the denominator re-expressed relative to it
+    float mt = mtrue[nb];
+#pragma unroll
+    for (int src = 0; src < 4; ++src)
+      mt = fmaxf(mt, *reinterpret_cast<const float*>(mlb + ((8 + src) * NQB + nb) * 256 + lane * 4));
+    const float Lall = L + __shfl_xor(L, 32, kWave);
+    const float toTrue = (mt == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(M - mt);
+    mfin[nb] = mt;
+    lfin[nb] = Lall * toTrue;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) ofold[nb][r] *= toTrue;
   }
 }
 
 template <int NQB>
 constexpr int tile_lds_bytes() {
-  constexpr int fold = 16 * NQB * 16 * 256 + 4 * 2 * NQB * 256;  // parked blocks + (m, l) of four waves
+  constexpr int fold = 16 * NQB * 16 * 256 + 4 * 3 * NQB * 256;  // parked blocks + (m, l, true max) of four waves
   return 4 * kWaveLds > fold ? 4 * kWaveLds : fold;
 }
 
