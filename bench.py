@@ -162,6 +162,8 @@ def extras(torch, dev):
                          "TFLOP/s": flops / t_pre / 1e12, "frac_mfma_peak": flops / t_pre / 1e12 / MFMA_F16_PEAK_TFLOPS,
                          "tokens/s/layer": T / t_pre}
     del kc4, vc4
+    # --- config 5: full LLaMA-13B decoder layer, 4 prefix groups x 32 branches, prefix 6000 ------------------
+    out["c5_layer"] = config5_layer(torch, dev)
     # --- RMSNorm at a bandwidth-sized row count (LLaMA-13B hidden) -----------------------------------------
     x = torch.randn((8192, 5120), device=dev, dtype=torch.float16)
     w = torch.ones(5120, device=dev, dtype=torch.float16)
@@ -170,6 +172,65 @@ def extras(torch, dev):
     out["rms_norm_8192x5120"] = {"us": t * 1e6, "GB/s": nbytes / t / 1e9, "frac_hbm": nbytes / t / 1e9 / HBM_PEAK_GBS,
                                  "algorithmic_bytes": nbytes}
     return out
+
+
+def config5_layer(torch, dev):
+    """RMSNorm -> QKV -> RoPE -> append -> grouped shared-prefix attention -> O-proj -> RMSNorm -> MLP, fp16,
+    hidden 5120, 40x128, FFN 13824, weights N(0, 0.02); GEMMs are library GEMMs (nn.Linear)."""
+    from parrotserve_amd import kernels, mem, synth
+    from parrotserve_amd.attn_func import BuiltinConfig
+    from parrotserve_amd.llama_layer import LlamaDecoderLayer
+
+    case = synth.config5()
+    dec = case.decode
+    B, H, D, hidden = dec.num_reqs, 40, 128, 5120
+    store = mem.init_model_cache_storage(1, dec.pool_slots, H, D, torch.float16, dev, max_seq_len=8192,
+                                         rope_theta=case.theta)
+    kc, vc = synth.pool_to_device(dec.k_rows, dec.v_rows, dec.used_slots, dec.pool_slots, dev)
+    store.k_cache[0].copy_(kc)
+    store.v_cache[0].copy_(vc)
+    del kc, vc
+    cfg = BuiltinConfig(num_kv_cache_blocks=dec.pool_slots, attn_func="hip_shared_prefix", dtype=torch.float16,
+                        device=dev)
+
+    class _State:  # the iteration state the plug-in builds from the jobs' context trees, here from the case's lists
+        pass
+
+    st = _State()
+    st.num_fill_tokens = []
+    st.generation_sampling_config = [None] * B
+    st.num_total_fill_tokens = 0
+    st.num_generation_jobs = B
+    st.slot_mapping = case.new_slots.to(torch.int32).to(dev)
+    st.fill_tables = None
+    st.decode_perm = None
+    st.decode_tables = kernels.DecodeTables.build(dec.pool_lists(dec.prefix_lists), dec.group_req_cu,
+                                                  dec.pool_lists(dec.suffix_lists), dev, num_heads=H, head_dim=D)
+    layer = LlamaDecoderLayer(hidden, H, 13824, case.eps, 0, cfg.attn_func).half().to(dev)
+    w = case.weights
+    with torch.no_grad():
+        layer.self_attn.qkv_proj.weight.copy_(w["qkv_proj"])
+        layer.self_attn.o_proj.weight.copy_(w["o_proj"])
+        layer.mlp.gate_proj.weight.copy_(w["gate_proj"])
+        layer.mlp.up_proj.weight.copy_(w["up_proj"])
+        layer.mlp.down_proj.weight.copy_(w["down_proj"])
+    x = case.x.to(dev)
+    pos = case.positions.to(dev)
+    q = torch.randn((B, H, D), device=dev, dtype=torch.float16)
+    o = torch.empty_like(q)
+    with torch.inference_mode():
+        t_layer = _time_gpu(torch, lambda: layer(x, pos, st), iters=20)
+        t_attn = _time_gpu(torch, lambda: kernels.decode_attention(q, store.k_cache[0], store.v_cache[0],
+                                                                   st.decode_tables, out=o), iters=20)
+    sum_s = sum(l.numel() for l in dec.suffix_lists)
+    P = dec.prefix_lists[0].numel()
+    kv_bytes = 2 * (len(dec.prefix_lists) * P + sum_s) * H * D * 2
+    res = {"batch": B, "groups": len(dec.prefix_lists), "prefix_len": P, "sum_suffix_len": sum_s,
+           "layer_ms": t_layer * 1e3, "attention_us": t_attn * 1e6, "attention_kv_bytes": kv_bytes,
+           "attention_GB/s": kv_bytes / t_attn / 1e9, "attention_frac_hbm": kv_bytes / t_attn / 1e9 / HBM_PEAK_GBS,
+           "tokens/s/layer": B / t_layer}
+    mem.Model_Cache = None
+    return res
 
 
 def kernels_cos_sin(torch, n, d, theta, dtype, dev):

@@ -15,8 +15,6 @@
 // parrot/engine/builtin/kernels/shared_flash_decoding.py:137-199 (n-way reduce).
 #include "decode.hpp"
 
-#include <cstdlib>
-
 namespace ph {
 
 // Streams the token rows slots[t0 .. t1) of one request through one wave (HPW adjacent heads) and
@@ -327,14 +325,7 @@ static int launch_items_t(const ItemArgs& a, hipStream_t st) {
   const int64_t waves = (int64_t)a.num_lanes * hgroups;
   if (waves == 0) return PH_OK;
   dim3 grid((unsigned)((waves + 3) / 4)), block(256);
-  static const int variant = getenv("PH_ITEMS_VARIANT") ? atoi(getenv("PH_ITEMS_VARIANT")) : 0;
-  switch (variant) {
-    case 1: hipLaunchKernelGGL((decode_items_kernel<E, D, 4, 1>), grid, block, 0, st, a); break;
-    case 2: hipLaunchKernelGGL((decode_items_kernel<E, D, 8, 2>), grid, block, 0, st, a); break;
-    case 3: hipLaunchKernelGGL((decode_items_kernel<E, D, 8, 1>), grid, block, 0, st, a); break;
-    case 4: hipLaunchKernelGGL((decode_items_kernel<E, D, 2, 2>), grid, block, 0, st, a); break;
-    default: hipLaunchKernelGGL((decode_items_kernel<E, D, 4, 2>), grid, block, 0, st, a); break;
-  }
+  hipLaunchKernelGGL((decode_items_kernel<E, D, 4, 2>), grid, block, 0, st, a);
   return launch_status();
 }
 

@@ -219,11 +219,23 @@ __device__ __forceinline__ void attn_tile(const TileWork& wk, const uint16_t* __
         ps += x[r];
       }
       lsum[nb] = lsum[nb] * alpha + ps;
-      if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {  // wave-uniform
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {  // wave-uniform, rare
+        // The accumulators live in accumulation registers, which the vector ALU cannot multiply in
+        // place.  The round trip is written as assembly pinned inside this branch so that it is not
+        // hoisted into the common path (where it would cost hundreds of register moves per tile).
+        // Wait states: the matrix results are 16 passes deep before the reads, and the rewritten
+        // registers are read as the C operand of the next matrix instruction after the writes.
+        asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 #pragma unroll
         for (int db = 0; db < 4; ++db)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) oacc[db][nb][r] *= alpha;
+          for (int r = 0; r < 16; ++r) {
+            float t;
+            asm volatile("v_accvgpr_read_b32 %0, %1\n\tv_mul_f32 %0, %0, %2\n\tv_accvgpr_write_b32 %1, %0"
+                         : "=&v"(t), "+a"(oacc[db][nb][r])
+                         : "v"(alpha));
+          }
+        asm volatile("s_nop 7" ::: "memory");
       }
 #pragma unroll
       for (int u = 0; u < 2; ++u)

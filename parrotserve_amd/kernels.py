@@ -343,8 +343,7 @@ def suffix_lanes(device, num_heads: int, head_dim: int, total_tokens: int) -> in
     cus = 256
     if torch.cuda.is_available() and str(device) != "cpu":
         cus = torch.cuda.get_device_properties(device).multi_processor_count
-    import os
-    lanes = max(1, int(cus * 4 * float(os.environ.get('PH_WPS', '3'))) // hgroups)
+    lanes = max(1, cus * 4 * 3 // hgroups)
     return max(1, min(lanes, (total_tokens + 15) // 16))
 
 
