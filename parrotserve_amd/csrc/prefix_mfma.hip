@@ -53,13 +53,15 @@ constexpr int kWaveLds = 2 * kStage; // two stages per wave
 constexpr int kVtOff = 8192;
 
 // 16 bytes per lane from global memory straight into LDS (no VGPR staging): lane i's data lands at
-// lds + 16 * i.  `lds` must be wave-uniform.  Issued as inline assembly on purpose: the compiler then
+// lds_addr + 16 * i (an LDS byte address, wave-uniform).  Issued as inline assembly on purpose: the compiler then
 // does not tie later LDS reads of the *other* stage to these loads, so a whole tile stays in flight
 // under the matrix work; completion is awaited explicitly (vmcnt) before a stage is read.
-__device__ __forceinline__ void lds_dma16(const void* gptr, const char* lds) {
-  const uint32_t dst =
-      __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)lds);
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(dst) : "memory");
+__device__ __forceinline__ void lds_dma16(const void* gptr, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(lds_addr) : "memory");
+}
+// LDS byte address of a generic pointer into shared memory, as a wave-uniform scalar
+__device__ __forceinline__ uint32_t lds_addr_of(const char* p) {
+  return __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)p);
 }
 
 __device__ __forceinline__ u32x4 lds_ld16(const char* p) { return *reinterpret_cast<const u32x4*>(p); }
@@ -114,20 +116,26 @@ __device__ __forceinline__ void attn_tile(const TileWork& wk, const uint16_t* __
   // token row; LDS chunk position c of row t receives global chunk c ^ swizzle(t), so the tiles sit
   // XOR-swizzled in LDS while every lane's destination stays lane-linear as the DMA requires.
   const int tl = lane >> 4, c = lane & 15;
-  const uint16_t* kcol = kc + (int64_t)head * kPD;
-  const uint16_t* vcol = vc + (int64_t)head * kPD + ((c ^ (4 * tl)) * 8);
-  int snext[8];  // slot ids one tile ahead of the K/V rows in flight, so no row load waits on a fresh slot fetch
-  auto fetch_slots = [&](int t0) {
+  // per-lane source bases (the row offset slot * row bytes is one 64-bit multiply-add per load)
+  const uint32_t row_bytes = (uint32_t)(row_stride * 2);
+  const char* kbase[8];
 #pragma unroll
-    for (int r = 0; r < 8; ++r) snext[r] = slots[min(t0 + 4 * r + tl, s1 - 1)];
-  };
+  for (int r = 0; r < 8; ++r)
+    kbase[r] = reinterpret_cast<const char*>(kc + (int64_t)head * kPD + ((c ^ ((4 * r + tl) & 15)) * 8));
+  const char* vbase_g = reinterpret_cast<const char*>(vc + (int64_t)head * kPD + ((c ^ (4 * tl)) * 8));
+  const uint32_t wl_lds = lds_addr_of(wl);
+  // the 32 slot ids of a tile sit in one VGPR (lane l: token l & 31), fetched one tile ahead of the
+  // rows in flight; a lane picks the id of the row it loads with a cross-lane read
+  int snext = 0;
+  auto fetch_slots = [&](int t0) { snext = slots[min(t0 + (lane & 31), s1 - 1)]; };
   auto fetch_rows = [&](int stage) {
-    const char* kb = wl + stage * kStage;
+    const uint32_t kb = wl_lds + stage * kStage;
 #pragma unroll
     for (int r = 0; r < 8; ++r) {
-      const int64_t ro = (int64_t)snext[r] * row_stride;
-      lds_dma16(kcol + ro + ((c ^ ((4 * r + tl) & 15)) * 8), kb + r * 1024);
-      lds_dma16(vcol + ro, kb + kVtOff + r * 1024);
+      const uint32_t slot = (uint32_t)__shfl(snext, 4 * r + tl, kWave);
+      const uint64_t ro = (uint64_t)slot * row_bytes;
+      lds_dma16(kbase[r] + ro, kb + r * 1024);
+      lds_dma16(vbase_g + ro, kb + kVtOff + r * 1024);
     }
   };
   int tb = wk.s0 + kTile * w;
@@ -172,17 +180,46 @@ __device__ __forceinline__ void attn_tile(const TileWork& wk, const uint16_t* __
     for (int nb = 0; nb < NQB; ++nb)
 #pragma unroll
       for (int r = 0; r < 16; ++r) sacc[nb][r] = 0.f;
+    // All LDS operand reads of the tile are issued ahead of their consumers and pinned there with
+    // scheduling barriers (left alone, the scheduler sinks every read next to the matrix instruction
+    // that uses it and the LDS latency is paid once per instruction): the eight K operands before the
+    // score product, the V operands right behind it so that they arrive under the softmax arithmetic.
+    u32x4 ka[8];
 #pragma unroll
-    for (int s = 0; s < 8; ++s) {
-      const u32x4 ka = lds_ld16(st + ql * 256 + (((8 * h + s) ^ (ql & 15)) * 16));
+    for (int s = 0; s < 8; ++s) ka[s] = lds_ld16(st + ql * 256 + (((8 * h + s) ^ (ql & 15)) * 16));
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int nb = 0; nb < NQB; ++nb) sacc[nb] = Mfma32<E>::run(ka, qop[nb][s], sacc[nb]);
+    for (int s = 0; s < 8; ++s)
+#pragma unroll
+      for (int nb = 0; nb < NQB; ++nb) sacc[nb] = Mfma32<E>::run(ka[s], qop[nb][s], sacc[nb]);
+    u32x4 va[4][2];
+    {
+      // A operand of O^T += V^T P^T (row = dim 32db + ql, contraction = the 8 tokens of (h, u)): two
+      // transposing reads, tokens 16u + 4h + {0..3} and 16u + 8 + 4h + {0..3}.
+      const int sl = lane & 15, rh = (lane >> 4) & 1;
+      const int trow = 4 * h + (sl >> 2);                       // + 16u + 8x
+      const int tcol = 2 * rh + ((sl & 3) >> 1);                // + 4db, in 16-byte chunks
+      const int tswz = 4 * (sl >> 2);                           // = 4 * (row & 3)
+      const char* vbase = st + kVtOff + trow * 256 + (sl & 1) * 8;
+#pragma unroll
+      for (int db = 0; db < 4; ++db) {
+        const int chunk = ((4 * db + tcol) ^ tswz) * 16;
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const u32x2 lo = lds_tr16(vbase + (16 * u) * 256 + chunk);
+          const u32x2 hi = lds_tr16(vbase + (16 * u + 8) * 256 + chunk);
+          va[db][u] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+        }
+      }
     }
+    __builtin_amdgcn_sched_barrier(0);
 
     // online softmax in the exp2 domain (scores are scaled inside the exponent's fma); P^T is packed
     // straight into B-operand form.  Only a split's last tile and causal tiles need token masks.
     u32x4 pop[NQB][2];
-    const bool full = !CAUSAL && tb + kTile <= s1;
+    // tokens need masking only in a split's last tile and, when causal, in tiles that reach past what
+    // the tile's first query may see
+    const bool full = tb + kTile <= s1 && (!CAUSAL || tb + kTile - 1 <= wk.causal_off);
 #pragma unroll
     for (int nb = 0; nb < NQB; ++nb) {
       float x[16];
@@ -243,27 +280,13 @@ __device__ __forceinline__ void attn_tile(const TileWork& wk, const uint16_t* __
         for (int e = 0; e < 4; ++e) pop[nb][u][e] = pack2<E>(x[8 * u + 2 * e], x[8 * u + 2 * e + 1]);
     }
 
-    // O^T += V^T P^T.  A operand (row = dim 32db + ql, contraction = the 8 tokens of (h, u)):
-    // two transposing reads, tokens 16u + 4h + {0..3} and 16u + 8 + 4h + {0..3}.
-    {
-      const int sl = lane & 15, rh = (lane >> 4) & 1;
-      const int trow = 4 * h + (sl >> 2);                       // + 16u + 8x
-      const int tcol = 2 * rh + ((sl & 3) >> 1);                // + 4db, in 16-byte chunks
-      const int tswz = 4 * (sl >> 2);                           // = 4 * (row & 3)
-      const char* vbase = st + kVtOff + trow * 256 + (sl & 1) * 8;
+    // O^T += V^T P^T
 #pragma unroll
-      for (int db = 0; db < 4; ++db) {
-        const int chunk = ((4 * db + tcol) ^ tswz) * 16;
+    for (int db = 0; db < 4; ++db)
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
-          const u32x2 lo = lds_tr16(vbase + (16 * u) * 256 + chunk);
-          const u32x2 hi = lds_tr16(vbase + (16 * u + 8) * 256 + chunk);
-          const u32x4 va = {lo[0], lo[1], hi[0], hi[1]};
+      for (int u = 0; u < 2; ++u)
 #pragma unroll
-          for (int nb = 0; nb < NQB; ++nb) oacc[db][nb] = Mfma32<E>::run(va, pop[nb][u], oacc[db][nb]);
-        }
-      }
-    }
+        for (int nb = 0; nb < NQB; ++nb) oacc[db][nb] = Mfma32<E>::run(va[db][u], pop[nb][u], oacc[db][nb]);
   }
 
   // Fold the four waves.  Every wave parks the three 32-dim blocks it does not own, and its (m, l);
