@@ -27,9 +27,10 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16
 
-# HBM traffic of one suffix-kernel launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (profiles/decode_partial_c2_pmc.txt); None until measured.
-SUFFIX_TRAFFIC_BYTES = None
+# HBM traffic of one suffix-kernel launch at this workload, measured with rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE in two runs of this file and scaled by the same counters' readings for a plain 1 GiB copy
+# (profiles/bench_config2_hbm_traffic.txt): 285.5 MB read + 7.4 MB written.
+SUFFIX_TRAFFIC_BYTES = 293.0e6
 
 
 class HipEvents:
@@ -87,19 +88,31 @@ def cpu_baseline(case, sample_reqs: int):
     }
 
 
-def _time_gpu(torch, fn, iters=20, warmup=3):
+def _time_gpu(torch, fn, iters=20, warmup=3, inner=10):
+    """Median over `iters` samples of the time per call when `inner` calls are queued back to back between two
+    events (the queue stays full, so host launch latency is not in the figure); also p10 and p90."""
     for _ in range(warmup):
         fn()
     a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     ts = []
     for _ in range(iters):
         a.record()
-        fn()
+        for _ in range(inner):
+            fn()
         b.record()
         b.synchronize()
-        ts.append(a.elapsed_time(b) * 1e-3)
+        ts.append(a.elapsed_time(b) * 1e-3 / inner)
     ts.sort()
     return ts[len(ts) // 2]
+
+
+class _Rotor:
+    def __init__(self, n):
+        self.n, self.i = n, 0
+
+    def next(self):
+        self.i = (self.i + 1) % self.n
+        return self.i
 
 
 def extras(torch, dev):
@@ -138,14 +151,27 @@ def extras(torch, dev):
     T, H4, _ = c4.q.shape
     kc4, vc4 = synth.pool_to_device(c4.k_rows, c4.v_rows, c4.used_slots, c4.pool_slots, dev)
     cache = kernels_cos_sin(torch, int(c4.positions.max()) + 1, D, c4.theta, torch.bfloat16, dev)
-    qkv = torch.randn((T, 3 * H4 * D), device=dev, dtype=torch.bfloat16)
-    q4, k4, v4 = qkv.chunk(3, dim=-1)
+    # RoPE and append rotate over 4 projections' outputs (4 x 289 MB) so that their inputs come from HBM,
+    # not from the 256 MB memory-side cache
+    qkvs = [torch.randn((T, 3 * H4 * D), device=dev, dtype=torch.bfloat16) for _ in range(4)]
+    rot = _Rotor(len(qkvs))
+    q4, k4, v4 = qkvs[0].chunk(3, dim=-1)
     pos = c4.positions.to(dev)
-    t_rope = _time_gpu(torch, lambda: kernels.vllm_rotary_emb(pos, q4, k4, cache, D))
+
+    def rope_step():
+        qi, ki, _ = qkvs[rot.next()].chunk(3, dim=-1)
+        kernels.vllm_rotary_emb(pos, qi, ki, cache, D)
+
+    t_rope = _time_gpu(torch, rope_step)
     rope_bytes = 2 * T * 2 * H4 * D * 2 + T * D * 2
     new_slots = torch.cat([c4.used_slots[n] for n in c4.new_lists]).to(torch.int32).to(dev)
     k3, v3 = k4.view(T, H4, D), v4.view(T, H4, D)
-    t_app = _time_gpu(torch, lambda: kernels.vllm_reshape_and_cache(k3, v3, kc4, vc4, new_slots))
+
+    def append_step():
+        _, ki, vi = qkvs[rot.next()].chunk(3, dim=-1)
+        kernels.vllm_reshape_and_cache(ki.view(T, H4, D), vi.view(T, H4, D), kc4, vc4, new_slots)
+
+    t_app = _time_gpu(torch, append_step)
     ctx = [c4.used_slots[torch.cat([p, n])].tolist() for p, n in zip(c4.parent_lists, c4.new_lists)]
     ptab = kernels.PrefillTables.build(c4.q_lens, ctx, dev)
     qc = q4.reshape(T, H4, D).contiguous()
@@ -161,14 +187,15 @@ def extras(torch, dev):
     out["c4_prefill"] = {"tokens": T, "chunks": len(c4.q_lens), "ms": t_pre * 1e3, "flops": flops,
                          "TFLOP/s": flops / t_pre / 1e12, "frac_mfma_peak": flops / t_pre / 1e12 / MFMA_F16_PEAK_TFLOPS,
                          "tokens/s/layer": T / t_pre}
-    del kc4, vc4
+    del kc4, vc4, qkvs
     # --- config 5: full LLaMA-13B decoder layer, 4 prefix groups x 32 branches, prefix 6000 ------------------
     out["c5_layer"] = config5_layer(torch, dev)
     # --- RMSNorm at a bandwidth-sized row count (LLaMA-13B hidden) -----------------------------------------
-    x = torch.randn((8192, 5120), device=dev, dtype=torch.float16)
+    xs = [torch.randn((8192, 5120), device=dev, dtype=torch.float16) for _ in range(8)]  # 8 x 84 MB, rotated
     w = torch.ones(5120, device=dev, dtype=torch.float16)
-    t = _time_gpu(torch, lambda: kernels.vllm_rms_norm(x, w, 1e-6))
-    nbytes = 2 * x.numel() * 2 + 5120 * 2
+    rot = _Rotor(len(xs))
+    t = _time_gpu(torch, lambda: kernels.vllm_rms_norm(xs[rot.next()], w, 1e-6))
+    nbytes = 2 * xs[0].numel() * 2 + 5120 * 2
     out["rms_norm_8192x5120"] = {"us": t * 1e6, "GB/s": nbytes / t / 1e9, "frac_hbm": nbytes / t / 1e9 / HBM_PEAK_GBS,
                                  "algorithmic_bytes": nbytes}
     return out
@@ -248,6 +275,9 @@ def main():
     ap.add_argument("--cpu-sample", type=int, default=16)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the other configurations' kernel rooflines")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run the move kernel as a plain 1 GiB copy (known traffic, to scale the profiler's "
+                         "FETCH_SIZE / WRITE_SIZE counters) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs the hot path on ONE GPU; --gpus must be 1 "
@@ -261,6 +291,17 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     lib = _lib.load()
+
+    if args.copy_calibration:
+        rows = 131072  # x 8 KiB = 1 GiB read + 1 GiB written per launch
+        src = torch.randn(rows, 32, 128, device=dev, dtype=torch.float16)
+        dst = torch.empty_like(src)
+        idx = torch.arange(rows, device=dev)
+        for _ in range(6):
+            kernels.discontinuous_move_tokens(src, dst, idx, idx)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_calibration": {"launches": 6, "bytes_read": rows * 8192, "bytes_written": rows * 8192}}))
+        return
 
     case = synth.config2()
     B, H, D = case.q.shape
@@ -305,15 +346,16 @@ def main():
     t_step = timed(step, args.steps, args.warmup)
     t_warm = timed(lambda i: kernels.decode_attention(qs[0], kc, vc, tables[0], out=out), args.steps, args.warmup)
 
-    # per-kernel durations inside the same rotation, HIP events on the launch stream
+    # per-kernel durations inside the same rotation: each kernel's own dispatch begin/end (start/stop events
+    # attached to its launch on the launch stream), the quantity a kernel trace reports
     ev = HipEvents()
     n_ev = min(args.steps, 200)
-    sets = [ev.create(4) for _ in range(n_ev)]
+    sets = [ev.create(6) for _ in range(n_ev)]
     for i in range(n_ev):
-        lib.ph_arm_phase_events(sets[i])
+        lib.ph_arm_kernel_events(sets[i])
         step(i)
     torch.cuda.synchronize()
-    ph = [[ev.elapsed_ms(s[k], s[k + 1]) for s in sets] for k in range(3)]
+    ph = [[ev.elapsed_ms(s[2 * k], s[2 * k + 1]) for s in sets] for k in range(3)]
     for s in sets:
         ev.destroy(s)
     t_prefix, t_suffix, t_merge = (sum(x) / len(x) * 1e-3 for x in ph)
@@ -345,7 +387,7 @@ def main():
             "batch": B, "prefix_len": P, "sum_suffix_len": sum_s, "heads": H, "head_dim": D, "kv_sets": NL,
         },
         "roofline": {
-            "kernel": "decode_partial_kernel (suffix phase)",
+            "kernel": "decode_items_kernel (suffix phase)",
             "bound": "hbm",
             "achieved": suffix_gbs,
             "peak": HBM_PEAK_GBS,

@@ -249,12 +249,15 @@ int ph_prefill_attention(void* out, const void* q, const void* k_cache, const vo
 /* ------------------------------------------------------------------------ */
 /* Instrumentation (no counterpart in the reference, which times whole
  * iterations from Python, parrot/engine/builtin/builtin_runner.py:158-175).
- * Arms the NEXT ph_decode_attention call on this thread's library state: it
- * records events[0] before the prefix kernel, events[1] before the suffix
- * kernel, events[2] before the merge kernel and events[3] after it, on the
- * call's stream (hipEvent_t handles owned by the caller).  One call consumes
- * the arming.  Pass NULL to disarm. */
-int ph_arm_phase_events(void* const* events4);
+ * Arms the NEXT ph_decode_attention call of the process: its prefix, suffix
+ * and merge kernels are launched with (start, stop) event pairs that carry
+ * each dispatch's own begin and end timestamps: events[0,1] prefix kernel,
+ * events[2,3] suffix kernel, events[4,5] merge kernel (hipEvent_t handles
+ * created and owned by the caller; read them with hipEventElapsedTime after
+ * synchronising).  A pair whose kernel the call does not launch is left
+ * untouched.  One call consumes the arming; pass NULL to disarm.  Not for
+ * concurrent callers. */
+int ph_arm_kernel_events(void* const* events6);
 
 #ifdef __cplusplus
 }

@@ -166,18 +166,23 @@ extern "C" const char* ph_status_string(int status) {
 
 extern "C" int ph_abi_version(void) { return 1; }
 
-static hipEvent_t g_phase_events[4];
-static bool g_phase_armed = false;
+static hipEvent_t g_kernel_events[6];
+static bool g_events_armed = false;
 
-extern "C" int ph_arm_phase_events(void* const* events4) {
-  g_phase_armed = events4 != nullptr;
-  if (events4)
-    for (int i = 0; i < 4; ++i) g_phase_events[i] = (hipEvent_t)events4[i];
+extern "C" int ph_arm_kernel_events(void* const* events6) {
+  g_events_armed = events6 != nullptr;
+  if (events6)
+    for (int i = 0; i < 6; ++i) g_kernel_events[i] = (hipEvent_t)events6[i];
   return PH_OK;
 }
 
-static inline void phase_mark(bool armed, int i, hipStream_t st) {
-  if (armed) (void)hipEventRecord(g_phase_events[i], st);
+ph::KernelEvents ph::take_kernel_events(int which) {
+  KernelEvents e;
+  if (g_events_armed && which >= 0 && which < 3) {
+    e.start = g_kernel_events[2 * which];
+    e.stop = g_kernel_events[2 * which + 1];
+  }
+  return e;
 }
 
 extern "C" size_t ph_decode_workspace_bytes(int64_t num_reqs, int64_t num_heads, int64_t head_dim,
@@ -219,10 +224,6 @@ extern "C" int ph_decode_attention(void* out, const void* q, const void* k_cache
   const Carve ws = carve(workspace, p, B, H, D);
   hipStream_t st = (hipStream_t)stream;
   const float sl2 = scale * kLog2e;
-  const bool armed = g_phase_armed;
-  g_phase_armed = false;
-
-  phase_mark(armed, 0, st);
   if (has_prefix) {
     int covered = 0, max_group_reqs = 0;
     for (int g = 0; g < num_groups; ++g) {
@@ -255,7 +256,6 @@ extern "C" int ph_decode_attention(void* out, const void* q, const void* k_cache
     rc = run_prefix(pa, dtype, D, (int)num_groups, group_req_cu_host, max_group_reqs, st);
     if (rc != PH_OK) return rc;
   }
-  phase_mark(armed, 1, st);
   const int64_t item_base = (int64_t)p.n_splits * B * H;  // first partial row of the balanced form's items
   if (planned) {
     ItemArgs ia{};
@@ -316,9 +316,8 @@ extern "C" int ph_decode_attention(void* out, const void* q, const void* k_cache
   ma.chunk = p.chunk;
   ma.req_item_cu = planned ? plan->req_item_cu : nullptr;
   ma.item_base = item_base;
-  phase_mark(armed, 2, st);
   rc = launch_merge(ma, dtype, D, st);
-  phase_mark(armed, 3, st);
+  g_events_armed = false;  // one call consumes the arming
   return rc;
 }
 

@@ -3,6 +3,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stdint.h>
 
 #include "../../include/parrot_hip.h"
@@ -114,6 +115,14 @@ __device__ __forceinline__ float group_max(float v) {
   for (int s = W / 2; s >= 1; s >>= 1) v = fmaxf(v, __shfl_xor(v, s, kWave));
   return v;
 }
+
+// Optional timing of one kernel's own dispatch: the three main kernels of the decode path (0 prefix,
+// 1 suffix, 2 merge) are launched through hipExtLaunchKernelGGL, which stamps a start and a stop event
+// with the dispatch's begin and end timestamps.  Null events (the normal case) make it a plain launch.
+struct KernelEvents {
+  hipEvent_t start = nullptr, stop = nullptr;
+};
+KernelEvents take_kernel_events(int which);  // attention_api.hip; nulls unless the call was armed
 
 inline int launch_status() { return hipGetLastError() == hipSuccess ? PH_OK : PH_ERR_LAUNCH; }
 

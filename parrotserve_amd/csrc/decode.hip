@@ -314,7 +314,8 @@ static int launch_partial_t(const PartialArgs& a, hipStream_t st) {
   const int64_t waves = (int64_t)a.num_reqs * a.n_chunks * hgroups;
   if (waves == 0) return PH_OK;
   dim3 grid((unsigned)((waves + 3) / 4)), block(256);
-  hipLaunchKernelGGL((decode_partial_kernel<E, D, 4, 2>), grid, block, 0, st, a);
+  const KernelEvents ev = take_kernel_events(1);
+  hipExtLaunchKernelGGL((decode_partial_kernel<E, D, 4, 2>), grid, block, 0, st, ev.start, ev.stop, 0, a);
   return launch_status();
 }
 
@@ -325,7 +326,8 @@ static int launch_items_t(const ItemArgs& a, hipStream_t st) {
   const int64_t waves = (int64_t)a.num_lanes * hgroups;
   if (waves == 0) return PH_OK;
   dim3 grid((unsigned)((waves + 3) / 4)), block(256);
-  hipLaunchKernelGGL((decode_items_kernel<E, D, 4, 2>), grid, block, 0, st, a);
+  const KernelEvents ev = take_kernel_events(1);
+  hipExtLaunchKernelGGL((decode_items_kernel<E, D, 4, 2>), grid, block, 0, st, ev.start, ev.stop, 0, a);
   return launch_status();
 }
 
@@ -336,7 +338,8 @@ static int launch_merge_t(const MergeArgs& a, hipStream_t st) {
   const int64_t groups = (int64_t)a.B * hgroups;
   if (groups == 0) return PH_OK;
   dim3 grid((unsigned)groups), block(256);
-  hipLaunchKernelGGL((merge_kernel<E, D>), grid, block, 0, st, a);
+  const KernelEvents ev = take_kernel_events(2);
+  hipExtLaunchKernelGGL((merge_kernel<E, D>), grid, block, 0, st, ev.start, ev.stop, 0, a);
   return launch_status();
 }
 

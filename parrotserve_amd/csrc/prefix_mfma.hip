@@ -176,10 +176,6 @@ __device__ __forceinline__ void attn_tile(const TileWork& wk, const uint16_t* __
 
     // S^T = K Q^T
     float16_t sacc[NQB];
-#pragma unroll
-    for (int nb = 0; nb < NQB; ++nb)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) sacc[nb][r] = 0.f;
     // All LDS operand reads of the tile are issued ahead of their consumers and pinned there with
     // scheduling barriers (left alone, the scheduler sinks every read next to the matrix instruction
     // that uses it and the LDS latency is paid once per instruction): the eight K operands before the
@@ -188,10 +184,15 @@ __device__ __forceinline__ void attn_tile(const TileWork& wk, const uint16_t* __
 #pragma unroll
     for (int s = 0; s < 8; ++s) ka[s] = lds_ld16(st + ql * 256 + (((8 * h + s) ^ (ql & 15)) * 16));
     __builtin_amdgcn_sched_barrier(0);
+    {
+      const float16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int s = 0; s < 8; ++s)
+      for (int nb = 0; nb < NQB; ++nb) sacc[nb] = Mfma32<E>::run(ka[0], qop[nb][0], zero);
 #pragma unroll
-      for (int nb = 0; nb < NQB; ++nb) sacc[nb] = Mfma32<E>::run(ka[s], qop[nb][s], sacc[nb]);
+      for (int s = 1; s < 8; ++s)
+#pragma unroll
+        for (int nb = 0; nb < NQB; ++nb) sacc[nb] = Mfma32<E>::run(ka[s], qop[nb][s], sacc[nb]);
+    }
     u32x4 va[4][2];
     {
       // A operand of O^T += V^T P^T (row = dim 32db + ql, contraction = the 8 tokens of (h, u)): two
@@ -214,55 +215,52 @@ __device__ __forceinline__ void attn_tile(const TileWork& wk, const uint16_t* __
     }
     __builtin_amdgcn_sched_barrier(0);
 
-    // online softmax in the exp2 domain (scores are scaled inside the exponent's fma); P^T is packed
-    // straight into B-operand form.  Only a split's last tile and causal tiles need token masks.
-    u32x4 pop[NQB][2];
-    // tokens need masking only in a split's last tile and, when causal, in tiles that reach past what
-    // the tile's first query may see
+    // Online softmax in the exp2 domain, in two phases around the (rare) accumulator rescale, so that
+    // the exponent work of one query block and the P.V matrix instructions of the other share a
+    // scheduling region and can overlap.  Tokens need masking only in a split's last tile and, when
+    // causal, in tiles that reach past what the tile's first query may see.
     const bool full = tb + kTile <= s1 && (!CAUSAL || tb + kTile - 1 <= wk.causal_off);
+    float x[NQB][16], mref[NQB], alpha[NQB];
 #pragma unroll
     for (int nb = 0; nb < NQB; ++nb) {
-      float x[16];
       if (full) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) x[r] = sacc[nb][r];
+        for (int r = 0; r < 16; ++r) x[nb][r] = sacc[nb][r];
       } else {
         const int tmax = CAUSAL ? min(s1 - 1, wk.causal_off + 32 * nb + ql) : s1 - 1;  // last visible token
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int t = 8 * (r >> 2) + 4 * h + (r & 3);
-          x[r] = (tb + t <= tmax) ? sacc[nb][r] : -INFINITY;
+          x[nb][r] = (tb + t <= tmax) ? sacc[nb][r] : -INFINITY;
         }
       }
-      float mloc = fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3]));
+      float mloc = fmaxf(fmaxf(x[nb][0], x[nb][1]), fmaxf(x[nb][2], x[nb][3]));
 #pragma unroll
-      for (int r = 4; r < 16; r += 4) mloc = fmaxf(mloc, fmaxf(fmaxf(x[r], x[r + 1]), fmaxf(x[r + 2], x[r + 3])));
+      for (int r = 4; r < 16; r += 4)
+        mloc = fmaxf(mloc, fmaxf(fmaxf(x[nb][r], x[nb][r + 1]), fmaxf(x[nb][r + 2], x[nb][r + 3])));
       mloc = fmaxf(mloc, __shfl_xor(mloc, 32, kWave)) * scale_log2e;  // scale > 0 keeps the order
       mtrue[nb] = fmaxf(mtrue[nb], mloc);
       // The exponent reference m[nb] follows the running maximum lazily: it moves only when the maximum
       // has outgrown it by more than kSlack (so P stays below 2^kSlack, well inside fp16/bf16 range).
-      // The 128 accumulators of a lane live in accumulation registers the vector ALU cannot multiply
-      // in place, so skipping the rescale on almost every tile matters.
       const bool move = mloc > m[nb] + kSlack;
       const float mnew = move ? mloc : m[nb];
-      const float mref = (mnew == -INFINITY) ? 0.f : mnew;  // a row with nothing visible yet
+      mref[nb] = (mnew == -INFINITY) ? 0.f : mnew;           // a row with nothing visible yet
       const bool had = m[nb] != -INFINITY;                   // accumulators are still zero otherwise
-      const float alpha = (move && had) ? __builtin_amdgcn_exp2f(m[nb] - mref) : 1.f;
+      alpha[nb] = (move && had) ? __builtin_amdgcn_exp2f(m[nb] - mref[nb]) : 1.f;
       m[nb] = mnew;
-      float ps = 0.f;
+    }
+    bool rescale = false;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        x[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(x[r], scale_log2e, -mref));
-        ps += x[r];
-      }
-      lsum[nb] = lsum[nb] * alpha + ps;
-      if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {  // wave-uniform, rare
-        // The accumulators live in accumulation registers, which the vector ALU cannot multiply in
-        // place.  The round trip is written as assembly pinned inside this branch so that it is not
-        // hoisted into the common path (where it would cost hundreds of register moves per tile).
-        // Wait states: the matrix results are 16 passes deep before the reads, and the rewritten
-        // registers are read as the C operand of the next matrix instruction after the writes.
-        asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    for (int nb = 0; nb < NQB; ++nb) rescale = rescale || alpha[nb] != 1.f;
+    if (__builtin_amdgcn_ballot_w64(rescale) != 0) {  // wave-uniform, rare
+      // The accumulators live in accumulation registers, which the vector ALU cannot multiply in
+      // place.  The round trip is written as assembly pinned inside this branch so that it is not
+      // hoisted into the common path (where it would cost hundreds of register moves per tile).
+      // Wait states: the matrix results are 16 passes deep before the reads, and the rewritten
+      // registers are read as the C operand of the next matrix instruction after the writes.
+      asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+#pragma unroll
+      for (int nb = 0; nb < NQB; ++nb)
 #pragma unroll
         for (int db = 0; db < 4; ++db)
 #pragma unroll
@@ -270,23 +268,30 @@ __device__ __forceinline__ void attn_tile(const TileWork& wk, const uint16_t* __
             float t;
             asm volatile("v_accvgpr_read_b32 %0, %1\n\tv_mul_f32 %0, %0, %2\n\tv_accvgpr_write_b32 %1, %0"
                          : "=&v"(t), "+a"(oacc[db][nb][r])
-                         : "v"(alpha));
+                         : "v"(alpha[nb]));
           }
-        asm volatile("s_nop 7" ::: "memory");
-      }
-#pragma unroll
-      for (int u = 0; u < 2; ++u)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) pop[nb][u][e] = pack2<E>(x[8 * u + 2 * e], x[8 * u + 2 * e + 1]);
+      asm volatile("s_nop 7" ::: "memory");
     }
-
-    // O^T += V^T P^T
+    // exponentials, denominators, P^T packed straight into B-operand form, and O^T += V^T P^T
 #pragma unroll
-    for (int db = 0; db < 4; ++db)
+    for (int nb = 0; nb < NQB; ++nb) {
+      float ps = 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        x[nb][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(x[nb][r], scale_log2e, -mref[nb]));
+        ps += x[nb][r];
+      }
+      lsum[nb] = lsum[nb] * alpha[nb] + ps;
+      u32x4 pop[2];
 #pragma unroll
       for (int u = 0; u < 2; ++u)
 #pragma unroll
-        for (int nb = 0; nb < NQB; ++nb) oacc[db][nb] = Mfma32<E>::run(va[db][u], pop[nb][u], oacc[db][nb]);
+        for (int e = 0; e < 4; ++e) pop[u][e] = pack2<E>(x[nb][8 * u + 2 * e], x[nb][8 * u + 2 * e + 1]);
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int u = 0; u < 2; ++u) oacc[db][nb] = Mfma32<E>::run(va[db][u], pop[u], oacc[db][nb]);
+    }
   }
 
   // Fold the four waves.  Every wave parks the three 32-dim blocks it does not own, and its (m, l);
@@ -492,14 +497,15 @@ static int launch_prefix_t(const PrefixArgs& a, int num_groups, int max_group_re
   const int nqb = max_group_reqs <= 32 ? 1 : 2;
   const int mtiles = (max_group_reqs + 32 * nqb - 1) / (32 * nqb);
   dim3 grid(a.n_splits, a.H, num_groups * mtiles), block(256);
+  const KernelEvents ev = take_kernel_events(0);
   if (nqb == 1) {
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefix_mfma_kernel<E, 1>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, tile_lds_bytes<1>());
-    hipLaunchKernelGGL((prefix_mfma_kernel<E, 1>), grid, block, tile_lds_bytes<1>(), st, a, mtiles);
+    hipExtLaunchKernelGGL((prefix_mfma_kernel<E, 1>), grid, block, tile_lds_bytes<1>(), st, ev.start, ev.stop, 0, a, mtiles);
   } else {
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefix_mfma_kernel<E, 2>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, tile_lds_bytes<2>());
-    hipLaunchKernelGGL((prefix_mfma_kernel<E, 2>), grid, block, tile_lds_bytes<2>(), st, a, mtiles);
+    hipExtLaunchKernelGGL((prefix_mfma_kernel<E, 2>), grid, block, tile_lds_bytes<2>(), st, ev.start, ev.stop, 0, a, mtiles);
   }
   return launch_status();
 }
