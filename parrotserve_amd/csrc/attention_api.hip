@@ -479,8 +479,7 @@ extern "C" int ph_prefill_attention(void* out, const void* q, const void* k_cach
     pa.num_chunks = (int)num_chunks;
     pa.H = H;
     pa.scale_log2e = scale * kLog2e;
-    const int64_t max_tiles = num_tokens / 64 + num_chunks;
-    return launch_prefill_mfma(pa, dtype, D, (int)max_tiles, st);
+    return launch_prefill_mfma(pa, dtype, D, num_tokens, st);
   }
   int64_t* offsets = (int64_t*)workspace;
   int32_t* lens = (int32_t*)((char*)workspace + round_up(num_tokens * 8, 256));

@@ -38,6 +38,7 @@ struct Elem<F16> {
   }
   static __device__ __forceinline__ float one(uint16_t b) { return (float)__builtin_bit_cast(_Float16, b); }
   static __device__ __forceinline__ uint16_t bits(float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }
+  static constexpr uint32_t kOnes = 0x3C003C00u;  // (1.0, 1.0)
   // acc + a.lo*b.lo + a.hi*b.hi with fp32 accumulate (v_dot2_f32_f16)
   static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float acc) {
     return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, a), __builtin_bit_cast(half2_t, b), acc, false);
@@ -52,6 +53,7 @@ struct Elem<BF16> {
   static __device__ __forceinline__ uint16_t bits(float f) {  // round to nearest even
     return __builtin_bit_cast(uint16_t, (__bf16)f);
   }
+  static constexpr uint32_t kOnes = 0x3F803F80u;  // (1.0, 1.0)
   static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float acc) {
     return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), acc, false);
   }

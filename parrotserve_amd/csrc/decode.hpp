@@ -104,8 +104,8 @@ struct PrefillArgs {
 };
 
 int launch_partial(const PartialArgs& a, int dtype, int D, hipStream_t st);
-// MFMA prefill: grid (head, query tile); max_tiles bounds the tile count (sum of ceil(n_c / 64)).
-int launch_prefill_mfma(const PrefillArgs& a, int dtype, int D, int max_tiles, hipStream_t st);
+// MFMA prefill: grid (head, query tile); num_tokens = total query rows (bounds the tile count).
+int launch_prefill_mfma(const PrefillArgs& a, int dtype, int D, int64_t num_tokens, hipStream_t st);
 int launch_items(const ItemArgs& a, int dtype, int D, hipStream_t st);
 int launch_merge(const MergeArgs& a, int dtype, int D, hipStream_t st);
 int launch_clear_ml(float* ml, int64_t entries, hipStream_t st);

@@ -1,15 +1,16 @@
-// Shared-prefix flash-decoding on CDNA4 matrix cores.
+// Shared-prefix flash-decoding and prefill with parent context on CDNA4 matrix cores.
 //
-// All queries of a group attend over the SAME prefix slots, so per head the
-// phase is a dense contraction: S^T = K Q^T (tokens x queries), O^T = V^T P^T.
-// Workgroup = (split of the prefix, head, group x 64-query tile), 4 waves.
-// Each wave owns every fourth 32-token tile of the split and ALL queries of
-// the tile, so each K/V byte is fetched from HBM once per (group, query tile)
-// and crosses LDS once: global -> wave-private LDS tile (coalesced 128-bit gathers by slot, written
-// by the load itself, double-buffered) -> MFMA operand layout.  No workgroup barrier in
-// the main loop.  Online softmax in the exp2 domain, fp32 accumulation in
-// v_mfma_f32_32x32x16_{f16,bf16}.  The four waves' partials are folded through
-// LDS at the end and one (O, m, l) part per (split, request, head) is written.
+// All queries of a group attend over the SAME prefix slots (decode), and all query rows of a prefill
+// chunk over the same parent + own slots, so per head the work is a dense contraction:
+// S^T = K Q^T (tokens x queries), O^T = V^T P^T, online softmax in the exp2 domain between them, fp32
+// accumulation in v_mfma_f32_32x32x16_{f16,bf16}.  K/V rows are gathered by slot straight from global
+// memory into XOR-swizzled LDS tiles (the load writes LDS itself, no register staging) and read back in
+// matrix-operand layout, so each K/V byte crosses LDS once.  Two forms of the tile loop:
+//   * four waves, one 32-query block (groups of up to 32 requests): every wave owns every fourth
+//     32-token tile in a private double-buffered LDS region, no workgroup barrier in the loop;
+//   * eight waves (two per SIMD), 64 to 256 queries per workgroup: the waves of a token group share each
+//     K/V tile through a ring of LDS stages, one barrier per step (attn_tile8 below).
+// Partials of the waves that split the tokens are folded through LDS at the end.
 //
 // Operand layouts (lane = 32*h + r):
 //   A (32 x 16): lane holds row r, 8 contraction elements chosen by (h, step)
@@ -79,6 +80,7 @@ struct TileWork {
   int64_t q_stride;
   int nq;                 // live queries in the tile
   const int32_t* slots;   // slot list base
+  int slots_len;          // entries of the list (reads beyond [s0, s1) are clamped to it)
   int s0, s1;             // token range of this workgroup
   int causal_off;         // CAUSAL: query i sees token t iff t <= causal_off + i
 };
@@ -406,6 +408,7 @@ __global__ __launch_bounds__(256, 1) void prefix_mfma_kernel(PrefixArgs a, int m
   wk.q_stride = a.q_stride;
   wk.nq = nq;
   wk.slots = a.slots + poff;
+  wk.slots_len = plen;
   wk.s0 = s0;
   wk.s1 = s1;
   wk.causal_off = 0;
@@ -433,17 +436,400 @@ __global__ __launch_bounds__(256, 1) void prefix_mfma_kernel(PrefixArgs a, int m
   }
 }
 
-// Prefill with parent context: workgroup = (head, 64-query tile of one chunk), all of the tile's
-// visible keys (ancestors, then the chunk's own tokens up to the diagonal); writes the final rows.
-// blockIdx.x is the head so that the query tiles of one (chunk, head), which stream the same K/V,
-// land on the same XCD (workgroups go round-robin over the 8 XCDs in linear order) and share its L2.
+// ---------------------------------------------------------------------------------------------------------
+// Eight-wave form of the tile.  The workgroup's eight waves are TQ token groups x QB = 8 / TQ query blocks:
+// wave (g, qb) works on every TQ-th 32-token tile (those with index = g mod TQ) for queries 32 qb .. 32 qb + 31,
+// so a workgroup covers 32 QB queries.  The QB waves of a token group share each K/V tile: every wave stages
+// 16 / QB of the tile's sixteen 1 KB row groups into the group's ring of 8 / TQ LDS stages (7, 3 or 1 tiles
+// in flight ahead of the one being multiplied), and one workgroup barrier per step publishes the parts to
+// each other (all waves run the same trip count).  Two waves per SIMD: one wave's softmax arithmetic overlaps
+// the other's matrix instructions, and at 256 registers per lane every matrix operand and result stays in
+// ordinary vector registers.  Slot ids come from a 4096-token window of the slot list kept in LDS (refilled
+// by the whole workgroup when the staging front crosses it), so the only vector-memory operations in the
+// loop are the LDS-direct row loads and their completion can be counted exactly.
+// On return wave (g, qb) holds 4 / TQ blocks of 32 dims, [32 (4/TQ) g, +32 (4/TQ)), of its queries, folded
+// over the token groups (register 4j+i of block n = dim 32 ((4/TQ) g + n) + 8j + 4h + i of query 32 qb + ql).
+constexpr int kWin = 4096;                        // tokens per slot window
+constexpr int kWinOff = 8 * kStage;               // LDS offset of the window (behind the 128 KB of stages)
+constexpr int kMlOff = kWinOff + kWin * 4;        // (m, l, true max) of eight waves for the fold
+constexpr int kTile8Lds = kMlOff + 8 * 3 * 256;
+
+// max over the two 32-lane halves of the wave: lane l gets max(x[l], x[l ^ 32]).  One lane-swap instruction
+// (lanes 32..63 of the first register trade places with lanes 0..31 of the second) instead of a trip
+// through LDS; written as assembly because the builtin's second result is mis-compiled by this toolchain.
+__device__ __forceinline__ float half_swap_max(float x) {
+  float a = x, b = x;
+  asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+  return fmaxf(a, b);
+}
+
+// LDS reads by byte address (the ring's stage offset then folds into the instruction's immediate)
+__device__ __forceinline__ u32x4 lds_ld16_a(uint32_t addr) {
+  return *reinterpret_cast<const u32x4 __attribute__((address_space(3)))*>((uintptr_t)addr);
+}
+__device__ __forceinline__ u32x2 lds_tr16_a(uint32_t addr) {
+  const short4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      reinterpret_cast<short4_t __attribute__((address_space(3)))*>((uintptr_t)addr));
+  return __builtin_bit_cast(u32x2, v);
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {  // vmcnt <= N, other counters untouched (gfx9 encoding)
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+template <typename E, bool CAUSAL, int TQ>
+__device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* __restrict__ kc,
+                                           const uint16_t* __restrict__ vc, int64_t row_stride, int head,
+                                           float scale_log2e, char* smem, float16_t (&ofold)[4 / TQ], float& mfin,
+                                           float& lfin) {
+  constexpr int QB = 8 / TQ;      // query blocks = waves sharing a tile
+  constexpr int NST = 8 / TQ;     // stages per token group
+  constexpr int A = NST - 1;      // tiles in flight ahead of the current one
+  constexpr int LPT = 16 / QB;    // row-group loads per wave per tile
+  constexpr int NDB = 4 / TQ;     // dim blocks a wave finishes
+  constexpr float kSlack = 8.f;
+  float16_t oacc[4];
+  float m = -INFINITY, lsum = 0.f, mtrue = -INFINITY;
+  const int lane = threadIdx.x & 63;
+  const int w8 = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), g = w8 / QB, qb = w8 % QB;
+  const int h = lane >> 5, ql = lane & 31;
+  char* gl = smem + g * NST * kStage;
+  int32_t* win = reinterpret_cast<int32_t*>(smem + kWinOff);
+  const int s0 = wk.s0, s1 = wk.s1;
+#pragma unroll
+  for (int db = 0; db < 4; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) oacc[db][r] = 0.f;
+
+  // slot window [win0, win0 + kWin) of the list, clamped to the list's end
+  int win0 = s0;
+  auto fill_window = [&]() {
+    for (int i = threadIdx.x; i < kWin; i += 512) win[i] = wk.slots[min(win0 + i, wk.slots_len - 1)];
+  };
+  fill_window();
+
+  // staging: row group L (0..7 K, 8..15 V) covers tokens 4 (L & 7) .. +3, 16 lanes per token row; this wave
+  // brings row groups qb LPT .. + LPT - 1 (same swizzles as the four-wave form)
+  const int tl = lane >> 4, c = lane & 15;
+  const uint32_t row_bytes = (uint32_t)(row_stride * 2);
+  const bool isv = qb * LPT >= 8;
+  const int r0 = (qb * LPT) & 7;
+  const char* gbase[LPT];
+#pragma unroll
+  for (int i = 0; i < LPT; ++i)
+    gbase[i] = isv ? reinterpret_cast<const char*>(vc + (int64_t)head * kPD + ((c ^ (4 * tl)) * 8))
+                   : reinterpret_cast<const char*>(kc + (int64_t)head * kPD + ((c ^ ((4 * (r0 + i) + tl) & 15)) * 8));
+  const uint32_t dst0 = lds_addr_of(gl) + (isv ? kVtOff : 0) + r0 * 1024;
+  // rows of the group's tile that starts at token tb, into ring stage `stage`
+  auto fetch_rows = [&](int tb, int stage) {
+    uint32_t sl[LPT];
+#pragma unroll
+    for (int i = 0; i < LPT; ++i) sl[i] = (uint32_t)win[tb - win0 + 4 * (r0 + i) + tl];
+    const uint32_t kb = dst0 + stage * kStage;
+#pragma unroll
+    for (int i = 0; i < LPT; ++i) lds_dma16(gbase[i] + (uint64_t)sl[i] * row_bytes, kb + i * 1024);
+  };
+  const int ntile = (s1 - s0 + kTile - 1) / kTile;
+  const int iters = (ntile + TQ - 1) / TQ;                 // same for all eight waves
+  const int my_iters = ntile > g ? (ntile - g + TQ - 1) / TQ : 0;  // tiles of this token group
+  __syncthreads();                                         // window visible
+#pragma unroll
+  for (int j = 0; j < A; ++j)
+    if (j < my_iters) fetch_rows(s0 + kTile * (g + TQ * j), j);
+
+  // Q as the B operand: column = query 32 qb + ql, contraction chunk (h, s) = dims 64h + 8s .. +8
+  u32x4 qop[8];
+  {
+    const int q = 32 * qb + ql;
+    const bool ok = q < wk.nq;
+    const uint16_t* qp = wk.qrow0 + (int64_t)(ok ? q : 0) * wk.q_stride + 64 * h;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      u32x4 v = ld16(qp + 8 * s);
+      if (!ok) v = u32x4{0, 0, 0, 0};
+      qop[s] = v;
+    }
+  }
+  // last token any query of this wave's block may see (none if the block has no live query)
+  const int wave_last = 32 * qb >= wk.nq ? -1 : CAUSAL ? min(s1 - 1, wk.causal_off + 32 * qb + 31) : s1 - 1;
+
+  // Operand read addresses of ring stage 0 (and of stage 4, beyond the reach of the 16-bit immediate).
+  // K: row ql, chunk (8h + s) swizzled by the row; V: the transposing read's row/column of this lane.
+  constexpr int NHI = NST > 4 ? 2 : 1;
+  uint32_t kaddr[NHI][8], vaddr[NHI][4];
+  {
+    const uint32_t gl_a = lds_addr_of(gl);
+    const int sl = lane & 15, rh = (lane >> 4) & 1;
+    const int trow = 4 * h + (sl >> 2);                       // + 16u + 8x
+    const int tcol = 2 * rh + ((sl & 3) >> 1);                // + 4db, in 16-byte chunks
+    const int tswz = 4 * (sl >> 2);                           // = 4 * (row & 3)
+#pragma unroll
+    for (int hi = 0; hi < NHI; ++hi) {
+#pragma unroll
+      for (int s = 0; s < 8; ++s) {
+        kaddr[hi][s] = gl_a + hi * 4 * kStage + ql * 256 + (((8 * h + s) ^ (ql & 15)) * 16);
+        asm("" : "+v"(kaddr[hi][s]));  // keep the sum in one register (otherwise it is re-added at every read)
+      }
+#pragma unroll
+      for (int db = 0; db < 4; ++db) {
+        vaddr[hi][db] = gl_a + hi * 4 * kStage + kVtOff + trow * 256 + (sl & 1) * 8 + (((4 * db + tcol) ^ tswz) * 16);
+        asm("" : "+v"(vaddr[hi][db]));
+      }
+    }
+  }
+  // the ring position is a compile-time constant in the unrolled inner loop, so every LDS address of a
+  // step is a fixed register plus an immediate offset
+  for (int it0 = 0; it0 < iters; it0 += NST) {
+#pragma unroll
+   for (int stage = 0; stage < NST; ++stage) {
+    const int it = it0 + stage;
+    if (it >= iters) break;
+    const int tb = s0 + kTile * (g + TQ * it);
+    // Tile `it` of this group has landed once at most the (A - 1) LPT loads issued after it are outstanding
+    // (near the end fewer were issued, so everything is awaited); the barrier publishes all parts of the
+    // tile and tells everyone that the stage read in the previous step is free again.
+    if (it + A - 1 < my_iters) wait_vmcnt<(A - 1) * LPT>(); else wait_vmcnt<0>();
+    __syncthreads();
+    {
+      const int front = s0 + kTile * TQ * (it + A);          // first token of the step being staged
+      if (front < s1 && front >= win0 + kWin) {              // workgroup-uniform: slide the slot window
+        win0 += kWin;
+        fill_window();
+        __syncthreads();
+      }
+      if (it + A < my_iters) fetch_rows(front + kTile * g, (stage + A) % NST);
+    }
+    if (it >= my_iters || tb > wave_last) continue;           // wave-uniform
+    const int shi = stage >> 2, slo = (stage & 3) * kStage;
+
+    u32x4 ka[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s) ka[s] = lds_ld16_a(kaddr[shi][s] + slo);
+    __builtin_amdgcn_sched_barrier(0);
+    float16_t sacc;
+    {
+      const float16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      sacc = Mfma32<E>::run(ka[0], qop[0], zero);
+#pragma unroll
+      for (int s = 1; s < 8; ++s) sacc = Mfma32<E>::run(ka[s], qop[s], sacc);
+    }
+    // A operand of O^T += V^T P^T (row = dim 32db + ql, contraction = the 8 tokens of (h, u)): two
+    // transposing reads, tokens 16u + 4h + {0..3} and 16u + 8 + 4h + {0..3}
+    u32x4 va[4][2];
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const u32x2 lo = lds_tr16_a(vaddr[shi][db] + slo + (16 * u) * 256);
+        const u32x2 hi = lds_tr16_a(vaddr[shi][db] + slo + (16 * u + 8) * 256);
+        va[db][u] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+      }
+    __builtin_amdgcn_sched_barrier(0);
+
+    const bool full = tb + kTile <= s1 && (!CAUSAL || tb + kTile - 1 <= wk.causal_off + 32 * qb);
+    float x[16];
+    if (full) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) x[r] = sacc[r];
+    } else {
+      const int tmax = CAUSAL ? min(s1 - 1, wk.causal_off + 32 * qb + ql) : s1 - 1;  // last visible token
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int t = 8 * (r >> 2) + 4 * h + (r & 3);
+        x[r] = (tb + t <= tmax) ? sacc[r] : -INFINITY;
+      }
+    }
+    float mloc = fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3]));
+#pragma unroll
+    for (int r = 4; r < 16; r += 4) mloc = fmaxf(mloc, fmaxf(fmaxf(x[r], x[r + 1]), fmaxf(x[r + 2], x[r + 3])));
+    mloc = half_swap_max(mloc) * scale_log2e;  // scale > 0 keeps the order
+    mtrue = fmaxf(mtrue, mloc);
+    // lazy exponent reference: moves only when the maximum has outgrown it by more than kSlack
+    const bool move = mloc > m + kSlack;
+    const float mnew = move ? mloc : m;
+    const float mref = (mnew == -INFINITY) ? 0.f : mnew;
+    const bool had = m != -INFINITY;
+    const float alpha = (move && had) ? __builtin_amdgcn_exp2f(m - mref) : 1.f;
+    m = mnew;
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {  // wave-uniform, rare
+      // pinned in assembly so that the multiply stays inside this branch; wait states cover the matrix
+      // results being read by the vector ALU and the rewritten registers feeding the next C operand
+      asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) asm volatile("v_mul_f32 %0, %0, %1" : "+v"(oacc[db][r]) : "v"(alpha));
+      asm volatile("s_nop 7" ::: "memory");
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) x[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(x[r], scale_log2e, -mref));
+    // P^T packed straight into B-operand form; the denominator sums the rounded values the product uses
+    float ps = 0.f;
+    u32x4 pop[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        pop[u][e] = pack2<E>(x[8 * u + 2 * e], x[8 * u + 2 * e + 1]);
+        ps = Elem<E>::dot2(pop[u][e], Elem<E>::kOnes, ps);
+      }
+    lsum = lsum * alpha + ps;
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int u = 0; u < 2; ++u) oacc[db] = Mfma32<E>::run(va[db][u], pop[u], oacc[db]);
+   }
+  }
+
+  if constexpr (TQ == 1) {
+    // one token group: nothing to fold across waves
+    const float Lall = lsum + __shfl_xor(lsum, 32, kWave);
+    const float toTrue = (mtrue == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m - mtrue);
+    mfin = mtrue;
+    lfin = Lall * toTrue;
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) ofold[db][r] = oacc[db][r] * toTrue;
+  } else {
+    // Fold the token groups of each query block: every wave parks the dim blocks it does not finish, and
+    // its (m, l, true max); after one barrier wave (g, qb) folds blocks [NDB g, NDB g + NDB) of its block.
+    constexpr int kBlk = 16 * 256;                  // one parked block: 16 floats x 64 lanes
+    char* fb = smem + qb * (TQ * 4) * kBlk;         // [source group][dim block]
+    char* mlb = smem + kMlOff + qb * TQ * 3 * 256;  // [group][m, l, true max][lane] floats
+    __syncthreads();                                // the staging tiles are dead from here on
+#pragma unroll
+    for (int db = 0; db < 4; ++db) {
+      if (db / NDB == g) continue;
+      char* base = fb + (g * 4 + db) * kBlk + lane * 16;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float4_t v = {oacc[db][4 * j], oacc[db][4 * j + 1], oacc[db][4 * j + 2], oacc[db][4 * j + 3]};
+        *reinterpret_cast<float4_t*>(base + j * 1024) = v;
+      }
+    }
+    *reinterpret_cast<float*>(mlb + (g * 3 + 0) * 256 + lane * 4) = m;
+    *reinterpret_cast<float*>(mlb + (g * 3 + 1) * 256 + lane * 4) = lsum;
+    *reinterpret_cast<float*>(mlb + (g * 3 + 2) * 256 + lane * 4) = mtrue;
+    __syncthreads();
+    float ms[TQ], ls[TQ];
+    float M = -INFINITY, mt = -INFINITY;
+#pragma unroll
+    for (int src = 0; src < TQ; ++src) {
+      ms[src] = *reinterpret_cast<const float*>(mlb + (src * 3 + 0) * 256 + lane * 4);
+      ls[src] = *reinterpret_cast<const float*>(mlb + (src * 3 + 1) * 256 + lane * 4);
+      mt = fmaxf(mt, *reinterpret_cast<const float*>(mlb + (src * 3 + 2) * 256 + lane * 4));
+      M = fmaxf(M, ms[src]);
+    }
+    float L = 0.f;
+#pragma unroll
+    for (int n = 0; n < NDB; ++n)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) ofold[n][r] = 0.f;
+#pragma unroll
+    for (int src = 0; src < TQ; ++src) {
+      const float sc = (ms[src] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(ms[src] - M);
+      L += ls[src] * sc;
+#pragma unroll
+      for (int n = 0; n < NDB; ++n) {
+        if (src == g) {
+          // the blocks this wave kept in registers (static register index per candidate g)
+#pragma unroll
+          for (int db = 0; db < 4; ++db)
+            if (db == NDB * g + n) {
+#pragma unroll
+              for (int r = 0; r < 16; ++r) ofold[n][r] += oacc[db][r] * sc;
+            }
+        } else {
+          const char* base = fb + (src * 4 + NDB * g + n) * kBlk + lane * 16;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float4_t v = *reinterpret_cast<const float4_t*>(base + j * 1024);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) ofold[n][4 * j + i] += v[i] * sc;
+          }
+        }
+      }
+    }
+    // report the true maximum, with the denominator re-expressed relative to it
+    const float Lall = L + __shfl_xor(L, 32, kWave);
+    const float toTrue = (mt == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(M - mt);
+    mfin = mt;
+    lfin = Lall * toTrue;
+#pragma unroll
+    for (int n = 0; n < NDB; ++n)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) ofold[n][r] *= toTrue;
+  }
+}
+
+// Shared-prefix phase, eight waves: workgroup = (split, head, group x 64-query tile)
 template <typename E>
-__global__ __launch_bounds__(256, 1) void prefill_mfma_kernel(PrefillArgs a) {
+__global__ __launch_bounds__(512) void prefix_mfma8_kernel(PrefixArgs a, int mtiles) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int split = blockIdx.x, head = blockIdx.y;
+  const int g = blockIdx.z / mtiles, mt = blockIdx.z - g * mtiles;
+  int r0 = 0, r1 = a.B, poff = 0, plen = a.fixed_prefix_len;
+  if (a.prefix_cu) {
+    r0 = a.group_req_cu[g];
+    r1 = a.group_req_cu[g + 1];
+    poff = a.prefix_cu[g];
+    plen = a.prefix_cu[g + 1] - poff;
+  }
+  const int qbase = r0 + mt * 64;
+  const int nq = min(64, r1 - qbase);
+  if (nq <= 0) return;
+  const int s0 = split * a.split_tokens;
+  const int s1 = min(plen, s0 + a.split_tokens);
+  if (s0 >= plen) {  // this group's prefix ends before the split: mark the part empty
+    for (int q = threadIdx.x; q < nq; q += 512) {
+      const int64_t pr = ((int64_t)split * a.B + qbase + q) * a.H + head;
+      a.ml[pr * 2] = -INFINITY;
+      a.ml[pr * 2 + 1] = 0.f;
+    }
+    return;
+  }
+  TileWork wk;
+  wk.qrow0 = a.q + (int64_t)qbase * a.q_stride + head * kPD;
+  wk.q_stride = a.q_stride;
+  wk.nq = nq;
+  wk.slots = a.slots + poff;
+  wk.slots_len = plen;
+  wk.s0 = s0;
+  wk.s1 = s1;
+  wk.causal_off = 0;
+  float16_t of[1];
+  float m, l;
+  attn_tile8<E, false, 4>(wk, a.kc, a.vc, a.row_stride, head, a.scale_log2e, smem, of, m, l);
+  const int lane = threadIdx.x & 63, w8 = threadIdx.x >> 6, tq = w8 >> 1, qh = w8 & 1, h = lane >> 5, ql = lane & 31;
+  const int q = 32 * qh + ql;
+  if (q < nq) {
+    const float inv = 1.f / l;
+    const int64_t pr = ((int64_t)split * a.B + qbase + q) * a.H + head;
+    float* op = a.opart + pr * kPD + 32 * tq + 4 * h;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float4_t v = {of[0][4 * j] * inv, of[0][4 * j + 1] * inv, of[0][4 * j + 2] * inv, of[0][4 * j + 3] * inv};
+      *reinterpret_cast<float4_t*>(op + 8 * j) = v;
+    }
+    if (h == 0 && tq == 0) {
+      a.ml[pr * 2] = m;
+      a.ml[pr * 2 + 1] = l;
+    }
+  }
+}
+
+// Prefill with parent context, eight waves: workgroup = (head, tile of 32 * (8 / TQ) queries of one chunk)
+template <typename E, int TQ>
+__global__ __launch_bounds__(512) void prefill_mfma8_kernel(PrefillArgs a) {
+  constexpr int QB = 8 / TQ, NDB = 4 / TQ, QT = 32 * QB;
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const int head = blockIdx.x;
-  const int ti = blockIdx.y;
   if (head >= a.H) return;
-  if (ti >= a.tile_cu[a.num_chunks]) return;
+  if ((int)blockIdx.y >= a.tile_cu[a.num_chunks]) return;
+  // later tiles of a chunk see more keys: hand them out first so the launch does not end on the longest ones
+  const int ti = a.tile_cu[a.num_chunks] - 1 - blockIdx.y;
   int lo = 0, hi = a.num_chunks;  // chunk with tile_cu[c] <= ti < tile_cu[c+1]
   while (hi - lo > 1) {
     const int mid = (lo + hi) >> 1;
@@ -451,30 +837,31 @@ __global__ __launch_bounds__(256, 1) void prefill_mfma_kernel(PrefillArgs a) {
   }
   const int cq0 = a.q_cu[lo], n = a.q_cu[lo + 1] - cq0;
   const int kv0 = a.kv_cu[lo], kvn = a.kv_cu[lo + 1] - kv0;
-  const int q0 = (ti - a.tile_cu[lo]) * 64;
-  const int nq = min(64, n - q0);
+  const int q0 = (ti - a.tile_cu[lo]) * QT;
+  const int nq = min(QT, n - q0);
   TileWork wk;
   wk.qrow0 = a.q + (int64_t)(cq0 + q0) * a.q_stride + head * kPD;
   wk.q_stride = a.q_stride;
   wk.nq = nq;
   wk.slots = a.ctx_slots + kv0;
+  wk.slots_len = kvn;
   wk.s0 = 0;
   wk.causal_off = kvn - n + q0;
   wk.s1 = min(kvn, wk.causal_off + nq);  // the last live query sees tokens up to causal_off + nq - 1
-  float16_t of[2];
-  float m[2], l[2];
-  attn_tile<E, 2, true>(wk, a.kc, a.vc, a.row_stride, head, a.scale_log2e, smem, of, m, l);
-  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, h = lane >> 5, ql = lane & 31;
+  float16_t of[NDB];
+  float m, l;
+  attn_tile8<E, true, TQ>(wk, a.kc, a.vc, a.row_stride, head, a.scale_log2e, smem, of, m, l);
+  const int lane = threadIdx.x & 63, w8 = threadIdx.x >> 6, g = w8 / QB, qb = w8 % QB, h = lane >> 5, ql = lane & 31;
+  const int q = 32 * qb + ql;
+  if (q < nq) {
+    const float inv = l > 0.f ? 1.f / l : 0.f;
 #pragma unroll
-  for (int nb = 0; nb < 2; ++nb) {
-    const int q = 32 * nb + ql;
-    if (q < nq) {
-      const float inv = l[nb] > 0.f ? 1.f / l[nb] : 0.f;
-      uint16_t* op = a.out + (int64_t)(cq0 + q0 + q) * a.out_stride + head * kPD + 32 * w + 4 * h;
+    for (int nd = 0; nd < NDB; ++nd) {
+      uint16_t* op = a.out + (int64_t)(cq0 + q0 + q) * a.out_stride + head * kPD + 32 * (NDB * g + nd) + 4 * h;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        u32x2 v = {pack2<E>(of[nb][4 * j] * inv, of[nb][4 * j + 1] * inv),
-                   pack2<E>(of[nb][4 * j + 2] * inv, of[nb][4 * j + 3] * inv)};
+        u32x2 v = {pack2<E>(of[nd][4 * j] * inv, of[nd][4 * j + 1] * inv),
+                   pack2<E>(of[nd][4 * j + 2] * inv, of[nd][4 * j + 3] * inv)};
         *reinterpret_cast<u32x2*>(op + 8 * j) = v;
       }
     }
@@ -482,42 +869,54 @@ __global__ __launch_bounds__(256, 1) void prefill_mfma_kernel(PrefillArgs a) {
 }
 
 // tile_cu[c] = number of 64-query tiles before chunk c (serial scan; chunk counts are small)
-__global__ void prefill_tiles_kernel(const int32_t* q_cu, int num_chunks, int32_t* tile_cu) {
+__global__ void prefill_tiles_kernel(const int32_t* q_cu, int num_chunks, int32_t* tile_cu, int tile_q) {
   if (threadIdx.x != 0 || blockIdx.x != 0) return;
   int acc = 0;
   for (int c = 0; c < num_chunks; ++c) {
     tile_cu[c] = acc;
-    acc += (q_cu[c + 1] - q_cu[c] + 63) / 64;
+    acc += (q_cu[c + 1] - q_cu[c] + tile_q - 1) / tile_q;
   }
   tile_cu[num_chunks] = acc;
 }
 
 template <typename E>
 static int launch_prefix_t(const PrefixArgs& a, int num_groups, int max_group_reqs, hipStream_t st) {
-  const int nqb = max_group_reqs <= 32 ? 1 : 2;
-  const int mtiles = (max_group_reqs + 32 * nqb - 1) / (32 * nqb);
-  dim3 grid(a.n_splits, a.H, num_groups * mtiles), block(256);
   const KernelEvents ev = take_kernel_events(0);
-  if (nqb == 1) {
+  if (max_group_reqs <= 32) {  // four waves, one 32-query block
+    dim3 grid(a.n_splits, a.H, num_groups), block(256);
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefix_mfma_kernel<E, 1>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, tile_lds_bytes<1>());
-    hipExtLaunchKernelGGL((prefix_mfma_kernel<E, 1>), grid, block, tile_lds_bytes<1>(), st, ev.start, ev.stop, 0, a, mtiles);
-  } else {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefix_mfma_kernel<E, 2>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, tile_lds_bytes<2>());
-    hipExtLaunchKernelGGL((prefix_mfma_kernel<E, 2>), grid, block, tile_lds_bytes<2>(), st, ev.start, ev.stop, 0, a, mtiles);
+    hipExtLaunchKernelGGL((prefix_mfma_kernel<E, 1>), grid, block, tile_lds_bytes<1>(), st, ev.start, ev.stop, 0, a, 1);
+  } else {                     // eight waves, 64-query tiles
+    const int mtiles = (max_group_reqs + 63) / 64;
+    dim3 grid(a.n_splits, a.H, num_groups * mtiles), block(512);
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefix_mfma8_kernel<E>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, kTile8Lds);
+    hipExtLaunchKernelGGL((prefix_mfma8_kernel<E>), grid, block, kTile8Lds, st, ev.start, ev.stop, 0, a, mtiles);
   }
   return launch_status();
 }
 
-template <typename E>
-static int launch_prefill_t(const PrefillArgs& a, int max_tiles, hipStream_t st) {
-  hipLaunchKernelGGL(prefill_tiles_kernel, dim3(1), dim3(64), 0, st, a.q_cu, a.num_chunks, a.tile_cu);
-  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_mfma_kernel<E>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, tile_lds_bytes<2>());
+template <typename E, int TQ>
+static int launch_prefill_tq(const PrefillArgs& a, int64_t num_tokens, hipStream_t st) {
+  constexpr int QT = 32 * (8 / TQ);  // queries per workgroup tile
+  hipLaunchKernelGGL(prefill_tiles_kernel, dim3(1), dim3(64), 0, st, a.q_cu, a.num_chunks, a.tile_cu, QT);
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_mfma8_kernel<E, TQ>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kTile8Lds);
   const int hx = (a.H + 7) / 8 * 8;  // keeps head == linear id mod 8 for every tile row
-  hipLaunchKernelGGL((prefill_mfma_kernel<E>), dim3(hx, max_tiles), dim3(256), tile_lds_bytes<2>(), st, a);
+  const int64_t max_tiles = num_tokens / QT + a.num_chunks;  // >= sum of ceil(n_c / QT)
+  hipLaunchKernelGGL((prefill_mfma8_kernel<E, TQ>), dim3(hx, (unsigned)max_tiles), dim3(512), kTile8Lds, st, a);
   return launch_status();
+}
+
+// Query tile by the average chunk length: 256-query tiles share every K/V tile among all eight waves (least
+// traffic, deepest staging ring) but idle whole waves on short chunks, which take 128- or 64-query tiles.
+template <typename E>
+static int launch_prefill_t(const PrefillArgs& a, int64_t num_tokens, hipStream_t st) {
+  const int64_t avg = num_tokens / (a.num_chunks > 0 ? a.num_chunks : 1);
+  if (avg >= 192) return launch_prefill_tq<E, 1>(a, num_tokens, st);
+  if (avg >= 96) return launch_prefill_tq<E, 2>(a, num_tokens, st);
+  return launch_prefill_tq<E, 4>(a, num_tokens, st);
 }
 
 bool prefix_mfma_supported(int dtype, int D) { return D == kPD && (dtype == PH_F16 || dtype == PH_BF16); }
@@ -529,10 +928,10 @@ int launch_prefix_mfma(const PrefixArgs& a, int dtype, int D, int num_groups, in
                          : launch_prefix_t<BF16>(a, num_groups, max_group_reqs, st);
 }
 
-int launch_prefill_mfma(const PrefillArgs& a, int dtype, int D, int max_tiles, hipStream_t st) {
+int launch_prefill_mfma(const PrefillArgs& a, int dtype, int D, int64_t num_tokens, hipStream_t st) {
   if (D != kPD) return PH_ERR_HEAD_DIM;
-  if (max_tiles <= 0) return PH_OK;
-  return dtype == PH_F16 ? launch_prefill_t<F16>(a, max_tiles, st) : launch_prefill_t<BF16>(a, max_tiles, st);
+  if (num_tokens <= 0 || a.num_chunks <= 0) return PH_OK;
+  return dtype == PH_F16 ? launch_prefill_t<F16>(a, num_tokens, st) : launch_prefill_t<BF16>(a, num_tokens, st);
 }
 
 }  // namespace ph

@@ -216,3 +216,75 @@ def test_balanced_and_grid_suffix_forms_agree(dev):
     torch.testing.assert_close(a.float(), ref.float(), **TOL[torch.float16])
     torch.testing.assert_close(b.float(), ref.float(), **TOL[torch.float16])
     torch.testing.assert_close(a.float(), b.float(), atol=1e-3, rtol=1e-2)
+
+
+def test_prefix_longer_than_slot_window(dev):
+    """Eight groups of 33 requests over 4200-token prefixes, 32 heads: enough workgroups that the planner
+    leaves each prefix in one split, so a workgroup walks more than the 4096 slot ids it keeps on chip."""
+    from parrotserve_amd import synth
+
+    g = torch.Generator().manual_seed(11)
+    s = torch.randint(1, 40, (8 * 33,), generator=g).tolist()
+    case = synth.make_decode_case("w", 11, torch.float16, 8, 33, 4200, s, 32, 128, 1 << 16)
+    _check(case, dev)
+
+
+def _split_halves_case(dtype, B, P, H, seed):
+    from parrotserve_amd import synth
+
+    g = torch.Generator().manual_seed(seed)
+    s = torch.randint(1, 150, (B,), generator=g).tolist()
+    s[0] = 0 if B > 1 else s[0]  # one request without a suffix
+    return synth.make_decode_case("halves", seed, dtype, 1, B, P, s, H, 128, 1 << 14)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("B,P,H", [(64, 700, 8), (20, 333, 4)])
+def test_prefix_and_post_entry_points(dev, dtype, B, P, H):
+    """The two halves exported separately, called through the C ABI the way the reference calls its Triton
+    prefix kernel (O, row max and denominator out) and then its post kernel (suffix + merge in place)."""
+    import ctypes
+
+    from parrotserve_amd import _lib, kernels, synth
+
+    case = _split_halves_case(dtype, B, P, H, 40 + B)
+    lib = _lib.load()
+    D = 128
+    kc, vc = synth.pool_to_device(case.k_rows, case.v_rows, case.used_slots, case.pool_slots, dev)
+    q = case.q.to(dev)
+    out = torch.zeros_like(q)
+    m = torch.empty((B, H), dtype=torch.float32, device=dev)
+    l = torch.empty((B, H), dtype=torch.float32, device=dev)
+    prefix = case.pool_lists(case.prefix_lists)[0]
+    pslots = torch.tensor(prefix, dtype=torch.int32, device=dev)
+    suffix = case.pool_lists(case.suffix_lists)
+    width = max(1, max(len(x) for x in suffix))
+    table = torch.zeros((B, width), dtype=torch.int32)
+    for i, x in enumerate(suffix):
+        table[i, : len(x)] = torch.tensor(x, dtype=torch.int32)
+    table = table.to(dev)
+    lens = torch.tensor([len(x) for x in suffix], dtype=torch.int32, device=dev)
+    nbytes = lib.ph_decode_workspace_bytes(B, H, D, 1, P, width, 0, 0)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    scale = D ** -0.5
+    st = torch.cuda.current_stream().cuda_stream
+    code = 0 if dtype == torch.float16 else 1
+    rc = lib.ph_prefix_attention(out.data_ptr(), m.data_ptr(), l.data_ptr(), q.data_ptr(), kc.data_ptr(), vc.data_ptr(),
+                                 B, H, D, code, q.stride(0), out.stride(0), kc.stride(0), scale,
+                                 pslots.data_ptr(), P, ws.data_ptr(), nbytes, st)
+    assert rc == 0
+    torch.cuda.synchronize()
+    # prefix half against the oracle's partial: normalised O, row max (exp2 domain) and denominator
+    ridx = [case.prefix_lists[0]] * B
+    o_ref, m_ref, l_ref = ref_partial(case.q, case.k_rows, case.v_rows, ridx, scale)
+    torch.testing.assert_close(out.cpu().float(), o_ref.float(), **TOL[dtype])
+    torch.testing.assert_close(m.cpu(), m_ref, atol=1e-3, rtol=1e-4)
+    torch.testing.assert_close(l.cpu(), l_ref, atol=1e-3, rtol=2e-2 if dtype == torch.bfloat16 else 5e-3)
+    rc = lib.ph_suffix_post_attention(out.data_ptr(), m.data_ptr(), l.data_ptr(), q.data_ptr(), kc.data_ptr(),
+                                      vc.data_ptr(), B, H, D, code, q.stride(0), out.stride(0), kc.stride(0), scale,
+                                      table.data_ptr(), None, table.stride(0), table.numel(), lens.data_ptr(),
+                                      width, 0, ws.data_ptr(), nbytes, st)
+    assert rc == 0
+    torch.cuda.synchronize()
+    ref = ref_decode_attention(case.q, case.k_rows, case.v_rows, case.full_lists())
+    torch.testing.assert_close(out.cpu().float(), ref.float(), **TOL[dtype])

@@ -112,3 +112,26 @@ def test_config4_full_size_property(dev):
     v_all = torch.cat([case.v_rows[case.parent_lists[0]], case.v_new[:n0]])
     ref0 = ref_prefill_with_parent(rq.view(n0, H, D), k_all, v_all, [n0], [torch.arange(k_all.shape[0])])
     torch.testing.assert_close(out[:n0].cpu().float(), ref0.float(), **TOL[torch.bfloat16])
+
+
+@pytest.mark.parametrize("q_lens,parent", [([260], 9000),          # average 260 -> 256-query tiles
+                                           ([40, 300], 5000),      # average 170 -> 128-query tiles
+                                           ([30, 64, 20], 4200)])  # average 38 -> 64-query tiles
+def test_prefill_long_parents_all_tile_sizes(dev, q_lens, parent):
+    """Parents longer than the 4096-token slot window the kernel keeps on chip (the window slides while the
+    staging ring runs ahead), for each of the three query-tile sizes the launcher picks by average chunk length."""
+    from parrotserve_amd import synth
+
+    case = synth.make_prefill_case("w", 5 + parent, torch.float16, q_lens, parent, 2, 128, 1 << 15)
+    out, ref = run_prefill_case(case, dev)
+    torch.testing.assert_close(out.float(), ref.float(), **TOL[torch.float16])
+
+
+def test_prefill_heads_not_multiple_of_eight_and_tail_tiles(dev):
+    """Head counts that leave part of the padded head axis empty, chunks that end inside every tile size."""
+    from parrotserve_amd import synth
+
+    for H, q_lens, parent in ((5, [257, 511, 193], 70), (9, [129, 100, 95], 33), (3, [65, 31, 96, 1], 200)):
+        case = synth.make_prefill_case("h", 900 + H, torch.bfloat16, q_lens, parent, H, 128, 1 << 13)
+        out, ref = run_prefill_case(case, dev)
+        torch.testing.assert_close(out.float(), ref.float(), **TOL[torch.bfloat16])
