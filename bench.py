@@ -190,6 +190,7 @@ def extras(torch, dev):
     del kc4, vc4, qkvs
     # --- config 5: full LLaMA-13B decoder layer, 4 prefix groups x 32 branches, prefix 6000 ------------------
     out["c5_layer"] = config5_layer(torch, dev)
+    out["c2_iteration_tables"] = iteration_tables_cost(torch, dev)
     # --- RMSNorm at a bandwidth-sized row count (LLaMA-13B hidden) -----------------------------------------
     xs = [torch.randn((8192, 5120), device=dev, dtype=torch.float16) for _ in range(8)]  # 8 x 84 MB, rotated
     w = torch.ones(5120, device=dev, dtype=torch.float16)
@@ -199,6 +200,57 @@ def extras(torch, dev):
     out["rms_norm_8192x5120"] = {"us": t * 1e6, "GB/s": nbytes / t / 1e9, "frac_hbm": nbytes / t / 1e9 / HBM_PEAK_GBS,
                                  "algorithmic_bytes": nbytes}
     return out
+
+
+def iteration_tables_cost(torch, dev):
+    """Host time per decode iteration of producing the device index tables (slot tables, lengths, suffix plan)
+    for config 2's batch, 64 Generate jobs forked from one 4096-token parent, own contexts U[16,512]: rebuilt
+    from the context trees every iteration as the reference does (attn_func.py:462-599), against patched in
+    place by the table cache (one appended slot per request)."""
+    from parrotserve_amd.attn_func import BuiltinConfig, HipGroupedPrefixAttn
+    from parrotserve_amd.context import BlockContext, RecyclePool
+    from parrotserve_amd.iter_state import IterationState
+    from parrotserve_amd.primitive_job import Generate
+    from parrotserve_amd.table_cache import DecodeTableCache
+
+    class Cfg:
+        num_attention_heads, hidden_size = 32, 4096
+
+    class Inc(HipGroupedPrefixAttn):
+        table_cache = DecodeTableCache()
+
+    class Fresh(HipGroupedPrefixAttn):
+        incremental = False
+
+    gen = torch.Generator().manual_seed(1)
+    lens = torch.randint(16, 513, (64,), generator=gen).tolist()
+    res = {"jobs": 64}
+    for label, cls in (("full_rebuild_us", Fresh), ("incremental_us", Inc)):
+        pool = RecyclePool(pool_size=1 << 20)
+        parent = BlockContext(0, None, pool, 1)
+        parent.allocate(4096)
+        jobs = []
+        for b, n in enumerate(lens):
+            c = BlockContext(1 + b, parent, pool, 1)
+            c.allocate(n)
+            j = Generate(0, b, c.context_id, parent.context_id, sampling_config=None)
+            j.context = c
+            jobs.append(j)
+        cfg = BuiltinConfig(num_kv_cache_blocks=1 << 20, attn_func=cls, dtype=torch.float16, device=dev)
+        ts = []
+        for it in range(24):
+            for j in jobs:
+                j.context.allocate(1)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            IterationState(jobs, Cfg, cfg)
+            torch.cuda.synchronize()
+            ts.append(time.perf_counter() - t0)
+        ts = sorted(ts[4:])
+        res[label] = ts[len(ts) // 2] * 1e6
+        res["sum_context"] = sum(j.context.get_context_len() for j in jobs)
+    res["speedup"] = res["full_rebuild_us"] / res["incremental_us"]
+    return res
 
 
 def config5_layer(torch, dev):

@@ -247,6 +247,19 @@ int ph_prefill_attention(void* out, const void* q, const void* k_cache, const vo
                          void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------ */
+/* Incremental suffix tables.  The reference rebuilds paged_block_tables /
+ * paged_context_lens from Python lists and uploads them every iteration
+ * (parrot/engine/builtin/attn_func.py:523-531,553-569); between two decode
+ * iterations of the same batch each request's list only gains the slot of the
+ * token being generated, so the device tables are patched instead:
+ *   table[rows[i] * table_stride + lens[rows[i]]] = new_slots[i];  lens[rows[i]] += 1
+ * for i < n.  rows (DEVICE int32, unique; NULL = identity) maps the caller's
+ * request order to table rows; a row that is already table_stride long is left
+ * untouched (the caller widens the table first).  All pointers DEVICE. */
+int ph_suffix_tables_append(int32_t* table, int64_t table_stride, int32_t* lens, const int32_t* rows,
+                            const int32_t* new_slots, int64_t n, void* stream);
+
+/* ------------------------------------------------------------------------ */
 /* Instrumentation (no counterpart in the reference, which times whole
  * iterations from Python, parrot/engine/builtin/builtin_runner.py:158-175).
  * Arms the NEXT ph_decode_attention call of the process: its prefix, suffix

@@ -33,6 +33,7 @@ SIGNATURES: Dict[str, Tuple[object, List[object]]] = {
     "ph_decode_attention": (I, [P, P, P, P, L, L, L, I, L, L, L, F, L, P, P, P, P, L, P, P, L, L, P, L, L, P, P, Z, P]),
     "ph_prefix_attention": (I, [P, P, P, P, P, P, L, L, L, I, L, L, L, F, P, L, P, Z, P]),
     "ph_suffix_post_attention": (I, [P, P, P, P, P, P, L, L, L, I, L, L, L, F, P, P, L, L, P, L, L, P, Z, P]),
+    "ph_suffix_tables_append": (I, [P, L, P, P, P, L, P]),
     "ph_arm_kernel_events": (I, [P]),
     "ph_prefill_workspace_bytes": (Z, [L, L, L, L]),
     "ph_prefill_attention": (I, [P, P, P, P, L, L, L, L, I, L, L, L, F, P, P, P, L, L, P, Z, P]),

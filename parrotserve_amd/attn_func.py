@@ -17,10 +17,12 @@ from __future__ import annotations
 import dataclasses
 from typing import Any, Dict, List, Optional, Sequence, Tuple
 
+import numpy as np
 import torch
 from torch import nn
 
 from . import kernels
+from .table_cache import DecodeTableCache
 from .mem import get_k_cache, get_v_cache
 from .primitive_job import Fill, Generate
 
@@ -161,18 +163,31 @@ class HipSharedPrefixAttn(AttnFunc):
     """Fill: prefill with parent context.  Generate: shared-prefix decode."""
 
     grouping = "lca"
+    # device tables of the last decode-only batch, patched in place while the same batch keeps generating
+    table_cache = DecodeTableCache()
+    incremental = True
 
     @classmethod
-    def _init(cls, iteration_state, builtin_config, jobs, num_heads, head_size):
-        tabs = build_iteration_tables(jobs, cls.grouping)
+    def init_iteration_state(cls, iteration_state, builtin_config, jobs, num_heads: int, head_size: int):
         device = builtin_config.device
         st = iteration_state
+        cached = cls.table_cache.advance(jobs, device) if cls.incremental else None
+        if cached is not None:
+            st.generation_sampling_config.extend(j.sampling_config for j in jobs)
+            st.tables = None  # the python-list form is not rebuilt on this path
+            st.flash_context_len = cached.flash_context_len
+            st.slot_mapping = cached.slot_mapping
+            st.fill_tables = None
+            st.decode_tables = cached.tables
+            st.decode_perm = cached.decode_perm
+            return
+        tabs = build_iteration_tables(jobs, cls.grouping)
         st.num_fill_tokens.extend(tabs.num_fill_tokens)
         st.generation_sampling_config.extend(j.sampling_config for j in jobs if isinstance(j, Generate))
         st.tables = tabs
         # names the reference attaches (attn_func.py:571-599)
         st.flash_context_len = tabs.flash_context_len
-        st.slot_mapping = torch.tensor(tabs.slot_mapping, dtype=torch.int32, device=device)
+        st.slot_mapping = torch.from_numpy(np.asarray(tabs.slot_mapping, dtype=np.int32)).to(device)
         st.fill_tables = None
         if tabs.fill_q_lens:
             st.fill_tables = kernels.PrefillTables.build(tabs.fill_q_lens, tabs.fill_slot_lists, device)
@@ -195,10 +210,11 @@ class HipSharedPrefixAttn(AttnFunc):
                 inv = torch.empty_like(perm)
                 inv[perm] = torch.arange(len(order), dtype=torch.int64, device=device)
                 st.decode_perm = (perm, inv)
-
-    @staticmethod
-    def init_iteration_state(iteration_state, builtin_config, jobs, num_heads: int, head_size: int):
-        HipSharedPrefixAttn._init(iteration_state, builtin_config, jobs, num_heads, head_size)
+            if cls.incremental:
+                cls.table_cache.store(jobs, order, [len(x) for x in suffix], st.decode_tables, st.decode_perm,
+                                      tabs.flash_context_len, num_heads, head_size, device)
+        elif cls.incremental:
+            cls.table_cache.clear()
 
     def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, iteration_state) -> torch.Tensor:
         st = iteration_state
@@ -229,10 +245,7 @@ class HipGroupedPrefixAttn(HipSharedPrefixAttn):
     groups in one batch each keep their shared-prefix phase."""
 
     grouping = "parent"
-
-    @staticmethod
-    def init_iteration_state(iteration_state, builtin_config, jobs, num_heads: int, head_size: int):
-        HipGroupedPrefixAttn._init(iteration_state, builtin_config, jobs, num_heads, head_size)
+    table_cache = DecodeTableCache()
 
 
 def get_attn_func(attn_func_name: str):

@@ -276,16 +276,24 @@ class DecodeTables:
         if items.shape[0] == 0:
             return
         lanes = lane_cu.shape[0] - 1
-        rec = np.zeros((lanes, 8), dtype=np.int32)
+        n_items = items.shape[0]
+        # one host buffer, one upload: items | lane records | per-request item offsets
+        o_rec = n_items * 4
+        o_cu = o_rec + lanes * 8
+        buf = np.zeros(o_cu + req_cu.shape[0], dtype=np.int32)
+        buf[:o_rec] = items.reshape(-1)
+        rec = buf[o_rec:o_cu].reshape(lanes, 8)
         rec[:, 0] = lane_cu[:-1]
         rec[:, 1] = lane_cu[1:] - lane_cu[:-1]
-        first = np.minimum(lane_cu[:-1], items.shape[0] - 1)
+        first = np.minimum(lane_cu[:-1], n_items - 1)
         rec[:, 2:5] = items[first, 0:3]
-        self.plan_items = torch.from_numpy(items).to(device)
-        self.plan_lane_item_cu = torch.from_numpy(rec).to(device)
-        self.plan_req_item_cu = torch.from_numpy(req_cu).to(device)
-        self.plan = _lib.SuffixPlan(self.plan_items.data_ptr(), items.shape[0], self.plan_lane_item_cu.data_ptr(),
-                                    lane_cu.shape[0] - 1, self.plan_req_item_cu.data_ptr())
+        buf[o_cu:] = req_cu
+        dev_buf = torch.from_numpy(buf).to(device)
+        self.plan_items = dev_buf[:o_rec].view(n_items, 4)
+        self.plan_lane_item_cu = dev_buf[o_rec:o_cu].view(lanes, 8)
+        self.plan_req_item_cu = dev_buf[o_cu:]
+        self.plan = _lib.SuffixPlan(self.plan_items.data_ptr(), n_items, self.plan_lane_item_cu.data_ptr(),
+                                    lanes, self.plan_req_item_cu.data_ptr())
 
     @staticmethod
     def build(prefix_lists: Sequence[Sequence[int]], group_req_cu: Sequence[int],
@@ -307,7 +315,7 @@ class DecodeTables:
                 cu.append(len(flat))
             t.num_groups = G
             t.max_prefix_len = max(len(p) for p in prefix_lists)
-            t.prefix_slots = torch.tensor(flat if flat else [0], dtype=torch.int32, device=device)
+            t.prefix_slots = torch.from_numpy(np.asarray(flat if flat else [0], dtype=np.int32)).to(device)
             t.prefix_cu = torch.tensor(cu, dtype=torch.int32, device=device)
             t.group_req_cu_host = torch.tensor(list(group_req_cu), dtype=torch.int32)
             t.group_req_cu = t.group_req_cu_host.to(device)
@@ -318,9 +326,16 @@ class DecodeTables:
             # padded [B, max] table: a request's list start needs no lookup, so the kernel can fetch
             # slot ids and the length at the same time
             width = (t.max_suffix_len + 15) // 16 * 16
+            # one conversion of all lists back to back, then a scatter into the padded rows
+            flat_suffix: List[int] = []
+            for sl in suffix_lists:
+                flat_suffix.extend(sl)
+            lens_a = np.asarray(lens, dtype=np.int64)
+            starts = np.zeros(B, dtype=np.int64)
+            np.cumsum(lens_a[:-1], out=starts[1:])
+            pos = np.arange(total, dtype=np.int64) - np.repeat(starts, lens_a)
             table = np.zeros((B, width), dtype=np.int32)
-            for i, sl in enumerate(suffix_lists):
-                table[i, : len(sl)] = np.asarray(sl, dtype=np.int32)
+            table[np.repeat(np.arange(B, dtype=np.int64), lens_a), pos] = np.asarray(flat_suffix, dtype=np.int32)
             t.suffix_slots = torch.from_numpy(table).to(device)
             t.suffix_offsets = None
             t.suffix_table_stride = width
@@ -335,14 +350,37 @@ class DecodeTables:
         return t
 
 
+_cu_counts: Dict[str, int] = {}
+
+
+def _cu_count(device) -> int:
+    key = str(device)
+    n = _cu_counts.get(key)
+    if n is None:
+        n = 256
+        if torch.cuda.is_available() and key != "cpu":
+            n = torch.cuda.get_device_properties(device).multi_processor_count
+        _cu_counts[key] = n
+    return n
+
+
+def suffix_tables_append(table: torch.Tensor, lens: torch.Tensor, rows: Optional[torch.Tensor],
+                         new_slots: torch.Tensor) -> None:
+    """``table[rows[i], lens[rows[i]]] = new_slots[i]; lens[rows[i]] += 1`` on the device (int32 tensors; the
+    per-iteration patch of the padded suffix table, in place of rebuilding it from lists)."""
+    _require_gpu(table, lens, new_slots)
+    assert table.dtype == lens.dtype == new_slots.dtype == torch.int32 and table.dim() == 2 and table.stride(1) == 1
+    assert rows is None or (rows.dtype == torch.int32 and rows.numel() == new_slots.numel())
+    check(_lib.load().ph_suffix_tables_append(_ptr(table), table.stride(0), _ptr(lens), _ptr(rows), _ptr(new_slots),
+                                              new_slots.numel(), _stream()), "suffix_tables_append")
+
+
 def suffix_lanes(device, num_heads: int, head_dim: int, total_tokens: int) -> int:
     """Pieces of the balanced suffix phase: one launch-wide round of waves at three waves per SIMD
     (a piece is streamed by one wave per 64/(head_dim/8) heads), and no piece under 16 tokens."""
     heads_per_wave = max(1, 64 // max(1, head_dim // 8))
     hgroups = (num_heads + heads_per_wave - 1) // heads_per_wave
-    cus = 256
-    if torch.cuda.is_available() and str(device) != "cpu":
-        cus = torch.cuda.get_device_properties(device).multi_processor_count
+    cus = _cu_count(device)
     lanes = max(1, cus * 4 * 3 // hgroups)
     return max(1, min(lanes, (total_tokens + 15) // 16))
 

@@ -204,3 +204,62 @@ def test_decoder_layer_config5_scaled(dev):
     mlp = (act @ w["down_proj"].float().t()).half().float()
     ref_y = (hcpu.float() + mlp).half()
     torch.testing.assert_close(y.cpu().float(), ref_y.float(), atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("name,n_groups", [("xformers_fill_shared_prompts_generate", 1), ("hip_shared_prefix", 3)])
+def test_incremental_tables_match_full_rebuild_over_a_decode_loop(dev, name, n_groups):
+    """A decode loop of 40 iterations: the tables the plug-in patches in place each iteration (one appended slot
+    per request, fresh plan) are bit-identical to the ones built from the context trees from scratch, through
+    the widening of the padded table, and the attention outputs agree."""
+    from parrotserve_amd import mem
+    from parrotserve_amd.attn_func import BuiltinConfig, get_attn_func
+    from parrotserve_amd.context import RecyclePool
+    from parrotserve_amd.iter_state import IterationState
+    from parrotserve_amd.table_cache import DecodeTableCache
+
+    H, D, slots = 8, 128, 8192
+    pool = RecyclePool(pool_size=slots)
+    jobs = _build_forest(pool, 17 + n_groups, n_groups, 5, 200, with_fills=False)
+    base = get_attn_func(name)
+
+    class Inc(base):  # own cache, so other tests' batches do not interfere
+        table_cache = DecodeTableCache()
+
+    class Fresh(base):  # the cache switched off: rebuilds everything every iteration
+        incremental = False
+
+    cfg_inc = BuiltinConfig(num_kv_cache_blocks=slots, attn_func=Inc, dtype=torch.float16, device=dev)
+    cfg_full = BuiltinConfig(num_kv_cache_blocks=slots, attn_func=Fresh, dtype=torch.float16, device=dev)
+    store = mem.init_model_cache_storage(1, slots, H, D, torch.float16, dev)
+    g = torch.Generator(device=dev).manual_seed(9)
+    store.k_cache[0].normal_(generator=g)
+    store.v_cache[0].normal_(generator=g)
+    attn_inc = Inc(layer_idx=0, scaling=D ** -0.5, num_heads=H, head_dim=D)
+    attn_full = Fresh(layer_idx=0, scaling=D ** -0.5, num_heads=H, head_dim=D)
+    B = len(jobs)
+    for it in range(40):
+        for j in jobs:
+            j.context.allocate(1)
+        st_i = IterationState(jobs, _Cfg(H, H * D), cfg_inc)
+        st_f = IterationState(jobs, _Cfg(H, H * D), cfg_full)
+        assert (st_i.tables is None) == (it > 0)  # every iteration after the first came from the cache
+        assert st_f.tables is not None
+        ti, tf = st_i.decode_tables, st_f.decode_tables
+        assert torch.equal(st_i.slot_mapping, st_f.slot_mapping)
+        assert torch.equal(ti.suffix_lens, tf.suffix_lens) and ti.max_suffix_len == tf.max_suffix_len
+        w = tf.suffix_slots.shape[1]
+        assert ti.suffix_slots.shape[1] >= w
+        cols = torch.arange(w, device=dev)[None, :] < tf.suffix_lens[:, None]
+        assert torch.equal(torch.where(cols, ti.suffix_slots[:, :w], 0), torch.where(cols, tf.suffix_slots, 0))
+        assert torch.equal(ti.plan_items, tf.plan_items) and torch.equal(ti.plan_lane_item_cu, tf.plan_lane_item_cu)
+        assert torch.equal(ti.plan_req_item_cu, tf.plan_req_item_cu)
+        assert (st_i.decode_perm is None) == (st_f.decode_perm is None)
+        if st_i.decode_perm is not None:
+            assert torch.equal(st_i.decode_perm[0], st_f.decode_perm[0])
+        if it % 13 == 0 or it == 39:
+            qkv = torch.randn(B, 3 * H * D, generator=g, device=dev, dtype=torch.float16)
+            q, k, v = (t.view(B, H, D) for t in qkv.chunk(3, dim=-1))
+            o_i = attn_inc(q, k, v, st_i)
+            o_f = attn_full(q, k, v, st_f)  # appends the same rows again: idempotent
+            assert torch.equal(o_i, o_f)
+    assert Inc.table_cache.hits == 39 and Inc.table_cache.rebuilds == 1

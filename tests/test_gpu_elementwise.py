@@ -105,7 +105,8 @@ def test_kv_append_bit_exact_from_qkv_views(dev, dtype, idx_dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("rows,n", [(128, 5120), (33, 4096), (5, 8192), (7, 1000), (3, 130)])
+@pytest.mark.parametrize("rows,n", [(128, 5120), (33, 4096), (5, 8192), (7, 1000), (3, 130),
+                                    (2049, 5120), (2051, 8192), (2048, 512), (2050, 1320), (2500, 16384)])
 def test_rms_norm(dev, dtype, rows, n):
     from parrotserve_amd import kernels
 

@@ -1,6 +1,7 @@
 """Host-side slot indexing of the product package against the list-based oracle model (bit-exact integers)."""
 import random
 
+import numpy as np
 import pytest
 
 from oracle.ref_context import RefContext, RefPoolError, RefRecyclePool, ref_iteration_tables, ref_shared_context_len
@@ -206,3 +207,75 @@ def test_suffix_plan_covers_every_token_once_and_balances(seed):
     # pieces differ by at most one token
     per_lane = [int(items[lane_cu[j] : lane_cu[j + 1], 2].sum()) for j in range(len(lane_cu) - 1)]
     assert sum(per_lane) == total and max(per_lane) - min(per_lane) <= 1
+
+
+def _decode_batch(pool, branches=5, prefix=40):
+    parent = BlockContext(0, None, pool, 1)
+    parent.allocate(prefix)
+    jobs = []
+    for b in range(branches):
+        child = BlockContext(1 + b, parent, pool, 1)
+        child.allocate(3 + b)
+        job = Generate(0, b, child.context_id, parent.context_id, sampling_config=None)
+        job.context = child
+        jobs.append(job)
+    return parent, jobs
+
+
+def test_table_cache_host_side_hits_only_on_the_same_batch_one_token_later():
+    """Host half of the incremental tables: a hit returns exactly the slots the contexts gained (what the
+    from-scratch build reports as slot_mapping) and moves the cached lengths; every way a batch can differ
+    from 'same jobs, one token later' is a miss that leaves the cache untouched."""
+    from parrotserve_amd.table_cache import DecodeTableCache, _Cached
+
+    pool = RecyclePool(pool_size=4096)
+    parent, jobs = _decode_batch(pool)
+    cache = DecodeTableCache()
+    assert cache.advance_host(jobs) is None  # nothing cached yet
+
+    def remember():
+        ctxs = [j.context for j in jobs]
+        lens = np.array([len(c.token_kv_block_ids) for c in ctxs], dtype=np.int64)
+        cache.state = _Cached(ctxs, [c.parent_context for c in ctxs], [len(c.token_kv_block_ids) for c in ctxs],
+                              [parent.get_context_len()] * len(jobs), None, lens, None, None, 0, 8, 128)
+
+    remember()
+    assert cache.advance_host(jobs) is None  # same lengths: not one token later
+    for it in range(3):
+        for j in jobs:
+            j.context.allocate(1)
+        got = cache.advance_host(jobs)
+        assert got == build_iteration_tables(jobs).slot_mapping  # the from-scratch path, itself pinned to the oracle
+        assert cache.state.lens_host.tolist() == [len(j.context.token_kv_block_ids) for j in jobs]
+    before = (list(cache.state.own_lens), cache.state.lens_host.copy())
+
+    def unchanged():
+        return cache.state.own_lens == before[0] and np.array_equal(cache.state.lens_host, before[1])
+
+    # two tokens at once
+    for j in jobs:
+        j.context.allocate(2)
+    assert cache.advance_host(jobs) is None and unchanged()
+    remember()
+    before = (list(cache.state.own_lens), cache.state.lens_host.copy())
+    for j in jobs:
+        j.context.allocate(1)
+    # a job left; the order changed
+    assert cache.advance_host(jobs[:-1]) is None and unchanged()
+    assert cache.advance_host(jobs[::-1]) is None and unchanged()
+    # a Fill on one of the contexts
+    f = Fill(0, 99, jobs[0].context_id, parent.context_id, token_ids=[1])
+    f.context = jobs[0].context
+    assert cache.advance_host([f] + jobs[1:]) is None and unchanged()
+    # the parent grew (the shared prefix changed)
+    parent.allocate(1)
+    assert cache.advance_host(jobs) is None and unchanged()
+    parent.token_kv_block_ids.pop()
+    # a different context object with the right length
+    other = BlockContext(50, parent, pool, 1)
+    other.allocate(len(jobs[0].context.token_kv_block_ids))
+    g = Generate(0, 98, 50, parent.context_id)
+    g.context = other
+    assert cache.advance_host([g] + jobs[1:]) is None and unchanged()
+    # and the unchanged batch still qualifies
+    assert cache.advance_host(jobs) == [j.context.token_kv_block_ids[-1] for j in jobs]
