@@ -192,6 +192,7 @@ def extras(torch, dev):
     out["c5_layer"] = config5_layer(torch, dev)
     out["c2_iteration_tables"] = iteration_tables_cost(torch, dev)
     out["e2e_decode_13b"] = e2e_decode(torch, dev)
+    out["e2e_decode_13b_fused_ops"] = e2e_decode(torch, dev, fused_ops=True)
     # --- RMSNorm at a bandwidth-sized row count (LLaMA-13B hidden) -----------------------------------------
     xs = [torch.randn((8192, 5120), device=dev, dtype=torch.float16) for _ in range(8)]  # 8 x 84 MB, rotated
     w = torch.ones(5120, device=dev, dtype=torch.float16)
@@ -254,7 +255,7 @@ def iteration_tables_cost(torch, dev):
     return res
 
 
-def e2e_decode(torch, dev):
+def e2e_decode(torch, dev, fused_ops=False):
     """The reference's decode experiment (benchmark/bench_kernel.py:11-86) end to end on the engine loop: LLaMA-13B
     shape (vicuna-13b-v1.3: 40 layers, hidden 5120, 40x128, FFN 13824, vocab 32000) with random weights, batch 64,
     one shared 8192-token Fill, 64 forked Fills of 10 tokens, then 10 Generate iterations."""
@@ -265,7 +266,7 @@ def e2e_decode(torch, dev):
 
     B, shared_len, diverged_len, output_len = 64, 8192, 10, 10
     mc = LlamaConfig(vocab_size=32000, hidden_size=5120, intermediate_size=13824, num_hidden_layers=40,
-                     num_attention_heads=40, rms_norm_eps=1e-6, max_position_embeddings=16384)
+                     num_attention_heads=40, rms_norm_eps=1e-6, max_position_embeddings=16384, fused_ops=fused_ops)
     cfg = BuiltinConfig(num_kv_cache_blocks=16384, attn_func="hip_shared_prefix", dtype=torch.float16, device=dev)
     cfg.attn_func.table_cache.clear()
     runner = BuiltinRunner(mc, cfg)
@@ -276,7 +277,7 @@ def e2e_decode(torch, dev):
     its = [runner.run_iter(gens) for _ in range(output_len - 1)]
     e2e = sorted(t[0] for t in its[1:])
     model = sorted(t[1] for t in its[1:])
-    res = {"model": "LLaMA-13B shape, random weights", "batch": B, "shared_len": shared_len, "diverged_len": diverged_len,
+    res = {"model": "LLaMA-13B shape, random weights", "fused_ops": fused_ops, "batch": B, "shared_len": shared_len, "diverged_len": diverged_len,
            "shared_fill_ms": t_fill[1] / 1e6, "diverged_fills_ms": t_div[1] / 1e6,
            "decode_iter_ms": e2e[len(e2e) // 2] / 1e6, "decode_model_ms": model[len(model) // 2] / 1e6,
            "decode_tokens/s": B / (e2e[len(e2e) // 2] / 1e9)}

@@ -247,6 +247,42 @@ int ph_prefill_attention(void* out, const void* q, const void* k_cache, const vo
                          void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------ */
+/* Fused forms of the small per-layer ops (same arithmetic as the unfused
+ * sequences, one launch each).
+ *
+ * ph_add_rms_norm: residual += x (stored back, rounded to the element type),
+ * out = RMSNorm(residual) * weight.  Replaces the torch residual add of
+ * parrot/engine/builtin/models/llama.py:160-178 followed by rms_norm
+ * (3rdparty/vllm/csrc/layernorm_kernels.cu:9-63 for round_before_weight = 1,
+ * parrot/engine/builtin/kernels/rms_norm.py:15-78 for 0).  Strides in elements.
+ *
+ * ph_silu_mul: out = silu(gate) * up, silu in fp32 rounded to the element
+ * type, then the product -- silu_and_mul of
+ * 3rdparty/vllm/csrc/activation_kernels.cu:6-48 with gate and up given by
+ * pointer and row stride (gate = input, up = input + d for its [T, 2d] form),
+ * and the act_fn(gate) * up of the Hugging Face LlamaMLP the reference imports
+ * (models/llama.py:36-39).
+ *
+ * ph_rope_append: NeoX rotation of q and k in place (as ph_rope_neox), then
+ * the rotated k rows and the v rows go to their slots (as ph_kv_append) --
+ * one pass over k instead of two.  Replaces rotary_embedding_neox +
+ * reshape_and_cache (pos_encoding_kernels.cu:38-104, cache_kernels.cu:142-224)
+ * as called back to back in models/llama.py:122-129 / attn_func.py:143-155. */
+int ph_add_rms_norm(void* out, void* residual, const void* x, const void* weight, float eps,
+                    int64_t rows, int64_t n, int64_t x_stride, int64_t residual_stride,
+                    int64_t out_stride, int dtype, int round_before_weight, void* stream);
+
+int ph_silu_mul(void* out, const void* gate, const void* up, int64_t rows, int64_t d,
+                int64_t gate_stride, int64_t up_stride, int64_t out_stride, int dtype, void* stream);
+
+int ph_rope_append(const int64_t* positions, void* q, void* k, const void* v,
+                   const void* cos_sin_cache, void* k_cache, void* v_cache,
+                   const void* slot_mapping, int index_type, int64_t num_tokens,
+                   int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim, int64_t rot_dim,
+                   int64_t q_stride, int64_t k_stride, int64_t v_stride, int64_t cache_stride_n,
+                   int dtype, void* stream);
+
+/* ------------------------------------------------------------------------ */
 /* Incremental suffix tables.  The reference rebuilds paged_block_tables /
  * paged_context_lens from Python lists and uploads them every iteration
  * (parrot/engine/builtin/attn_func.py:523-531,553-569); between two decode

@@ -317,3 +317,25 @@ def ref_rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, round_before
     if round_before_weight:
         return ((xf * rstd).to(dt) * weight.to(dt)).to(dt)
     return (xf * rstd * _f32(weight)).to(dt)
+
+
+# --------------------------------------------------------------------------- #
+# fused per-layer ops (compositions of the above, kept as the unfused sequences)
+# --------------------------------------------------------------------------- #
+def ref_add_rms_norm(x: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor, eps: float,
+                     round_before_weight: bool = True) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``h = residual + x`` as a tensor of the element type (the torch add of
+    parrot/engine/builtin/models/llama.py:160-178), then ``ref_rms_norm(h)``.
+    Returns ``(y, h)``: the norm runs on the rounded, stored ``h``."""
+    h = (_f32(residual) + _f32(x)).to(x.dtype)
+    return ref_rms_norm(h, weight, eps, round_before_weight), h
+
+
+def ref_silu_mul(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """``t(t(g / (1 + exp(-g))) * u)``: silu in fp32 rounded to the element type, then the product rounded
+    (3rdparty/vllm/csrc/activation_kernels.cu:6-24; the same two roundings as ``act_fn(gate) * up`` of the
+    Hugging Face LlamaMLP the reference imports, parrot/engine/builtin/models/llama.py:36-39)."""
+    dt = gate.dtype
+    g = _f32(gate)
+    s = (g / (1.0 + torch.exp(-g))).to(dt)
+    return (_f32(s) * _f32(up)).to(dt)

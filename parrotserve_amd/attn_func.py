@@ -216,11 +216,15 @@ class HipSharedPrefixAttn(AttnFunc):
         elif cls.incremental:
             cls.table_cache.clear()
 
-    def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, iteration_state) -> torch.Tensor:
+    def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, iteration_state,
+                kv_appended: bool = False) -> torch.Tensor:
+        """``kv_appended``: the caller has already written this iteration's k, v rows to their slots (the fused
+        rotary + append kernel does); the reference's four-argument call appends here."""
         st = iteration_state
         k_cache = get_k_cache(self.layer_idx)
         v_cache = get_v_cache(self.layer_idx)
-        kernels.kv_append(k, v, k_cache, v_cache, st.slot_mapping)
+        if not kv_appended:
+            kernels.kv_append(k, v, k_cache, v_cache, st.slot_mapping)
         T = q.shape[0]
         if q.stride(1) != self.head_dim or q.stride(2) != 1:
             q = q.contiguous()

@@ -118,6 +118,25 @@ __device__ __forceinline__ float group_max(float v) {
   return v;
 }
 
+// NeoX rotation of 8 pairs in the element type: every product and the final sum / difference is rounded
+// to the element type, as the reference's CUDA kernel does (3rdparty/vllm/csrc/pos_encoding_kernels.cu:6-36).
+template <typename E>
+__device__ __forceinline__ void rotate8(u32x4& x, u32x4& y, const u32x4 c, const u32x4 s) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const float xl = Elem<E>::lo(x[j]), xh = Elem<E>::hi(x[j]);
+    const float yl = Elem<E>::lo(y[j]), yh = Elem<E>::hi(y[j]);
+    const float cl = Elem<E>::lo(c[j]), ch = Elem<E>::hi(c[j]);
+    const float sl = Elem<E>::lo(s[j]), sh = Elem<E>::hi(s[j]);
+    const float nxl = rnd<E>(xl * cl) - rnd<E>(yl * sl);
+    const float nxh = rnd<E>(xh * ch) - rnd<E>(yh * sh);
+    const float nyl = rnd<E>(yl * cl) + rnd<E>(xl * sl);
+    const float nyh = rnd<E>(yh * ch) + rnd<E>(xh * sh);
+    x[j] = pack2<E>(nxl, nxh);
+    y[j] = pack2<E>(nyl, nyh);
+  }
+}
+
 // Optional timing of one kernel's own dispatch: the three main kernels of the decode path (0 prefix,
 // 1 suffix, 2 merge) are launched through hipExtLaunchKernelGGL, which stamps a start and a stop event
 // with the dispatch's begin and end timestamps.  Null events (the normal case) make it a plain launch.

@@ -121,23 +121,6 @@ static int launch_rms(void* out, const void* x, const void* w, float eps, int64_
 // Element-type arithmetic: every product and the final sum/difference is
 // rounded to the element type, as the reference's CUDA kernel does.
 template <typename E>
-__device__ __forceinline__ void rotate8(u32x4& x, u32x4& y, const u32x4 c, const u32x4 s) {
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const float xl = Elem<E>::lo(x[j]), xh = Elem<E>::hi(x[j]);
-    const float yl = Elem<E>::lo(y[j]), yh = Elem<E>::hi(y[j]);
-    const float cl = Elem<E>::lo(c[j]), ch = Elem<E>::hi(c[j]);
-    const float sl = Elem<E>::lo(s[j]), sh = Elem<E>::hi(s[j]);
-    const float nxl = rnd<E>(xl * cl) - rnd<E>(yl * sl);
-    const float nxh = rnd<E>(xh * ch) - rnd<E>(yh * sh);
-    const float nyl = rnd<E>(yl * cl) + rnd<E>(xl * sl);
-    const float nyh = rnd<E>(yh * ch) + rnd<E>(xh * sh);
-    x[j] = pack2<E>(nxl, nxh);
-    y[j] = pack2<E>(nyl, nyh);
-  }
-}
-
-template <typename E>
 __global__ __launch_bounds__(256) void rope_vec(const int64_t* __restrict__ positions, uint16_t* q, uint16_t* k,
                                                 const uint16_t* __restrict__ cos_base,
                                                 const uint16_t* __restrict__ sin_base, int64_t cs_stride,

@@ -76,7 +76,14 @@ def _require_gpu(*ts: torch.Tensor) -> torch.device:
     return dev
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream() -> int:
+    """Handle of torch's current stream on the current device (the raw getter costs a fraction of a
+    microsecond; building a torch.cuda.Stream object per launch costs several)."""
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
@@ -100,7 +107,6 @@ def _workspace(nbytes: int, device: torch.device) -> torch.Tensor:
 # --------------------------------------------------------------------------- #
 # token move / KV append
 # --------------------------------------------------------------------------- #
-@torch.inference_mode()
 def discontinuous_move_tokens(src_storage, dest_storage, src_indices, dest_indices):
     """``dest_storage[dest_indices[i]] = src_storage[src_indices[i]]``
     (parrot/engine/builtin/kernels/tokens_moving.py:67-100).  Storages are
@@ -143,7 +149,6 @@ def move_tokens_from_blocked_v_cache(blocked_v_cache, dest_storage, src_slot_ind
     _move_from_cache(blocked_v_cache, dest_storage, src_slot_indices, dest_indices, "move_tokens_from_blocked_v_cache")
 
 
-@torch.inference_mode()
 def kv_append(key, value, key_cache, value_cache, slot_mapping):
     """``key_cache[slot[t]] = key[t]`` and the same for V, one launch."""
     assert key.shape == value.shape and key.dim() == 3
@@ -186,20 +191,76 @@ def _rms(x, weight, eps, round_first, name):
     return out.view(x.shape)
 
 
-@torch.inference_mode()
 def vllm_rms_norm(input, weight, eps):
     """``layernorm_ops.rms_norm`` (parrot/engine/builtin/kernels/vllm/rms_norm.py:9-16):
     the normalised value is rounded to the element type before the weight multiply."""
     return _rms(input, weight, eps, True, "vllm_rms_norm")
 
 
-@torch.inference_mode()
 def rmsnorm_forward(x, weight, eps):
     """Triton twin (parrot/engine/builtin/kernels/rms_norm.py:49-78): fp32 math, one rounding."""
     return _rms(x, weight, eps, False, "rmsnorm_forward")
 
 
-@torch.inference_mode()
+def fused_add_rms_norm(x: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor, eps: float,
+                       round_before_weight: bool = True) -> torch.Tensor:
+    """``residual += x`` in place, returns ``RMSNorm(residual) * weight`` (one launch for the residual add of
+    the decoder layer and the norm that follows it)."""
+    _require_gpu(x, residual, weight)
+    n = x.shape[-1]
+    assert x.shape == residual.shape and weight.shape == (n,) and x.dtype == residual.dtype == weight.dtype
+    x2, r2 = x.reshape(-1, n), residual.view(-1, n)
+    assert x2.stride(1) == 1 and r2.stride(1) == 1
+    out = torch.empty(x2.shape, dtype=x.dtype, device=x.device)
+    check(_lib.load().ph_add_rms_norm(_ptr(out), _ptr(r2), _ptr(x2), _ptr(weight), float(eps), x2.shape[0], n,
+                                      x2.stride(0), r2.stride(0), out.stride(0), _dtype_code(x),
+                                      1 if round_before_weight else 0, _stream()), "fused_add_rms_norm")
+    return out.view(x.shape)
+
+
+def silu_mul(gate: torch.Tensor, up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``silu(gate) * up`` in one launch; ``gate`` / ``up`` may be column slices of one fused projection."""
+    _require_gpu(gate, up)
+    d = gate.shape[-1]
+    assert gate.shape == up.shape and gate.dtype == up.dtype
+    g2 = gate if gate.dim() == 2 else gate.reshape(-1, d)
+    u2 = up if up.dim() == 2 else up.reshape(-1, d)
+    assert g2.stride(1) == 1 and u2.stride(1) == 1
+    if out is None:
+        out = torch.empty(g2.shape, dtype=gate.dtype, device=gate.device)
+    o2 = out.view(-1, d)
+    check(_lib.load().ph_silu_mul(_ptr(o2), _ptr(g2), _ptr(u2), g2.shape[0], d, g2.stride(0), u2.stride(0),
+                                  o2.stride(0), _dtype_code(gate), _stream()), "silu_mul")
+    return out.view(gate.shape)
+
+
+def silu_and_mul(out: torch.Tensor, input: torch.Tensor) -> None:
+    """vLLM's form (3rdparty/vllm/csrc/activation.cpp:3-6): ``input`` is ``[T, 2d]`` = gate | up."""
+    d = input.shape[-1] // 2
+    silu_mul(input[..., :d], input[..., d:], out=out)
+
+
+def rope_and_cache(positions, query, key, value, cos_sin_cache, head_size, key_cache, value_cache, slot_mapping):
+    """``vllm_rotary_emb(positions, query, key, ...)`` followed by ``vllm_reshape_and_cache(key, value, ...)``
+    in one launch: q and k rotated in place, rotated k rows and v rows written to their slots."""
+    _require_gpu(query, key, value, key_cache, value_cache, cos_sin_cache, positions, slot_mapping)
+    assert positions.dtype == torch.int64 and positions.dim() == 1
+    T = positions.shape[0]
+    q2, k2, v2 = query.view(T, -1) if query.dim() == 3 else query, key.view(T, -1) if key.dim() == 3 else key, \
+        value.view(T, -1) if value.dim() == 3 else value
+    assert q2.stride(1) == 1 and k2.stride(1) == 1 and v2.stride(1) == 1
+    hq, hk = q2.shape[1] // head_size, k2.shape[1] // head_size
+    assert v2.shape[1] == hk * head_size and key_cache.shape[1:] == (hk, head_size)
+    assert key_cache.stride() == value_cache.stride() and key_cache.stride(2) == 1 and key_cache.stride(1) == head_size
+    assert query.dtype == key.dtype == value.dtype == key_cache.dtype == cos_sin_cache.dtype
+    assert slot_mapping.numel() == T and cos_sin_cache.is_contiguous()
+    check(_lib.load().ph_rope_append(_ptr(positions), _ptr(q2), _ptr(k2), _ptr(v2), _ptr(cos_sin_cache),
+                                     _ptr(key_cache), _ptr(value_cache), _ptr(slot_mapping), _index_code(slot_mapping),
+                                     T, hq, hk, head_size, cos_sin_cache.shape[-1], q2.stride(0), k2.stride(0),
+                                     v2.stride(0), key_cache.stride(0), _dtype_code(query), _stream()),
+          "rope_and_cache")
+
+
 def vllm_rotary_emb(positions, query, key, cos_sin_cache, head_size):
     """NeoX rotary embedding of ``query`` and ``key`` in place
     (parrot/engine/builtin/kernels/vllm/rotary_embed.py:10-25).  query / key are
@@ -218,7 +279,6 @@ def vllm_rotary_emb(positions, query, key, cos_sin_cache, head_size):
     check(rc, "vllm_rotary_emb")
 
 
-@torch.inference_mode()
 def rotary_embedding(state, cos, sin):
     """In-place NeoX rotation of ``state [T, H, D]`` with per-token ``cos``,
     ``sin`` of shape ``[T, 1, D/2]`` (parrot/engine/builtin/kernels/rotary_embedding.py:107-143)."""
@@ -412,7 +472,6 @@ def plan_suffix_items(lens: Sequence[int], num_lanes: int):
     return items, lane_cu, req_cu
 
 
-@torch.inference_mode()
 def decode_attention(query: torch.Tensor, key_cache: torch.Tensor, value_cache: torch.Tensor, tables: DecodeTables,
                      scale: Optional[float] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Shared-prefix (or plain ragged) decode attention: prefix phase on the
@@ -472,7 +531,6 @@ def _check_paged_args(query, key_cache, value_cache, head_mapping, context_lens,
     assert block_tables.shape[0] == query.shape[0]
 
 
-@torch.inference_mode()
 def vllm_paged_attention(query, key_cache, value_cache, head_mapping, context_lens, block_tables):
     """Non-shared ragged decode (parrot/engine/builtin/kernels/vllm/paged_attention.py:12-38):
     request i attends over ``block_tables[i, :context_lens[i]]``."""
@@ -484,7 +542,6 @@ def vllm_paged_attention(query, key_cache, value_cache, head_mapping, context_le
     return decode_attention(query, key_cache, value_cache, t)
 
 
-@torch.inference_mode()
 def flash_paged_attention(query, key_cache, value_cache, head_mapping, flash_context_len, flash_block_table,
                           paged_context_lens, paged_block_tables):
     """Shared-prefix decode (parrot/engine/builtin/kernels/shared_flash_decoding.py:285-329):
@@ -543,7 +600,6 @@ class PrefillTables:
             max_kv_len=max((len(s) for s in ctx_slot_lists), default=0))
 
 
-@torch.inference_mode()
 def prefill_attention(query, key_cache, value_cache, tables: PrefillTables, scale: Optional[float] = None,
                       out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Packed ragged prefill, each chunk causal (bottom-right aligned) over its

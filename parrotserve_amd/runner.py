@@ -49,6 +49,7 @@ class LlamaConfig:
     max_position_embeddings: int = 4096
     rope_theta: float = 10000.0
     pad_token_id: Optional[int] = None
+    fused_ops: bool = False  # fewer launches, same arithmetic (see llama_layer)
 
 
 class EngineContextManager:
@@ -119,12 +120,18 @@ class LlamaModel(nn.Module):
         self.embed_tokens = nn.Embedding(config.vocab_size, config.hidden_size, config.pad_token_id)
         self.layers = nn.ModuleList([
             LlamaDecoderLayer(config.hidden_size, config.num_attention_heads, config.intermediate_size,
-                              config.rms_norm_eps, i, builtin_config.attn_func)
+                              config.rms_norm_eps, i, builtin_config.attn_func, config.fused_ops)
             for i in range(config.num_hidden_layers)])
         self.norm = LlamaRMSNorm(config.hidden_size, eps=config.rms_norm_eps)
+        self.fused_ops = config.fused_ops
 
     def forward(self, input_ids, positions, iteration_state):
         hidden_states = self.embed_tokens(input_ids)
+        if self.fused_ops:
+            residual = None
+            for layer in self.layers:
+                hidden_states, residual = layer.forward_fused(hidden_states, residual, positions, iteration_state)
+            return self.norm.forward_add(hidden_states, residual)
         for layer in self.layers:
             hidden_states = layer(hidden_states, positions, iteration_state)
         return self.norm(hidden_states)

@@ -197,3 +197,84 @@ def test_rope_round_trip_property(dev):
     kernels.rotary_embedding(d, cos.to(dev), sin.to(dev))
     kernels.rotary_embedding(d, cos.to(dev), (-sin).to(dev))
     torch.testing.assert_close(d.cpu().float(), x.float(), atol=8e-3, rtol=1e-2)
+
+
+# --------------------------------------------------------------------------- #
+# fused per-layer ops
+# --------------------------------------------------------------------------- #
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("rows,n", [(128, 5120), (64, 4096), (5, 8192), (7, 1000), (3, 130)])
+def test_fused_add_rms_norm(dev, dtype, rows, n):
+    """residual += x is bit-exact (it is a rounded fp add); the norm matches the oracle, and equals the library's
+    own unfused norm of the stored sum bit for bit."""
+    from oracle.ref_ops import ref_add_rms_norm
+    from parrotserve_amd import kernels
+
+    g = torch.Generator().manual_seed(16)
+    x = (torch.randn(rows, n, generator=g) * 2).to(dtype)
+    r = (torch.randn(rows, n, generator=g) * 2 - 0.5).to(dtype)
+    w = (torch.rand(n, generator=g) + 0.5).to(dtype)
+    for first in (True, False):
+        rd = r.to(dev)
+        y = kernels.fused_add_rms_norm(x.to(dev), rd, w.to(dev), 1e-6, round_before_weight=first)
+        y_ref, h_ref = ref_add_rms_norm(x, r, w, 1e-6, round_before_weight=first)
+        assert torch.equal(_bits(rd.cpu()), _bits(h_ref))
+        torch.testing.assert_close(y.cpu().float(), y_ref.float(), **TOL[dtype])
+        unfused = (kernels.vllm_rms_norm if first else kernels.rmsnorm_forward)(rd, w.to(dev), 1e-6)
+        assert torch.equal(_bits(y.cpu()), _bits(unfused.cpu()))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("rows,d", [(128, 13824), (9, 11008), (3, 100), (1, 7)])
+def test_silu_mul(dev, dtype, rows, d):
+    from oracle.ref_ops import ref_silu_mul
+    from parrotserve_amd import kernels
+
+    g = torch.Generator().manual_seed(17)
+    gu = (torch.randn(rows, 2 * d, generator=g) * 2).to(dtype)
+    ref = ref_silu_mul(gu[:, :d], gu[:, d:])
+    dgu = gu.to(dev)
+    out = kernels.silu_mul(dgu[:, :d], dgu[:, d:])          # strided column views of one fused projection
+    torch.testing.assert_close(out.cpu().float(), ref.float(), **TOL[dtype])
+    out2 = torch.empty(rows, d, dtype=dtype, device=dev)
+    kernels.silu_and_mul(out2, dgu)                          # vLLM's [T, 2d] form
+    assert torch.equal(_bits(out2.cpu()), _bits(out.cpu()))
+    sep = kernels.silu_mul(dgu[:, :d].contiguous(), dgu[:, d:].contiguous())
+    assert torch.equal(_bits(sep.cpu()), _bits(out.cpu()))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("T,H,D,idx", [(77, 8, 128, torch.int32), (5, 40, 128, torch.int64), (33, 3, 64, torch.int32),
+                                       (9, 2, 72, torch.int32)])
+def test_rope_and_cache_equals_rope_then_append(dev, dtype, T, H, D, idx):
+    """The fused op leaves q, k and both pools bit-identical to the two separate kernels, which are themselves
+    checked against the oracle (rotation in the element type, append by slot); D = 72 takes the unfused path."""
+    from parrotserve_amd import kernels
+
+    g = torch.Generator().manual_seed(18)
+    slots = 512
+    qkv = torch.randn(T, 3 * H * D, generator=g).to(dtype)
+    pos = torch.randint(0, 300, (T,), generator=g)
+    sm = torch.randperm(slots, generator=g)[:T].to(idx)
+    cache = ref_cos_sin_cache(300, D, 10000.0, dtype)
+    kc0 = torch.randn(slots, H, D, generator=g).to(dtype)
+    vc0 = torch.randn(slots, H, D, generator=g).to(dtype)
+    # oracle
+    rq, rk = ref_rope_neox(pos, qkv[:, : H * D], qkv[:, H * D : 2 * H * D], cache, D, elem_rounding=True)
+    kc_ref, vc_ref = kc0.clone(), vc0.clone()
+    ref_kv_append(rk.reshape(T, H, D), qkv[:, 2 * H * D :].reshape(T, H, D), kc_ref, vc_ref, sm)
+    # fused
+    d1 = qkv.to(dev)
+    q1, k1, v1 = d1.chunk(3, dim=-1)
+    kc1, vc1 = kc0.to(dev), vc0.to(dev)
+    kernels.rope_and_cache(pos.to(dev), q1, k1, v1, cache.to(dev), D, kc1, vc1, sm.to(dev))
+    # separate
+    d2 = qkv.to(dev)
+    q2, k2, v2 = d2.chunk(3, dim=-1)
+    kc2, vc2 = kc0.to(dev), vc0.to(dev)
+    kernels.vllm_rotary_emb(pos.to(dev), q2, k2, cache.to(dev), D)
+    kernels.vllm_reshape_and_cache(k2.view(T, H, D), v2.view(T, H, D), kc2, vc2, sm.to(dev))
+    assert torch.equal(_bits(d1.cpu()), _bits(d2.cpu()))
+    assert torch.equal(_bits(kc1.cpu()), _bits(kc2.cpu())) and torch.equal(_bits(vc1.cpu()), _bits(vc2.cpu()))
+    assert torch.equal(_bits(q1.cpu()), _bits(rq)) and torch.equal(_bits(k1.cpu()), _bits(rk))
+    assert torch.equal(_bits(kc1.cpu()), _bits(kc_ref)) and torch.equal(_bits(vc1.cpu()), _bits(vc_ref))

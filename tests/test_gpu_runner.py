@@ -31,8 +31,9 @@ def _set_weights(model, seed):
     return w
 
 
-@pytest.mark.parametrize("attn_func", ["xformers_fill_shared_prompts_generate", "hip_shared_prefix"])
-def test_shared_prompt_generation_loop_matches_flat_oracle(dev, attn_func):
+@pytest.mark.parametrize("attn_func,fused", [("xformers_fill_shared_prompts_generate", False),
+                                             ("hip_shared_prefix", False), ("hip_shared_prefix", True)])
+def test_shared_prompt_generation_loop_matches_flat_oracle(dev, attn_func, fused):
     """The scenario of the reference's decode benchmark (benchmark/bench_kernel.py:11-66), small: one shared
     Fill, B forked Fills, then Generate iterations on the forked contexts.  Every hidden state handed to the
     sampler must equal the oracle's hidden state of the same token in the branch's flat sequence, and every
@@ -44,9 +45,10 @@ def test_shared_prompt_generation_loop_matches_flat_oracle(dev, attn_func):
     V, N, H, L, Fdim = 211, 256, 2, 2, 384
     B, shared_len, diverged_len, output_len = 6, 40, 5, 7
     mc = LlamaConfig(vocab_size=V, hidden_size=N, intermediate_size=Fdim, num_hidden_layers=L, num_attention_heads=H,
-                     rms_norm_eps=1e-6, max_position_embeddings=256)
+                     rms_norm_eps=1e-6, max_position_embeddings=256, fused_ops=fused)
     cfg = BuiltinConfig(num_kv_cache_blocks=2048, attn_func=attn_func, dtype=torch.float16, device=dev)
     cfg.attn_func.table_cache.clear()
+    hits0 = cfg.attn_func.table_cache.hits
     runner = BuiltinRunner(mc, cfg, dummy_weights=False)
     w = _set_weights(runner.model, 7)
     seen = []
@@ -62,7 +64,7 @@ def test_shared_prompt_generation_loop_matches_flat_oracle(dev, attn_func):
     for _ in range(output_len - 1):  # the first token comes from the Fill's last hidden state
         runner.run_iter(gens)
     assert all(j.finish_event.is_set() and j.gen_length == output_len for j in gens)
-    hits = cfg.attn_func.table_cache.hits
+    hits = cfg.attn_func.table_cache.hits - hits0
     assert hits == output_len - 2  # every Generate iteration after the first reused the cached tables
 
     # seen: [first sampling (B rows)], then per iteration B rows; empty calls (Fill-only iterations) have 0 rows

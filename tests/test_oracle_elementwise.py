@@ -172,3 +172,47 @@ def test_rms_norm_rounding_order_half():
     xx = (-2.3 + 0.5 * torch.randn(16, 256, generator=g)).half()
     ww = torch.rand(256, generator=g).half()
     assert torch.allclose(ref_rms_norm(xx, ww, 1e-5, True).float(), ref_rms_norm(xx, ww, 1e-5, False).float(), atol=1e-2, rtol=0)
+
+
+# --------------------------------------------------------------------------- #
+# fused per-layer ops
+# --------------------------------------------------------------------------- #
+def test_add_rms_norm_is_torch_add_then_norm_on_the_stored_sum():
+    from oracle.ref_ops import ref_add_rms_norm
+
+    g = torch.Generator().manual_seed(31)
+    for dt in (torch.float16, torch.bfloat16):
+        x = (torch.randn(7, 96, generator=g) * 3).to(dt)
+        r = (torch.randn(7, 96, generator=g) * 3).to(dt)
+        w = (torch.rand(96, generator=g) + 0.5).to(dt)
+        y, h = ref_add_rms_norm(x, r, w, 1e-6, round_before_weight=False)
+        h_t = r + x                                   # torch's own add in the element type
+        assert torch.equal(h.view(torch.int16), h_t.view(torch.int16))
+        y_t = torch.nn.functional.rms_norm(h_t.float(), (96,), w.float(), 1e-6).to(dt)
+        torch.testing.assert_close(y.float(), y_t.float(), atol=1e-2, rtol=1e-2)
+    # the norm sees the ROUNDED sum: 2048 + 1 is not representable in fp16 (spacing 2), so h = 2048, not 2049
+    x = torch.tensor([[2048.0, 0.0]], dtype=torch.float16)
+    r = torch.tensor([[1.0, 0.0]], dtype=torch.float16)
+    y, h = ref_add_rms_norm(x, r, torch.ones(2, dtype=torch.float16), 0.0, round_before_weight=False)
+    assert h[0, 0].item() == 2048.0
+    assert abs(y[0, 0].item() - 2 ** 0.5) < 1e-3      # 2048 / sqrt((2048^2 + 0) / 2)
+
+
+def test_silu_mul_closed_forms_and_torch():
+    from oracle.ref_ops import ref_silu_mul
+
+    one = torch.ones(5, dtype=torch.float16)
+    gate = torch.tensor([0.0, 20.0, -20.0, 1.0, -1.0], dtype=torch.float16)
+    got = ref_silu_mul(gate, one).float()
+    want = torch.tensor([0.0, 20.0, 0.0, 1 / (1 + math.exp(-1.0)), -1 / (1 + math.exp(1.0))])
+    torch.testing.assert_close(got, want, atol=1e-3, rtol=1e-3)
+    g = torch.Generator().manual_seed(32)
+    for dt in (torch.float16, torch.bfloat16):
+        a = (torch.randn(4, 64, generator=g) * 3).to(dt)
+        b = (torch.randn(4, 64, generator=g) * 3).to(dt)
+        ref = torch.nn.functional.silu(a) * b         # torch rounds silu, then the product, in the element type
+        assert torch.equal(ref_silu_mul(a, b).view(torch.int16), ref.view(torch.int16))
+    # linear in `up`, and the two roundings are visible: silu(1) rounds before the product
+    a = torch.tensor([1.0], dtype=torch.float16)
+    s = torch.nn.functional.silu(a.float()).half()
+    assert ref_silu_mul(a, torch.tensor([3.0], dtype=torch.float16)).item() == (s.float() * 3).half().item()
