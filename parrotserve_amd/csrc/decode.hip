@@ -46,8 +46,8 @@ __device__ __forceinline__ void stream_item(const uint16_t* __restrict__ kc, con
         const int64_t slot = __builtin_amdgcn_readlane(myslot, min(j0 + j, nb - 1));
         const uint16_t* kr = kc + slot * row_stride;
         const uint16_t* vr = vc + slot * row_stride;
-        kk[j] = ld16(kr + lane_off);
-        vv[j] = ld16(vr + lane_off);
+        kk[j] = ld16_nt(kr + lane_off);
+        vv[j] = ld16_nt(vr + lane_off);
       }
     };
     auto compute = [&](const u32x4(&kk)[TB], const u32x4(&vv)[TB], int j0) {
