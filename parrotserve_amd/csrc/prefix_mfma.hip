@@ -57,8 +57,13 @@ constexpr int kVtOff = 8192;
 // lds_addr + 16 * i (an LDS byte address, wave-uniform).  Issued as inline assembly on purpose: the compiler then
 // does not tie later LDS reads of the *other* stage to these loads, so a whole tile stays in flight
 // under the matrix work; completion is awaited explicitly (vmcnt) before a stage is read.
+// NT: non-temporal (streaming) cache policy for rows that are read once per launch.
+template <bool NT = false>
 __device__ __forceinline__ void lds_dma16(const void* gptr, uint32_t lds_addr) {
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(lds_addr) : "memory");
+  if (NT)
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt" ::"v"(gptr), "s"(lds_addr) : "memory");
+  else
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(lds_addr) : "memory");
 }
 // LDS byte address of a generic pointer into shared memory, as a wave-uniform scalar
 __device__ __forceinline__ uint32_t lds_addr_of(const char* p) {
@@ -136,8 +141,8 @@ __device__ __forceinline__ void attn_tile(const TileWork& wk, const uint16_t* __
     for (int r = 0; r < 8; ++r) {
       const uint32_t slot = (uint32_t)__shfl(snext, 4 * r + tl, kWave);
       const uint64_t ro = (uint64_t)slot * row_bytes;
-      lds_dma16(kbase[r] + ro, kb + r * 1024);
-      lds_dma16(vbase_g + ro, kb + kVtOff + r * 1024);
+      lds_dma16<!CAUSAL>(kbase[r] + ro, kb + r * 1024);
+      lds_dma16<!CAUSAL>(vbase_g + ro, kb + kVtOff + r * 1024);
     }
   };
   int tb = wk.s0 + kTile * w;
@@ -488,6 +493,9 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
   constexpr int A = NST - 1;      // tiles in flight ahead of the current one
   constexpr int LPT = 16 / QB;    // row-group loads per wave per tile
   constexpr int NDB = 4 / TQ;     // dim blocks a wave finishes
+  // decode reads every prefix row once per launch (streaming policy); prefill tiles are re-read by the
+  // other query tiles of the chunk and should stay in L2
+  constexpr bool NTLOAD = !CAUSAL;
   constexpr float kSlack = 8.f;
   float16_t oacc[4];
   float m = -INFINITY, lsum = 0.f, mtrue = -INFINITY;
@@ -528,7 +536,7 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
     for (int i = 0; i < LPT; ++i) sl[i] = (uint32_t)win[tb - win0 + 4 * (r0 + i) + tl];
     const uint32_t kb = dst0 + stage * kStage;
 #pragma unroll
-    for (int i = 0; i < LPT; ++i) lds_dma16(gbase[i] + (uint64_t)sl[i] * row_bytes, kb + i * 1024);
+    for (int i = 0; i < LPT; ++i) lds_dma16<NTLOAD>(gbase[i] + (uint64_t)sl[i] * row_bytes, kb + i * 1024);
   };
   const int ntile = (s1 - s0 + kTile - 1) / kTile;
   const int iters = (ntile + TQ - 1) / TQ;                 // same for all eight waves
