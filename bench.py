@@ -31,6 +31,8 @@ MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16
 # WRITE_SIZE in two runs of this file and scaled by the same counters' readings for a plain 1 GiB copy
 # (profiles/bench_config2_hbm_traffic.txt): 285.5 MB read + 7.4 MB written.
 SUFFIX_TRAFFIC_BYTES = 293.0e6
+# same for the kernel that runs the prefix and suffix phases in one launch: 354.1 MB read + 13.8 MB written
+FUSED_TRAFFIC_BYTES = 367.9e6
 
 
 class HipEvents:
@@ -50,10 +52,13 @@ class HipEvents:
             evs[i] = e
         return evs
 
-    def elapsed_ms(self, a, b) -> float:
+    def elapsed_ms(self, a, b):
+        """None when the pair was never recorded (the call did not launch that kernel)."""
         out = ctypes.c_float()
         rc = self.hip.hipEventElapsedTime(ctypes.byref(out), a, b)
-        assert rc == 0, f"hipEventElapsedTime rc={rc}"
+        if rc != 0:
+            self.hip.hipGetLastError()  # the failed query must not surface in a later, unrelated call
+            return None
         return out.value
 
     def destroy(self, evs):
@@ -445,15 +450,24 @@ def main():
     ph = [[ev.elapsed_ms(s[2 * k], s[2 * k + 1]) for s in sets] for k in range(3)]
     for s in sets:
         ev.destroy(s)
-    t_prefix, t_suffix, t_merge = (sum(x) / len(x) * 1e-3 for x in ph)
+    # the prefix pair stays unrecorded when the library runs the prefix and suffix phases in one launch
+    fused = all(x is None for x in ph[0])
+    t_prefix, t_suffix, t_merge = (None if any(v is None for v in x) else sum(x) / len(x) * 1e-3 for x in ph)
 
     e = 2  # bytes per fp16 element
     suffix_bytes = 2 * sum_s * H * D * e
     prefix_bytes = 2 * P * H * D * e
     prefix_flops = 4 * B * H * P * D
-    suffix_gbs = suffix_bytes / t_suffix / 1e9
-    prefix_tflops = prefix_flops / t_prefix / 1e12
-    prefix_bound_tflops = min(MFMA_F16_PEAK_TFLOPS, B * HBM_PEAK_GBS / 1e3)  # AI = B FLOP per KV byte
+    if fused:
+        # one kernel streams the prefix K/V (through the matrix cores) and every request's suffix K/V
+        kernel_name = "decode_fused_kernel (prefix + suffix phases)"
+        kernel_bytes = prefix_bytes + suffix_bytes
+        traffic = FUSED_TRAFFIC_BYTES
+    else:
+        kernel_name = "decode_items_kernel (suffix phase)"
+        kernel_bytes = suffix_bytes
+        traffic = SUFFIX_TRAFFIC_BYTES
+    kernel_gbs = kernel_bytes / t_suffix / 1e9
 
     result = {
         "metric": "shared-prefix decode attn tokens/s/layer",
@@ -474,27 +488,30 @@ def main():
             "batch": B, "prefix_len": P, "sum_suffix_len": sum_s, "heads": H, "head_dim": D, "kv_sets": NL,
         },
         "roofline": {
-            "kernel": "decode_items_kernel (suffix phase)",
+            "kernel": kernel_name,
             "bound": "hbm",
-            "achieved": suffix_gbs,
+            "achieved": kernel_gbs,
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
-            "frac": suffix_gbs / HBM_PEAK_GBS,
-            "traffic": SUFFIX_TRAFFIC_BYTES,
-            "algorithmic_bytes": suffix_bytes,
+            "frac": kernel_gbs / HBM_PEAK_GBS,
+            "traffic": traffic,
+            "algorithmic_bytes": kernel_bytes,
             "avg_launch_us": t_suffix * 1e6,
         },
-        "prefix_phase": {
-            "kernel": "prefix_mfma_kernel",
+        "merge_us": t_merge * 1e6,
+        "warm_single_kv_set": {"value": B / t_warm, "ms_per_step": t_warm * 1e3},
+    }
+    if not fused:
+        prefix_tflops = prefix_flops / t_prefix / 1e12
+        prefix_bound_tflops = min(MFMA_F16_PEAK_TFLOPS, B * HBM_PEAK_GBS / 1e3)  # AI = B FLOP per KV byte
+        result["prefix_phase"] = {
+            "kernel": "prefix_mfma8_kernel",
             "avg_launch_us": t_prefix * 1e6,
             "tflops": prefix_tflops,
             "frac_mfma_peak": prefix_tflops / MFMA_F16_PEAK_TFLOPS,
             "frac_of_min_mfma_hbm_bound": prefix_tflops / prefix_bound_tflops,
             "kv_gbs": prefix_bytes / t_prefix / 1e9,
-        },
-        "merge_us": t_merge * 1e6,
-        "warm_single_kv_set": {"value": B / t_warm, "ms_per_step": t_warm * 1e3},
-    }
+        }
     if not args.no_extras:
         del kc, vc, tables, qs
         torch.cuda.empty_cache()

@@ -166,6 +166,19 @@ extern "C" const char* ph_status_string(int status) {
 
 extern "C" int ph_abi_version(void) { return 1; }
 
+// compute units of the current device (cached per device id)
+static int device_cus() {
+  static int cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
+
 static hipEvent_t g_kernel_events[6];
 static bool g_events_armed = false;
 
@@ -224,6 +237,9 @@ extern "C" int ph_decode_attention(void* out, const void* q, const void* k_cache
   const Carve ws = carve(workspace, p, B, H, D);
   hipStream_t st = (hipStream_t)stream;
   const float sl2 = scale * kLog2e;
+  bool fuse = false;  // prefix and suffix phases in one launch
+  PrefixArgs fused_pa{};
+  int fused_groups = 0, fused_max_reqs = 0;
   if (has_prefix) {
     int covered = 0, max_group_reqs = 0;
     for (int g = 0; g < num_groups; ++g) {
@@ -253,8 +269,15 @@ extern "C" int ph_decode_attention(void* out, const void* q, const void* k_cache
     pa.B = B;
     pa.H = H;
     pa.scale_log2e = sl2;
-    rc = run_prefix(pa, dtype, D, (int)num_groups, group_req_cu_host, max_group_reqs, st);
-    if (rc != PH_OK) return rc;
+    fuse = planned && decode_fused_supported(dtype, D, max_group_reqs);
+    if (fuse) {
+      fused_pa = pa;
+      fused_groups = (int)num_groups;
+      fused_max_reqs = max_group_reqs;
+    } else {
+      rc = run_prefix(pa, dtype, D, (int)num_groups, group_req_cu_host, max_group_reqs, st);
+      if (rc != PH_OK) return rc;
+    }
   }
   const int64_t item_base = (int64_t)p.n_splits * B * H;  // first partial row of the balanced form's items
   if (planned) {
@@ -274,7 +297,8 @@ extern "C" int ph_decode_attention(void* out, const void* q, const void* k_cache
     ia.ml = ws.ml + item_base * 2;
     ia.H = H;
     ia.scale_log2e = sl2;
-    rc = launch_items(ia, dtype, D, st);
+    rc = fuse ? launch_decode_fused(fused_pa, ia, dtype, fused_groups, fused_max_reqs, device_cus(), st)
+              : launch_items(ia, dtype, D, st);
     if (rc != PH_OK) return rc;
   } else if (has_suffix) {
     PartialArgs sa{};

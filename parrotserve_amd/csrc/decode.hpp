@@ -112,5 +112,9 @@ int launch_clear_ml(float* ml, int64_t entries, hipStream_t st);
 // MFMA shared-prefix kernel: grid (split, head, group x m-tile).
 int launch_prefix_mfma(const PrefixArgs& a, int dtype, int D, int num_groups, int max_group_reqs, hipStream_t st);
 bool prefix_mfma_supported(int dtype, int D);
+// Prefix + suffix phases in one launch (see decode_fused_kernel); cus = compute units of the device.
+bool decode_fused_supported(int dtype, int D, int max_group_reqs);
+int launch_decode_fused(const PrefixArgs& a, const ItemArgs& ia, int dtype, int num_groups, int max_group_reqs, int cus,
+                        hipStream_t st);
 
 }  // namespace ph

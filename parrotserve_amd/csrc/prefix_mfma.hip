@@ -26,7 +26,7 @@
 // transposing V reads are free of bank conflicts.
 //
 // Math restated from parrot/engine/builtin/kernels/shared_flash_decoding.py:34-134.
-#include "decode.hpp"
+#include "stream_item.hpp"
 
 namespace ph {
 
@@ -483,11 +483,18 @@ __device__ __forceinline__ void wait_vmcnt() {  // vmcnt <= N, other counters un
   __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
 }
 
-template <typename E, bool CAUSAL, int TQ>
+// `mid` is called once by every wave between the prologue (slot window filled, first tiles in flight into
+// LDS, Q loaded) and the main loop: work placed there runs while the first tiles land, and must leave LDS
+// alone.  The default does nothing.
+struct NoMid {
+  __device__ __forceinline__ void operator()() const {}
+};
+
+template <typename E, bool CAUSAL, int TQ, typename Mid = NoMid>
 __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* __restrict__ kc,
                                            const uint16_t* __restrict__ vc, int64_t row_stride, int head,
                                            float scale_log2e, char* smem, float16_t (&ofold)[4 / TQ], float& mfin,
-                                           float& lfin) {
+                                           float& lfin, Mid mid = Mid()) {
   constexpr int QB = 8 / TQ;      // query blocks = waves sharing a tile
   constexpr int NST = 8 / TQ;     // stages per token group
   constexpr int A = NST - 1;      // tiles in flight ahead of the current one
@@ -542,8 +549,9 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
   const int iters = (ntile + TQ - 1) / TQ;                 // same for all eight waves
   const int my_iters = ntile > g ? (ntile - g + TQ - 1) / TQ : 0;  // tiles of this token group
   __syncthreads();                                         // window visible
+  // the whole ring is filled up front: tiles 0 .. A (the main loop issues tile it + A at step it >= 1)
 #pragma unroll
-  for (int j = 0; j < A; ++j)
+  for (int j = 0; j < NST; ++j)
     if (j < my_iters) fetch_rows(s0 + kTile * (g + TQ * j), j);
 
   // Q as the B operand: column = query 32 qb + ql, contraction chunk (h, s) = dims 64h + 8s .. +8
@@ -561,6 +569,8 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
   }
   // last token any query of this wave's block may see (none if the block has no live query)
   const int wave_last = 32 * qb >= wk.nq ? -1 : CAUSAL ? min(s1 - 1, wk.causal_off + 32 * qb + 31) : s1 - 1;
+
+  mid();
 
   // Operand read addresses of ring stage 0 (and of stage 4, beyond the reach of the 16-bit immediate).
   // K: row ql, chunk (8h + s) swizzled by the row; V: the transposing read's row/column of this lane.
@@ -606,7 +616,7 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
         fill_window();
         __syncthreads();
       }
-      if (it + A < my_iters) fetch_rows(front + kTile * g, (stage + A) % NST);
+      if (it > 0 && it + A < my_iters) fetch_rows(front + kTile * g, (stage + A) % NST);
     }
     if (it >= my_iters || tb > wave_last) continue;           // wave-uniform
     const int shi = stage >> 2, slo = (stage & 3) * kStage;
@@ -772,12 +782,12 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
   }
 }
 
-// Shared-prefix phase, eight waves: workgroup = (split, head, group x 64-query tile)
-template <typename E>
-__global__ __launch_bounds__(512) void prefix_mfma8_kernel(PrefixArgs a, int mtiles) {
-  extern __shared__ __attribute__((aligned(16))) char smem[];
-  const int split = blockIdx.x, head = blockIdx.y;
-  const int g = blockIdx.z / mtiles, mt = blockIdx.z - g * mtiles;
+// Shared-prefix phase, eight waves: one unit of work = (split, head, group x 64-query tile z), run by the
+// whole workgroup; writes one (O, m, l) part per request of the tile.
+template <typename E, typename Mid = NoMid>
+__device__ __forceinline__ void prefix_unit8(const PrefixArgs& a, int split, int head, int z, int mtiles, char* smem,
+                                             Mid mid = Mid()) {
+  const int g = z / mtiles, mt = z - g * mtiles;
   int r0 = 0, r1 = a.B, poff = 0, plen = a.fixed_prefix_len;
   if (a.prefix_cu) {
     r0 = a.group_req_cu[g];
@@ -787,7 +797,10 @@ __global__ __launch_bounds__(512) void prefix_mfma8_kernel(PrefixArgs a, int mti
   }
   const int qbase = r0 + mt * 64;
   const int nq = min(64, r1 - qbase);
-  if (nq <= 0) return;
+  if (nq <= 0) {
+    mid();
+    return;
+  }
   const int s0 = split * a.split_tokens;
   const int s1 = min(plen, s0 + a.split_tokens);
   if (s0 >= plen) {  // this group's prefix ends before the split: mark the part empty
@@ -796,6 +809,7 @@ __global__ __launch_bounds__(512) void prefix_mfma8_kernel(PrefixArgs a, int mti
       a.ml[pr * 2] = -INFINITY;
       a.ml[pr * 2 + 1] = 0.f;
     }
+    mid();
     return;
   }
   TileWork wk;
@@ -809,7 +823,7 @@ __global__ __launch_bounds__(512) void prefix_mfma8_kernel(PrefixArgs a, int mti
   wk.causal_off = 0;
   float16_t of[1];
   float m, l;
-  attn_tile8<E, false, 4>(wk, a.kc, a.vc, a.row_stride, head, a.scale_log2e, smem, of, m, l);
+  attn_tile8<E, false, 4>(wk, a.kc, a.vc, a.row_stride, head, a.scale_log2e, smem, of, m, l, mid);
   const int lane = threadIdx.x & 63, w8 = threadIdx.x >> 6, tq = w8 >> 1, qh = w8 & 1, h = lane >> 5, ql = lane & 31;
   const int q = 32 * qh + ql;
   if (q < nq) {
@@ -825,6 +839,58 @@ __global__ __launch_bounds__(512) void prefix_mfma8_kernel(PrefixArgs a, int mti
       a.ml[pr * 2] = m;
       a.ml[pr * 2 + 1] = l;
     }
+  }
+}
+
+template <typename E>
+__global__ __launch_bounds__(512) void prefix_mfma8_kernel(PrefixArgs a, int mtiles) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  prefix_unit8<E>(a, blockIdx.x, blockIdx.y, blockIdx.z, mtiles, smem);
+}
+
+// Prefix and suffix phases of one decode step in one launch.  Workgroup b owns the prefix units b,
+// b + grid, ... (normally at most one: the planner sizes the splits to the CU count) and its eight waves
+// one suffix piece each of the host-planned balanced form, (piece, head group) per wave.  Order inside a
+// workgroup: suffix records requested, prefix prologue (slot window, first K/V tiles sent on their way into
+// LDS, Q), then the suffix stream (it needs no LDS and runs at the same rate on two waves per SIMD as on
+// more), then the prefix main loop on tiles that landed long ago, then the fold.  Against two launches this
+// removes one launch, hides the prefix prologue behind the suffix stream and keeps the memory system busy
+// from the first microseconds.  The merge stays a separate launch: it needs every part.
+template <typename E>
+__global__ __launch_bounds__(512) void decode_fused_kernel(PrefixArgs pa, int mtiles, int n_units, ItemArgs ia) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  constexpr int HPW = kWave / (kPD / 8);
+  const int hgroups = (ia.H + HPW - 1) / HPW;
+  const int slots = ia.num_lanes * hgroups;
+  const int wave = __builtin_amdgcn_readfirstlane(blockIdx.x * 8 + (threadIdx.x >> 6));
+  // this wave's first suffix piece: its record is requested before anything else
+  const int piece0 = wave < slots ? wave / hgroups : -1;
+  int4 rec0 = {0, 0, 0, 0}, rec1 = {0, 0, 0, 0};
+  if (piece0 >= 0) {
+    rec0 = ia.lane_rec[2 * piece0];
+    rec1 = ia.lane_rec[2 * piece0 + 1];
+  }
+  auto suffix = [&]() {
+    if (piece0 >= 0) run_piece_rec<E, kPD, 4, 2>(ia, wave - piece0 * hgroups, rec0, rec1);
+    for (int s = wave + gridDim.x * 8; s < slots; s += gridDim.x * 8) {
+      const int piece = s / hgroups;
+      run_piece<E, kPD, 4, 2>(ia, piece, s - piece * hgroups);
+    }
+  };
+  if ((int)blockIdx.x < n_units) {
+    // the suffix stream runs between the first unit's prologue and its main loop
+    const int u = blockIdx.x;
+    const int split = u % pa.n_splits;
+    const int rest = u / pa.n_splits;
+    prefix_unit8<E>(pa, split, rest % pa.H, rest / pa.H, mtiles, smem, suffix);
+    for (int v = u + gridDim.x; v < n_units; v += gridDim.x) {
+      __syncthreads();  // the fold scratch of the last unit is the staging ring of the next
+      const int sp = v % pa.n_splits;
+      const int rs = v / pa.n_splits;
+      prefix_unit8<E>(pa, sp, rs % pa.H, rs / pa.H, mtiles, smem);
+    }
+  } else {
+    suffix();
   }
 }
 
@@ -925,6 +991,37 @@ static int launch_prefill_t(const PrefillArgs& a, int64_t num_tokens, hipStream_
   if (avg >= 192) return launch_prefill_tq<E, 1>(a, num_tokens, st);
   if (avg >= 96) return launch_prefill_tq<E, 2>(a, num_tokens, st);
   return launch_prefill_tq<E, 4>(a, num_tokens, st);
+}
+
+template <typename E>
+static int launch_fused_t(const PrefixArgs& a, const ItemArgs& ia, int num_groups, int max_group_reqs, int cus,
+                          hipStream_t st) {
+  const int mtiles = (max_group_reqs + 63) / 64;
+  const int n_units = a.n_splits * a.H * num_groups * mtiles;
+  const int hgroups = (ia.H + 3) / 4;
+  const int wave_slots = ia.num_lanes * hgroups;
+  int grid = (wave_slots + 7) / 8;
+  const int unit_grid = n_units < cus ? n_units : cus;
+  if (grid < unit_grid) grid = unit_grid;
+  if (grid <= 0) return PH_OK;
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&decode_fused_kernel<E>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kTile8Lds);
+  const KernelEvents ev = take_kernel_events(1);
+  hipExtLaunchKernelGGL((decode_fused_kernel<E>), dim3(grid), dim3(512), kTile8Lds, st, ev.start, ev.stop, 0, a, mtiles,
+                        n_units, ia);
+  return launch_status();
+}
+
+// One launch for the prefix and suffix phases: head size 128, groups of more than 32 requests (the
+// eight-wave prefix form), balanced suffix plan present.
+bool decode_fused_supported(int dtype, int D, int max_group_reqs) {
+  return D == kPD && (dtype == PH_F16 || dtype == PH_BF16) && max_group_reqs > 32;
+}
+
+int launch_decode_fused(const PrefixArgs& a, const ItemArgs& ia, int dtype, int num_groups, int max_group_reqs, int cus,
+                        hipStream_t st) {
+  return dtype == PH_F16 ? launch_fused_t<F16>(a, ia, num_groups, max_group_reqs, cus, st)
+                         : launch_fused_t<BF16>(a, ia, num_groups, max_group_reqs, cus, st);
 }
 
 bool prefix_mfma_supported(int dtype, int D) { return D == kPD && (dtype == PH_F16 || dtype == PH_BF16); }

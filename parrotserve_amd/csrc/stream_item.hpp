@@ -1,0 +1,139 @@
+// The streaming body of the per-request decode kernels (suffix phase, ragged decode): one wave, HPW adjacent
+// heads, token rows gathered by slot with 128-bit non-temporal loads, online softmax in the exp2 domain.
+// Shared by the stand-alone kernels (decode.hip) and the fused prefix + suffix kernel (prefix_mfma.hip).
+//
+// Math restated from csrc/attention/attention_post_kernels.cu:74-341 and
+// attention_prev_kernels.cu:147,223,332-337 (m / l export).
+#pragma once
+
+#include "decode.hpp"
+
+namespace ph {
+
+// Streams the token rows slots[t0 .. t1) of one request through one wave (HPW adjacent heads) and
+// writes the (O, m, l) part at row `pr` of the partial buffers.  `myslot` holds the slot ids of the
+// first 64 tokens (lane i: token t0 + i, clamped), already fetched by the caller.
+template <typename E, int D, int TB, int STAGES>
+__device__ __forceinline__ void stream_item(const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
+                                            int64_t row_stride, const int32_t* __restrict__ slots, int myslot,
+                                            int t0, int t1, u32x4 qv, uint32_t lane_off, float scale_log2e,
+                                            bool head_ok, float* __restrict__ opart, float* __restrict__ ml,
+                                            int64_t pr) {
+  constexpr int LPH = D / 8;
+  const int lane = threadIdx.x & 63;
+  float m = -INFINITY, l = 0.f;
+  float o[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) o[i] = 0.f;
+
+  u32x4 kb[STAGES][TB], vb[STAGES][TB];
+
+  for (int tb = t0; tb < t1; tb += kWave) {
+    if (tb > t0) myslot = slots[min(tb + lane, t1 - 1)];
+    const int nb = min(kWave, t1 - tb);
+
+    // TB token rows (K and V) in flight per stage; row bases are wave-uniform (SGPR)
+    auto load = [&](u32x4(&kk)[TB], u32x4(&vv)[TB], int j0) {
+#pragma unroll
+      for (int j = 0; j < TB; ++j) {
+        const int64_t slot = __builtin_amdgcn_readlane(myslot, min(j0 + j, nb - 1));
+        const uint16_t* kr = kc + slot * row_stride;
+        const uint16_t* vr = vc + slot * row_stride;
+        kk[j] = ld16_nt(kr + lane_off);
+        vv[j] = ld16_nt(vr + lane_off);
+      }
+    };
+    auto compute = [&](const u32x4(&kk)[TB], const u32x4(&vv)[TB], int j0) {
+      float s[TB];
+      float mb = -INFINITY;
+#pragma unroll
+      for (int j = 0; j < TB; ++j) {
+        float d = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) d = Elem<E>::dot2(qv[w], kk[j][w], d);
+        d = group_sum<LPH>(d) * scale_log2e;
+        s[j] = (j0 + j < nb) ? d : -INFINITY;
+        mb = fmaxf(mb, s[j]);
+      }
+      const float mn = fmaxf(m, mb);
+      const float alpha = __builtin_amdgcn_exp2f(m - mn);
+      l *= alpha;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) o[i] *= alpha;
+#pragma unroll
+      for (int j = 0; j < TB; ++j) {
+        const float p = __builtin_amdgcn_exp2f(s[j] - mn);
+        l += p;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          o[2 * w] = __builtin_fmaf(p, Elem<E>::lo(vv[j][w]), o[2 * w]);
+          o[2 * w + 1] = __builtin_fmaf(p, Elem<E>::hi(vv[j][w]), o[2 * w + 1]);
+        }
+      }
+      m = mn;
+    };
+
+    if (STAGES == 2) {
+      // two-stage software pipeline: the next batch's rows are in flight while this one is reduced
+      load(kb[0], vb[0], 0);
+      for (int j0 = 0; j0 < nb; j0 += 2 * TB) {
+        const bool more1 = j0 + TB < nb;
+        if (more1) load(kb[STAGES - 1], vb[STAGES - 1], j0 + TB);
+        compute(kb[0], vb[0], j0);
+        if (j0 + 2 * TB < nb) load(kb[0], vb[0], j0 + 2 * TB);
+        if (more1) compute(kb[STAGES - 1], vb[STAGES - 1], j0 + TB);
+      }
+    } else {
+      for (int j0 = 0; j0 < nb; j0 += TB) {
+        load(kb[0], vb[0], j0);
+        compute(kb[0], vb[0], j0);
+      }
+    }
+  }
+
+  if (!head_ok) return;
+  const float inv = 1.f / l;
+  float* op = opart + pr * D + (lane % LPH) * 8;
+  float4_t o0 = {o[0] * inv, o[1] * inv, o[2] * inv, o[3] * inv};
+  float4_t o1 = {o[4] * inv, o[5] * inv, o[6] * inv, o[7] * inv};
+  *reinterpret_cast<float4_t*>(op) = o0;
+  *reinterpret_cast<float4_t*>(op + 4) = o1;
+  if (lane % LPH == 0) {
+    ml[pr * 2] = m;
+    ml[pr * 2 + 1] = l;
+  }
+}
+
+// One piece of the balanced form for one head group: the piece's items (request, first token, count) are
+// streamed one after the other by this wave, one partial row per item.
+// (rec0, rec1) = the piece's lane record, already loaded by the caller
+template <typename E, int D, int TB, int STAGES>
+__device__ __forceinline__ void run_piece_rec(const ItemArgs& a, int hg, int4 rec0, int4 rec1) {
+  constexpr int LPH = D / 8;
+  constexpr int HPW = kWave / LPH;
+  const int lane = threadIdx.x & 63;
+  const int head = hg * HPW + lane / LPH;
+  const bool head_ok = head < a.H;
+  const int hclamp = head_ok ? head : a.H - 1;
+  const uint32_t lane_off = (uint32_t)(hclamp * D + (lane % LPH) * 8);
+  const int i0 = rec0.x, i1 = rec0.x + rec0.y;
+  for (int it = i0; it < i1; ++it) {
+    int4 meta = {rec0.z, rec0.w, rec1.x, 0};
+    if (it > i0) meta = a.items[it];  // request, first token, token count
+    const int b = meta.x, t0 = meta.y, t1 = meta.y + meta.z;
+    const int32_t* slots = a.slots + (a.offsets ? a.offsets[b] : (int64_t)b * a.table_stride);
+    const int myslot = slots[min(t0 + lane, t1 - 1)];
+    const u32x4 qv = ld16(a.q + (int64_t)b * a.q_stride + lane_off);
+    stream_item<E, D, TB, STAGES>(a.kc, a.vc, a.row_stride, slots, myslot, t0, t1, qv, lane_off, a.scale_log2e,
+                                  head_ok, a.opart, a.ml, (int64_t)it * a.H + hclamp);
+  }
+}
+
+template <typename E, int D, int TB, int STAGES>
+__device__ __forceinline__ void run_piece(const ItemArgs& a, int piece, int hg) {
+  // lane record: (first item, item count, then the first item's request / first token / count inline,
+  // so the first K/V rows are three dependent loads away from launch, not five)
+  run_piece_rec<E, D, TB, STAGES>(a, hg, a.lane_rec[2 * piece], a.lane_rec[2 * piece + 1]);
+}
+
+}  // namespace ph
