@@ -288,3 +288,53 @@ def test_prefix_and_post_entry_points(dev, dtype, B, P, H):
     torch.cuda.synchronize()
     ref = ref_decode_attention(case.q, case.k_rows, case.v_rows, case.full_lists())
     torch.testing.assert_close(out.cpu().float(), ref.float(), **TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_single_launch_path_with_uneven_groups(dev, dtype):
+    """Groups large enough for the path that runs the prefix and suffix phases in one launch, shaped to reach its
+    corners: prefixes of very different lengths (the short groups' later splits are empty), a group of more than
+    64 requests (two query tiles), more prefix units than workgroups (a workgroup runs several), requests with
+    no prefix and requests with no suffix, and a batch whose suffix stream is shorter than the prefix work."""
+    from parrotserve_amd import kernels
+
+    g = torch.Generator().manual_seed(21)
+    H, D = 40, 128
+    sizes = [40, 70, 33]
+    plens = [90, 2600, 700]
+    B = sum(sizes) + 4
+    n_rows = 6000
+    q = torch.randn(B, H, D, generator=g).to(dtype)
+    k = torch.randn(n_rows, H, D, generator=g).to(dtype)
+    v = torch.randn(n_rows, H, D, generator=g).to(dtype)
+    perm = torch.randperm(n_rows, generator=g)
+    pre, pos = [], 0
+    for n in plens:
+        pre.append(perm[pos:pos + n])
+        pos += n
+    gcu = [0]
+    for n in sizes:
+        gcu.append(gcu[-1] + n)
+    suf = []
+    for b in range(B):
+        n = int(torch.randint(0, 12, (1,), generator=g))
+        if b >= gcu[-1]:
+            n = max(n, 1)  # ungrouped requests need something to attend to
+        suf.append(perm[pos:pos + n])
+        pos += n
+    full = []
+    for b in range(B):
+        grp = next((i for i in range(len(sizes)) if gcu[i] <= b < gcu[i + 1]), None)
+        full.append(torch.cat([pre[grp] if grp is not None else perm[:0], suf[b]]))
+    ref = ref_decode_attention(q, k, v, full)
+    tables = kernels.DecodeTables.build([p.tolist() for p in pre], gcu, [s.tolist() for s in suf], dev, num_heads=H,
+                                        head_dim=D)
+    assert tables.plan is not None
+    out = kernels.decode_attention(q.to(dev), k.to(dev), v.to(dev), tables).cpu()
+    torch.testing.assert_close(out.float(), ref.float(), **TOL[dtype])
+    # the same batch as separate launches (no plan) must agree with the single launch
+    grid = kernels.DecodeTables.build([p.tolist() for p in pre], gcu, [s.tolist() for s in suf], dev, num_heads=H,
+                                      head_dim=D, balanced=False)
+    out2 = kernels.decode_attention(q.to(dev), k.to(dev), v.to(dev), grid).cpu()
+    torch.testing.assert_close(out2.float(), ref.float(), **TOL[dtype])
+    torch.testing.assert_close(out.float(), out2.float(), **TOL[dtype])
