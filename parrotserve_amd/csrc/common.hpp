@@ -145,6 +145,16 @@ struct KernelEvents {
 };
 KernelEvents take_kernel_events(int which);  // attention_api.hip; nulls unless the call was armed
 
+// Launch with the optional event pair; without events this is the ordinary launch call (the one that
+// stream capture and every tool expects), the extended call is only used when a caller asked for timing.
+#define PH_LAUNCH_TIMED(kernel, grid, block, shmem, stream, ev, ...)                                     \
+  do {                                                                                                   \
+    if ((ev).start || (ev).stop)                                                                         \
+      hipExtLaunchKernelGGL(kernel, grid, block, shmem, stream, (ev).start, (ev).stop, 0, __VA_ARGS__);  \
+    else                                                                                                 \
+      hipLaunchKernelGGL(kernel, grid, block, shmem, stream, __VA_ARGS__);                               \
+  } while (0)
+
 inline int launch_status() { return hipGetLastError() == hipSuccess ? PH_OK : PH_ERR_LAUNCH; }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

@@ -201,7 +201,7 @@ static int launch_partial_t(const PartialArgs& a, hipStream_t st) {
   if (waves == 0) return PH_OK;
   dim3 grid((unsigned)((waves + 3) / 4)), block(256);
   const KernelEvents ev = take_kernel_events(1);
-  hipExtLaunchKernelGGL((decode_partial_kernel<E, D, 4, 2>), grid, block, 0, st, ev.start, ev.stop, 0, a);
+  PH_LAUNCH_TIMED((decode_partial_kernel<E, D, 4, 2>), grid, block, 0, st, ev, a);
   return launch_status();
 }
 
@@ -213,7 +213,7 @@ static int launch_items_t(const ItemArgs& a, hipStream_t st) {
   if (waves == 0) return PH_OK;
   dim3 grid((unsigned)((waves + 3) / 4)), block(256);
   const KernelEvents ev = take_kernel_events(1);
-  hipExtLaunchKernelGGL((decode_items_kernel<E, D, 4, 2>), grid, block, 0, st, ev.start, ev.stop, 0, a);
+  PH_LAUNCH_TIMED((decode_items_kernel<E, D, 4, 2>), grid, block, 0, st, ev, a);
   return launch_status();
 }
 
@@ -225,7 +225,7 @@ static int launch_merge_t(const MergeArgs& a, hipStream_t st) {
   if (groups == 0) return PH_OK;
   dim3 grid((unsigned)groups), block(256);
   const KernelEvents ev = take_kernel_events(2);
-  hipExtLaunchKernelGGL((merge_kernel<E, D>), grid, block, 0, st, ev.start, ev.stop, 0, a);
+  PH_LAUNCH_TIMED((merge_kernel<E, D>), grid, block, 0, st, ev, a);
   return launch_status();
 }
 

@@ -960,13 +960,13 @@ static int launch_prefix_t(const PrefixArgs& a, int num_groups, int max_group_re
     dim3 grid(a.n_splits, a.H, num_groups), block(256);
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefix_mfma_kernel<E, 1>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, tile_lds_bytes<1>());
-    hipExtLaunchKernelGGL((prefix_mfma_kernel<E, 1>), grid, block, tile_lds_bytes<1>(), st, ev.start, ev.stop, 0, a, 1);
+    PH_LAUNCH_TIMED((prefix_mfma_kernel<E, 1>), grid, block, tile_lds_bytes<1>(), st, ev, a, 1);
   } else {                     // eight waves, 64-query tiles
     const int mtiles = (max_group_reqs + 63) / 64;
     dim3 grid(a.n_splits, a.H, num_groups * mtiles), block(512);
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefix_mfma8_kernel<E>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, kTile8Lds);
-    hipExtLaunchKernelGGL((prefix_mfma8_kernel<E>), grid, block, kTile8Lds, st, ev.start, ev.stop, 0, a, mtiles);
+    PH_LAUNCH_TIMED((prefix_mfma8_kernel<E>), grid, block, kTile8Lds, st, ev, a, mtiles);
   }
   return launch_status();
 }
@@ -1007,7 +1007,7 @@ static int launch_fused_t(const PrefixArgs& a, const ItemArgs& ia, int num_group
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&decode_fused_kernel<E>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, kTile8Lds);
   const KernelEvents ev = take_kernel_events(1);
-  hipExtLaunchKernelGGL((decode_fused_kernel<E>), dim3(grid), dim3(512), kTile8Lds, st, ev.start, ev.stop, 0, a, mtiles,
+  PH_LAUNCH_TIMED((decode_fused_kernel<E>), dim3(grid), dim3(512), kTile8Lds, st, ev, a, mtiles,
                         n_units, ia);
   return launch_status();
 }

@@ -338,3 +338,39 @@ def test_single_launch_path_with_uneven_groups(dev, dtype):
     out2 = kernels.decode_attention(q.to(dev), k.to(dev), v.to(dev), grid).cpu()
     torch.testing.assert_close(out2.float(), ref.float(), **TOL[dtype])
     torch.testing.assert_close(out.float(), out2.float(), **TOL[dtype])
+
+
+def test_decode_attention_replays_from_a_captured_graph(dev):
+    """The decode step (single-launch prefix + suffix, merge) recorded into a graph: every replay, with eager
+    work and synchronisation between replays, must reproduce the eager result for the inputs then in place."""
+    from parrotserve_amd import kernels, synth
+
+    g = torch.Generator().manual_seed(23)
+    s = torch.randint(1, 120, (48,), generator=g).tolist()
+    case = synth.make_decode_case("graph", 23, torch.float16, 1, 48, 900, s, 8, 128, 1 << 14)
+    kc, vc = synth.pool_to_device(case.k_rows, case.v_rows, case.used_slots, case.pool_slots, dev)
+    tables = kernels.DecodeTables.build(case.pool_lists(case.prefix_lists), case.group_req_cu,
+                                        case.pool_lists(case.suffix_lists), dev, num_heads=8, head_dim=128)
+    q_static = case.q.to(dev)
+    out_static = torch.empty_like(q_static)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # warm-up on the capture stream: workspace and lazy state exist before recording
+        kernels.decode_attention(q_static, kc, vc, tables, out=out_static)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        kernels.decode_attention(q_static, kc, vc, tables, out=out_static)
+    gq = torch.Generator(device=dev).manual_seed(5)
+    for rep in range(4):
+        q_new = torch.randn(q_static.shape, generator=gq, device=dev, dtype=torch.float16)
+        eager = kernels.decode_attention(q_new, kc, vc, tables)  # eager work between the replays
+        torch.cuda.synchronize()
+        q_static.copy_(q_new)
+        out_static.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_static, eager), f"replay {rep} differs from the eager result"
+    ref = ref_decode_attention(q_static.cpu(), case.k_rows, case.v_rows, case.full_lists())
+    torch.testing.assert_close(out_static.cpu().float(), ref.float(), **TOL[torch.float16])
