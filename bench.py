@@ -177,6 +177,12 @@ def extras(torch, dev):
         kernels.vllm_reshape_and_cache(ki.view(T, H4, D), vi.view(T, H4, D), kc4, vc4, new_slots)
 
     t_app = _time_gpu(torch, append_step)
+
+    def fused_step():
+        qi, ki, vi = qkvs[rot.next()].chunk(3, dim=-1)
+        kernels.rope_and_cache(pos, qi, ki, vi, cache, D, kc4, vc4, new_slots)
+
+    t_fused = _time_gpu(torch, fused_step)
     ctx = [c4.used_slots[torch.cat([p, n])].tolist() for p, n in zip(c4.parent_lists, c4.new_lists)]
     ptab = kernels.PrefillTables.build(c4.q_lens, ctx, dev)
     qc = q4.reshape(T, H4, D).contiguous()
@@ -189,6 +195,10 @@ def extras(torch, dev):
     app_bytes = 2 * 2 * T * H4 * D * 2
     out["c4_kv_append"] = {"tokens": T, "us": t_app * 1e6, "GB/s": app_bytes / t_app / 1e9,
                            "frac_hbm": app_bytes / t_app / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": app_bytes}
+    fused_bytes = rope_bytes + 3 * T * H4 * D * 2  # + v read, K and V rows written to their slots
+    out["c4_rope_append_fused"] = {"tokens": T, "us": t_fused * 1e6, "GB/s": fused_bytes / t_fused / 1e9,
+                                   "frac_hbm": fused_bytes / t_fused / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": fused_bytes,
+                                   "unfused_us": (t_rope + t_app) * 1e6}
     out["c4_prefill"] = {"tokens": T, "chunks": len(c4.q_lens), "ms": t_pre * 1e3, "flops": flops,
                          "TFLOP/s": flops / t_pre / 1e12, "frac_mfma_peak": flops / t_pre / 1e12 / MFMA_F16_PEAK_TFLOPS,
                          "tokens/s/layer": T / t_pre}

@@ -132,15 +132,35 @@ __global__ __launch_bounds__(256) void rope_vec(const int64_t* __restrict__ posi
   const uint16_t* sr = sin_base + p * cs_stride;
   const int upd = half_rot >> 3;  // units per head
   const int units = (hq + hk) * upd;
-  for (int u = threadIdx.x; u < units; u += 256) {
-    const int h = u / upd;
-    const int c = (u - h * upd) * 8;
-    uint16_t* base = h < hq ? q + t * q_stride_n + (int64_t)h * q_stride_h
-                            : k + t * k_stride_n + (int64_t)(h - hq) * k_stride_h;
-    u32x4 x = ld16(base + c), y = ld16(base + half_rot + c);
-    rotate8<E>(x, y, ld16(cr + c), ld16(sr + c));
-    st16(base + c, x);
-    st16(base + half_rot + c, y);
+  // four units per thread and pass: all their loads are issued before the first rotation, so a thread keeps
+  // up to sixteen 16-byte loads in flight instead of four
+  constexpr int UN = 4;
+  for (int u0 = threadIdx.x; u0 < units; u0 += 256 * UN) {
+    uint16_t* base[UN];
+    int cc[UN];
+    u32x4 x[UN], y[UN], cs[UN], sn[UN];
+#pragma unroll
+    for (int j = 0; j < UN; ++j) {
+      const int u = u0 + j * 256;
+      const bool ok = u < units;
+      const int uu = ok ? u : u0;
+      const int h = uu / upd;
+      cc[j] = (uu - h * upd) * 8;
+      base[j] = h < hq ? q + t * q_stride_n + (int64_t)h * q_stride_h
+                       : k + t * k_stride_n + (int64_t)(h - hq) * k_stride_h;
+      x[j] = ld16(base[j] + cc[j]);
+      y[j] = ld16(base[j] + half_rot + cc[j]);
+      cs[j] = ld16(cr + cc[j]);
+      sn[j] = ld16(sr + cc[j]);
+    }
+#pragma unroll
+    for (int j = 0; j < UN; ++j) {
+      if (u0 + j * 256 < units) {
+        rotate8<E>(x[j], y[j], cs[j], sn[j]);
+        st16(base[j] + cc[j], x[j]);
+        st16(base[j] + half_rot + cc[j], y[j]);
+      }
+    }
   }
 }
 
