@@ -490,15 +490,21 @@ struct NoMid {
   __device__ __forceinline__ void operator()() const {}
 };
 
-template <typename E, bool CAUSAL, int TQ, typename Mid = NoMid>
+template <typename E, bool CAUSAL, int TQ, typename Mid = NoMid, int SUB = 1>
 __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* __restrict__ kc,
                                            const uint16_t* __restrict__ vc, int64_t row_stride, int head,
                                            float scale_log2e, char* smem, float16_t (&ofold)[4 / TQ], float& mfin,
                                            float& lfin, Mid mid = Mid()) {
-  constexpr int QB = 8 / TQ;      // query blocks = waves sharing a tile
-  constexpr int NST = 8 / TQ;     // stages per token group
-  constexpr int A = NST - 1;      // tiles in flight ahead of the current one
-  constexpr int LPT = 16 / QB;    // row-group loads per wave per tile
+  // SUB: 32-token sub-tiles per step of a token group (a ring stage holds SUB of them back to back).  Two
+  // halve the per-step costs (barrier, waits, staging bookkeeping, one softmax bookkeeping per 64 tokens) and
+  // give the scheduler two independent score products to overlap with the vector work.
+  constexpr int QB = 8 / TQ;            // query blocks = waves sharing a tile
+  constexpr int STEP = kTile * SUB;     // tokens per step
+  constexpr int SBYTES = kStage * SUB;  // bytes per ring stage
+  constexpr int NST = 8 / (TQ * SUB);   // stages per token group
+  constexpr int A = NST - 1;            // steps in flight ahead of the current one
+  constexpr int LPT = 16 * SUB / QB;    // row-group loads per wave per step
+  static_assert(NST >= 2 && LPT >= 1 && LPT <= 8, "unsupported tile split");
   constexpr int NDB = 4 / TQ;     // dim blocks a wave finishes
   // decode reads every prefix row once per launch (streaming policy); prefill tiles are re-read by the
   // other query tiles of the chunk and should stay in L2
@@ -509,7 +515,7 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
   const int lane = threadIdx.x & 63;
   const int w8 = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), g = w8 / QB, qb = w8 % QB;
   const int h = lane >> 5, ql = lane & 31;
-  char* gl = smem + g * NST * kStage;
+  char* gl = smem + g * NST * SBYTES;
   int32_t* win = reinterpret_cast<int32_t*>(smem + kWinOff);
   const int s0 = wk.s0, s1 = wk.s1;
 #pragma unroll
@@ -528,31 +534,32 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
   // brings row groups qb LPT .. + LPT - 1 (same swizzles as the four-wave form)
   const int tl = lane >> 4, c = lane & 15;
   const uint32_t row_bytes = (uint32_t)(row_stride * 2);
-  const bool isv = qb * LPT >= 8;
+  const int sub0 = (qb * LPT) / 16;            // sub-tile, K or V half and first row group of this wave's loads
+  const bool isv = ((qb * LPT) & 15) >= 8;
   const int r0 = (qb * LPT) & 7;
   const char* gbase[LPT];
 #pragma unroll
   for (int i = 0; i < LPT; ++i)
     gbase[i] = isv ? reinterpret_cast<const char*>(vc + (int64_t)head * kPD + ((c ^ (4 * tl)) * 8))
                    : reinterpret_cast<const char*>(kc + (int64_t)head * kPD + ((c ^ ((4 * (r0 + i) + tl) & 15)) * 8));
-  const uint32_t dst0 = lds_addr_of(gl) + (isv ? kVtOff : 0) + r0 * 1024;
+  const uint32_t dst0 = lds_addr_of(gl) + sub0 * kStage + (isv ? kVtOff : 0) + r0 * 1024;
   // rows of the group's tile that starts at token tb, into ring stage `stage`
   auto fetch_rows = [&](int tb, int stage) {
     uint32_t sl[LPT];
 #pragma unroll
-    for (int i = 0; i < LPT; ++i) sl[i] = (uint32_t)win[tb - win0 + 4 * (r0 + i) + tl];
-    const uint32_t kb = dst0 + stage * kStage;
+    for (int i = 0; i < LPT; ++i) sl[i] = (uint32_t)win[tb - win0 + kTile * sub0 + 4 * (r0 + i) + tl];
+    const uint32_t kb = dst0 + stage * SBYTES;
 #pragma unroll
     for (int i = 0; i < LPT; ++i) lds_dma16<NTLOAD>(gbase[i] + (uint64_t)sl[i] * row_bytes, kb + i * 1024);
   };
-  const int ntile = (s1 - s0 + kTile - 1) / kTile;
+  const int ntile = (s1 - s0 + STEP - 1) / STEP;
   const int iters = (ntile + TQ - 1) / TQ;                 // same for all eight waves
   const int my_iters = ntile > g ? (ntile - g + TQ - 1) / TQ : 0;  // tiles of this token group
   __syncthreads();                                         // window visible
   // the whole ring is filled up front: tiles 0 .. A (the main loop issues tile it + A at step it >= 1)
 #pragma unroll
   for (int j = 0; j < NST; ++j)
-    if (j < my_iters) fetch_rows(s0 + kTile * (g + TQ * j), j);
+    if (j < my_iters) fetch_rows(s0 + STEP * (g + TQ * j), j);
 
   // Q as the B operand: column = query 32 qb + ql, contraction chunk (h, s) = dims 64h + 8s .. +8
   u32x4 qop[8];
@@ -574,7 +581,7 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
 
   // Operand read addresses of ring stage 0 (and of stage 4, beyond the reach of the 16-bit immediate).
   // K: row ql, chunk (8h + s) swizzled by the row; V: the transposing read's row/column of this lane.
-  constexpr int NHI = NST > 4 ? 2 : 1;
+  constexpr int NHI = NST * SBYTES > 65536 ? 2 : 1;
   uint32_t kaddr[NHI][8], vaddr[NHI][4];
   {
     const uint32_t gl_a = lds_addr_of(gl);
@@ -586,12 +593,12 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
     for (int hi = 0; hi < NHI; ++hi) {
 #pragma unroll
       for (int s = 0; s < 8; ++s) {
-        kaddr[hi][s] = gl_a + hi * 4 * kStage + ql * 256 + (((8 * h + s) ^ (ql & 15)) * 16);
+        kaddr[hi][s] = gl_a + hi * 65536 + ql * 256 + (((8 * h + s) ^ (ql & 15)) * 16);
         asm("" : "+v"(kaddr[hi][s]));  // keep the sum in one register (otherwise it is re-added at every read)
       }
 #pragma unroll
       for (int db = 0; db < 4; ++db) {
-        vaddr[hi][db] = gl_a + hi * 4 * kStage + kVtOff + trow * 256 + (sl & 1) * 8 + (((4 * db + tcol) ^ tswz) * 16);
+        vaddr[hi][db] = gl_a + hi * 65536 + kVtOff + trow * 256 + (sl & 1) * 8 + (((4 * db + tcol) ^ tswz) * 16);
         asm("" : "+v"(vaddr[hi][db]));
       }
     }
@@ -603,64 +610,77 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
    for (int stage = 0; stage < NST; ++stage) {
     const int it = it0 + stage;
     if (it >= iters) break;
-    const int tb = s0 + kTile * (g + TQ * it);
+    const int tb = s0 + STEP * (g + TQ * it);
     // Tile `it` of this group has landed once at most the (A - 1) LPT loads issued after it are outstanding
     // (near the end fewer were issued, so everything is awaited); the barrier publishes all parts of the
     // tile and tells everyone that the stage read in the previous step is free again.
     if (it + A - 1 < my_iters) wait_vmcnt<(A - 1) * LPT>(); else wait_vmcnt<0>();
     __syncthreads();
     {
-      const int front = s0 + kTile * TQ * (it + A);          // first token of the step being staged
+      const int front = s0 + STEP * TQ * (it + A);           // first token of the step being staged
       if (front < s1 && front >= win0 + kWin) {              // workgroup-uniform: slide the slot window
         win0 += kWin;
         fill_window();
         __syncthreads();
       }
-      if (it > 0 && it + A < my_iters) fetch_rows(front + kTile * g, (stage + A) % NST);
+      if (it > 0 && it + A < my_iters) fetch_rows(front + STEP * g, (stage + A) % NST);
     }
     if (it >= my_iters || tb > wave_last) continue;           // wave-uniform
-    const int shi = stage >> 2, slo = (stage & 3) * kStage;
-
-    u32x4 ka[8];
+    float16_t sacc[SUB];
 #pragma unroll
-    for (int s = 0; s < 8; ++s) ka[s] = lds_ld16_a(kaddr[shi][s] + slo);
-    __builtin_amdgcn_sched_barrier(0);
-    float16_t sacc;
-    {
+    for (int sb = 0; sb < SUB; ++sb) {
+      const int off = stage * SBYTES + sb * kStage;
+      const int shi = off >> 16, slo = off & 65535;
+      u32x4 ka[8];
+#pragma unroll
+      for (int s = 0; s < 8; ++s) ka[s] = lds_ld16_a(kaddr[shi][s] + slo);
+      if (SUB == 1) __builtin_amdgcn_sched_barrier(0);
       const float16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-      sacc = Mfma32<E>::run(ka[0], qop[0], zero);
+      sacc[sb] = Mfma32<E>::run(ka[0], qop[0], zero);
 #pragma unroll
-      for (int s = 1; s < 8; ++s) sacc = Mfma32<E>::run(ka[s], qop[s], sacc);
+      for (int s = 1; s < 8; ++s) sacc[sb] = Mfma32<E>::run(ka[s], qop[s], sacc[sb]);
     }
     // A operand of O^T += V^T P^T (row = dim 32db + ql, contraction = the 8 tokens of (h, u)): two
     // transposing reads, tokens 16u + 4h + {0..3} and 16u + 8 + 4h + {0..3}
-    u32x4 va[4][2];
+    u32x4 va[SUB][4][2];
 #pragma unroll
-    for (int db = 0; db < 4; ++db)
+    for (int sb = 0; sb < SUB; ++sb) {
+      const int off = stage * SBYTES + sb * kStage;
+      const int shi = off >> 16, slo = off & 65535;
 #pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        const u32x2 lo = lds_tr16_a(vaddr[shi][db] + slo + (16 * u) * 256);
-        const u32x2 hi = lds_tr16_a(vaddr[shi][db] + slo + (16 * u + 8) * 256);
-        va[db][u] = u32x4{lo[0], lo[1], hi[0], hi[1]};
-      }
-    __builtin_amdgcn_sched_barrier(0);
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const u32x2 lo = lds_tr16_a(vaddr[shi][db] + slo + (16 * u) * 256);
+          const u32x2 hi = lds_tr16_a(vaddr[shi][db] + slo + (16 * u + 8) * 256);
+          va[sb][db][u] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+        }
+    }
+    if (SUB == 1) __builtin_amdgcn_sched_barrier(0);
 
-    const bool full = tb + kTile <= s1 && (!CAUSAL || tb + kTile - 1 <= wk.causal_off + 32 * qb);
-    float x[16];
+    const bool full = tb + STEP <= s1 && (!CAUSAL || tb + STEP - 1 <= wk.causal_off + 32 * qb);
+    float x[SUB][16];
     if (full) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) x[r] = sacc[r];
+      for (int sb = 0; sb < SUB; ++sb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) x[sb][r] = sacc[sb][r];
     } else {
       const int tmax = CAUSAL ? min(s1 - 1, wk.causal_off + 32 * qb + ql) : s1 - 1;  // last visible token
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int t = 8 * (r >> 2) + 4 * h + (r & 3);
-        x[r] = (tb + t <= tmax) ? sacc[r] : -INFINITY;
-      }
-    }
-    float mloc = fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3]));
+      for (int sb = 0; sb < SUB; ++sb)
 #pragma unroll
-    for (int r = 4; r < 16; r += 4) mloc = fmaxf(mloc, fmaxf(fmaxf(x[r], x[r + 1]), fmaxf(x[r + 2], x[r + 3])));
+        for (int r = 0; r < 16; ++r) {
+          const int t = kTile * sb + 8 * (r >> 2) + 4 * h + (r & 3);
+          x[sb][r] = (tb + t <= tmax) ? sacc[sb][r] : -INFINITY;
+        }
+    }
+    float mloc = -INFINITY;
+#pragma unroll
+    for (int sb = 0; sb < SUB; ++sb)
+#pragma unroll
+      for (int r = 0; r < 16; r += 4)
+        mloc = fmaxf(mloc, fmaxf(fmaxf(x[sb][r], x[sb][r + 1]), fmaxf(x[sb][r + 2], x[sb][r + 3])));
     mloc = half_swap_max(mloc) * scale_log2e;  // scale > 0 keeps the order
     mtrue = fmaxf(mtrue, mloc);
     // lazy exponent reference: moves only when the maximum has outgrown it by more than kSlack
@@ -680,23 +700,26 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
         for (int r = 0; r < 16; ++r) asm volatile("v_mul_f32 %0, %0, %1" : "+v"(oacc[db][r]) : "v"(alpha));
       asm volatile("s_nop 7" ::: "memory");
     }
-#pragma unroll
-    for (int r = 0; r < 16; ++r) x[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(x[r], scale_log2e, -mref));
     // P^T packed straight into B-operand form; the denominator sums the rounded values the product uses
     float ps = 0.f;
-    u32x4 pop[2];
 #pragma unroll
-    for (int u = 0; u < 2; ++u)
+    for (int sb = 0; sb < SUB; ++sb) {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        pop[u][e] = pack2<E>(x[8 * u + 2 * e], x[8 * u + 2 * e + 1]);
-        ps = Elem<E>::dot2(pop[u][e], Elem<E>::kOnes, ps);
-      }
+      for (int r = 0; r < 16; ++r) x[sb][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(x[sb][r], scale_log2e, -mref));
+      u32x4 pop[2];
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          pop[u][e] = pack2<E>(x[sb][8 * u + 2 * e], x[sb][8 * u + 2 * e + 1]);
+          ps = Elem<E>::dot2(pop[u][e], Elem<E>::kOnes, ps);
+        }
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int u = 0; u < 2; ++u) oacc[db] = Mfma32<E>::run(va[sb][db][u], pop[u], oacc[db]);
+    }
     lsum = lsum * alpha + ps;
-#pragma unroll
-    for (int db = 0; db < 4; ++db)
-#pragma unroll
-      for (int u = 0; u < 2; ++u) oacc[db] = Mfma32<E>::run(va[db][u], pop[u], oacc[db]);
    }
   }
 
@@ -895,7 +918,7 @@ __global__ __launch_bounds__(512) void decode_fused_kernel(PrefixArgs pa, int mt
 }
 
 // Prefill with parent context, eight waves: workgroup = (head, tile of 32 * (8 / TQ) queries of one chunk)
-template <typename E, int TQ>
+template <typename E, int TQ, int SUB>
 __global__ __launch_bounds__(512) void prefill_mfma8_kernel(PrefillArgs a) {
   constexpr int QB = 8 / TQ, NDB = 4 / TQ, QT = 32 * QB;
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -924,7 +947,7 @@ __global__ __launch_bounds__(512) void prefill_mfma8_kernel(PrefillArgs a) {
   wk.s1 = min(kvn, wk.causal_off + nq);  // the last live query sees tokens up to causal_off + nq - 1
   float16_t of[NDB];
   float m, l;
-  attn_tile8<E, true, TQ>(wk, a.kc, a.vc, a.row_stride, head, a.scale_log2e, smem, of, m, l);
+  attn_tile8<E, true, TQ, NoMid, SUB>(wk, a.kc, a.vc, a.row_stride, head, a.scale_log2e, smem, of, m, l);
   const int lane = threadIdx.x & 63, w8 = threadIdx.x >> 6, g = w8 / QB, qb = w8 % QB, h = lane >> 5, ql = lane & 31;
   const int q = 32 * qb + ql;
   if (q < nq) {
@@ -971,15 +994,15 @@ static int launch_prefix_t(const PrefixArgs& a, int num_groups, int max_group_re
   return launch_status();
 }
 
-template <typename E, int TQ>
+template <typename E, int TQ, int SUB>
 static int launch_prefill_tq(const PrefillArgs& a, int64_t num_tokens, hipStream_t st) {
   constexpr int QT = 32 * (8 / TQ);  // queries per workgroup tile
   hipLaunchKernelGGL(prefill_tiles_kernel, dim3(1), dim3(64), 0, st, a.q_cu, a.num_chunks, a.tile_cu, QT);
-  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_mfma8_kernel<E, TQ>),
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_mfma8_kernel<E, TQ, SUB>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, kTile8Lds);
   const int hx = (a.H + 7) / 8 * 8;  // keeps head == linear id mod 8 for every tile row
   const int64_t max_tiles = num_tokens / QT + a.num_chunks;  // >= sum of ceil(n_c / QT)
-  hipLaunchKernelGGL((prefill_mfma8_kernel<E, TQ>), dim3(hx, (unsigned)max_tiles), dim3(512), kTile8Lds, st, a);
+  hipLaunchKernelGGL((prefill_mfma8_kernel<E, TQ, SUB>), dim3(hx, (unsigned)max_tiles), dim3(512), kTile8Lds, st, a);
   return launch_status();
 }
 
@@ -988,9 +1011,9 @@ static int launch_prefill_tq(const PrefillArgs& a, int64_t num_tokens, hipStream
 template <typename E>
 static int launch_prefill_t(const PrefillArgs& a, int64_t num_tokens, hipStream_t st) {
   const int64_t avg = num_tokens / (a.num_chunks > 0 ? a.num_chunks : 1);
-  if (avg >= 192) return launch_prefill_tq<E, 1>(a, num_tokens, st);
-  if (avg >= 96) return launch_prefill_tq<E, 2>(a, num_tokens, st);
-  return launch_prefill_tq<E, 4>(a, num_tokens, st);
+  if (avg >= 192) return launch_prefill_tq<E, 1, 2>(a, num_tokens, st);  // 64-token steps (measured 4 % faster)
+  if (avg >= 96) return launch_prefill_tq<E, 2, 1>(a, num_tokens, st);
+  return launch_prefill_tq<E, 4, 1>(a, num_tokens, st);
 }
 
 template <typename E>
