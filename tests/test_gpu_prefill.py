@@ -135,3 +135,14 @@ def test_prefill_heads_not_multiple_of_eight_and_tail_tiles(dev):
         case = synth.make_prefill_case("h", 900 + H, torch.bfloat16, q_lens, parent, H, 128, 1 << 13)
         out, ref = run_prefill_case(case, dev)
         torch.testing.assert_close(out.float(), ref.float(), **TOL[torch.bfloat16])
+
+
+@pytest.mark.parametrize("D,H", [(64, 6), (256, 2)])
+def test_prefill_other_head_sizes(dev, D, H):
+    """Head sizes the matrix-core kernel does not cover run every query row through the per-request kernel
+    over its visible slots; same results."""
+    from parrotserve_amd import synth
+
+    case = synth.make_prefill_case("hd", 300 + D, torch.float16, [33, 5, 70], 41, H, D, 1 << 12)
+    out, ref = run_prefill_case(case, dev)
+    torch.testing.assert_close(out.float(), ref.float(), **TOL[torch.float16])
