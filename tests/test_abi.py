@@ -63,6 +63,22 @@ def test_argument_validation_needs_no_gpu():
     rc = lib.ph_decode_attention(1, 1, 1, 1, 4, 2, 80, 0, 160, 160, 160, 1.0, 0, None, None, None, None, 0,
                                  None, None, 0, 0, None, 0, 0, None, None, 0, None)
     assert rc == _lib.PH_ERR_HEAD_DIM
+    # fused per-layer ops and the table patch
+    assert lib.ph_add_rms_norm(None, None, None, None, 1e-6, 4, 64, 64, 64, 64, 9, 1, None) == _lib.PH_ERR_DTYPE
+    assert lib.ph_add_rms_norm(None, None, None, None, 1e-6, 4, 64, 32, 64, 64, 0, 1, None) == _lib.PH_ERR_ARG  # stride < n
+    assert lib.ph_add_rms_norm(None, None, None, None, 1e-6, 0, 64, 64, 64, 64, 0, 1, None) == _lib.PH_OK       # no rows
+    assert lib.ph_add_rms_norm(None, None, None, None, 1e-6, 4, 64, 64, 64, 64, 0, 1, None) == _lib.PH_ERR_ARG  # null pointers
+    assert lib.ph_silu_mul(None, None, None, 4, 0, 8, 8, 8, 0, None) == _lib.PH_ERR_ARG
+    assert lib.ph_silu_mul(None, None, None, 4, 8, 8, 8, 8, 5, None) == _lib.PH_ERR_DTYPE
+    assert lib.ph_rope_append(None, None, None, None, None, None, None, None, 0, 4, 2, 2, 128, 130, 256, 256, 256, 256,
+                              0, None) == _lib.PH_ERR_ARG  # rotary size beyond the head size
+    assert lib.ph_rope_append(None, None, None, None, None, None, None, None, 7, 4, 2, 2, 128, 128, 256, 256, 256, 256,
+                              0, None) == _lib.PH_ERR_ARG  # unknown index type
+    assert lib.ph_rope_append(None, None, None, None, None, None, None, None, 0, 0, 2, 2, 128, 128, 256, 256, 256, 256,
+                              0, None) == _lib.PH_OK       # no tokens
+    assert lib.ph_suffix_tables_append(None, 64, None, None, None, -1, None) == _lib.PH_ERR_ARG
+    assert lib.ph_suffix_tables_append(None, 64, None, None, None, 0, None) == _lib.PH_OK
+    assert lib.ph_suffix_tables_append(None, 64, None, None, None, 3, None) == _lib.PH_ERR_ARG
 
 
 def test_cpu_tensors_are_refused_loudly():
