@@ -212,7 +212,7 @@ __global__ __launch_bounds__(256) void rope_append_vec(const int64_t* __restrict
       const int c = (u - h * upd) * 8;
       const bool is_k = h >= hq;
       uint16_t* base = is_k ? k + t * k_stride + (int64_t)(h - hq) * D : q + t * q_stride + (int64_t)h * D;
-      u32x4 x = ld16(base + c), y = ld16(base + half + c);
+      u32x4 x = ld16_nt(base + c), y = ld16_nt(base + half + c);
       rotate8<E>(x, y, ld16(cr + c), ld16(sr + c));
       st16(base + c, x);
       st16(base + half + c, y);
@@ -223,7 +223,7 @@ __global__ __launch_bounds__(256) void rope_append_vec(const int64_t* __restrict
       }
     } else {
       const int c = (u - rot_units) * 8;
-      st16(vc + c, ld16(v + t * v_stride + c));
+      st16(vc + c, ld16_nt(v + t * v_stride + c));
     }
   }
 }

@@ -37,7 +37,7 @@ __global__ __launch_bounds__(kNormThreads) void rms_norm_vec(uint16_t* __restric
   for (int i = 0; i < ITERS; ++i) {
     const int c = threadIdx.x + i * kNormThreads;
     if (c < chunks) {
-      v[i] = ld16(xr + c * 8);
+      v[i] = ld16_nt(xr + c * 8);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const float a = Elem<E>::lo(v[i][j]), b = Elem<E>::hi(v[i][j]);
