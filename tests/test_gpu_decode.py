@@ -374,3 +374,44 @@ def test_decode_attention_replays_from_a_captured_graph(dev):
         assert torch.equal(out_static, eager), f"replay {rep} differs from the eager result"
     ref = ref_decode_attention(q_static.cpu(), case.k_rows, case.v_rows, case.full_lists())
     torch.testing.assert_close(out_static.cpu().float(), ref.float(), **TOL[torch.float16])
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_randomized_grouped_decode_shapes(dev, seed):
+    """Seeded random batches: 1-3 prefix groups of 1-140 requests, prefixes of 1-1500 tokens (not multiples of
+    any tile size), suffixes of 0-90 tokens, odd head counts, a few ungrouped requests, both element types."""
+    from parrotserve_amd import kernels
+
+    g = torch.Generator().manual_seed(1000 + seed)
+    ri = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))  # noqa: E731
+    dtype = torch.float16 if seed % 2 == 0 else torch.bfloat16
+    H, D = ri(1, 9), 128
+    n_groups = ri(1, 3)
+    sizes = [ri(1, 140) if i == 0 else ri(1, 50) for i in range(n_groups)]
+    plens = [ri(1, 1500) for _ in range(n_groups)]
+    loners = ri(0, 3)
+    B = sum(sizes) + loners
+    n_rows = sum(plens) + 90 * B + 8
+    q = torch.randn(B, H, D, generator=g).to(dtype)
+    k = torch.randn(n_rows, H, D, generator=g).to(dtype)
+    v = torch.randn(n_rows, H, D, generator=g).to(dtype)
+    perm = torch.randperm(n_rows, generator=g)
+    pre, pos = [], 0
+    for n in plens:
+        pre.append(perm[pos:pos + n])
+        pos += n
+    gcu = [0]
+    for n in sizes:
+        gcu.append(gcu[-1] + n)
+    suf, full = [], []
+    for b in range(B):
+        grp = next((i for i in range(n_groups) if gcu[i] <= b < gcu[i + 1]), None)
+        n = ri(0, 90) if grp is not None else ri(1, 90)
+        suf.append(perm[pos:pos + n])
+        pos += n
+        full.append(torch.cat([pre[grp] if grp is not None else perm[:0], suf[-1]]))
+    ref = ref_decode_attention(q, k, v, full)
+    tables = kernels.DecodeTables.build([p.tolist() for p in pre], gcu, [s.tolist() for s in suf], dev, num_heads=H,
+                                        head_dim=D)
+    out = kernels.decode_attention(q.to(dev), k.to(dev), v.to(dev), tables).cpu()
+    torch.testing.assert_close(out.float(), ref.float(), **TOL[dtype])

@@ -146,3 +146,20 @@ def test_prefill_other_head_sizes(dev, D, H):
     case = synth.make_prefill_case("hd", 300 + D, torch.float16, [33, 5, 70], 41, H, D, 1 << 12)
     out, ref = run_prefill_case(case, dev)
     torch.testing.assert_close(out.float(), ref.float(), **TOL[torch.float16])
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_randomized_prefill_shapes(dev, seed):
+    """Seeded random chunk sets: 1-6 chunks of 1-400 new tokens over parents of 0-700 tokens, odd head counts,
+    both element types (covers every query-tile size and partial tiles on both axes)."""
+    from parrotserve_amd import synth
+
+    g = torch.Generator().manual_seed(2000 + seed)
+    ri = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))  # noqa: E731
+    dtype = torch.float16 if seed % 2 else torch.bfloat16
+    chunks = ri(1, 6)
+    hi = [30, 120, 400][seed % 3]
+    q_lens = [ri(1, hi) for _ in range(chunks)]
+    case = synth.make_prefill_case("rnd", 2000 + seed, dtype, q_lens, ri(0, 700), ri(1, 6), 128, 1 << 13)
+    out, ref = run_prefill_case(case, dev)
+    torch.testing.assert_close(out.float(), ref.float(), **TOL[dtype])
