@@ -137,6 +137,22 @@ def extras(torch, dev):
     nbytes = 2 * src.numel() * H * D * 2
     out["c3_token_move"] = {"rows": src.numel(), "row_bytes": H * D * 2, "us": t * 1e6, "GB/s": nbytes / t / 1e9,
                             "frac_hbm": nbytes / t / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": nbytes}
+    # --- the same 65,536 rows gathered out of the block-structured layouts (block 16, x 8) of a 4M-slot cache:
+    # whole blocks in random order (a context that owns its blocks) and fully random slots -----------------------
+    bs, x = 16, 8
+    gen = torch.Generator().manual_seed(3)
+    blocks = torch.randperm(pool // bs, generator=gen)[: src.numel() // bs]
+    runs = (blocks[:, None] * bs + torch.arange(bs)[None, :]).reshape(-1).to(dev)
+    dest = torch.empty((src.numel(), H, D), dtype=torch.float16, device=dev)
+    rows = torch.arange(src.numel(), device=dev)
+    for name, cache, fn in (("k", kc.view(pool // bs, H, D // x, bs, x), kernels.move_tokens_from_blocked_k_cache),
+                            ("v", kc.view(pool // bs, H, D, bs), kernels.move_tokens_from_blocked_v_cache)):
+        for pat, slots in (("block_runs", runs), ("random_slots", src)):
+            t = _time_gpu(torch, lambda: fn(cache, dest, slots, rows))
+            out[f"c3_blocked_{name}_gather_{pat}"] = {"rows": src.numel(), "us": t * 1e6, "GB/s": nbytes / t / 1e9,
+                                                      "frac_hbm": nbytes / t / 1e9 / HBM_PEAK_GBS,
+                                                      "algorithmic_bytes": nbytes}
+    del dest
     # --- config 3: ragged non-shared decode, B 256, ctx log-uniform[128, 8192] ------------------------------
     vc = torch.empty_like(kc)
     vc.normal_()

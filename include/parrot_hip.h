@@ -60,6 +60,36 @@ int ph_move_tokens(const void* src, void* dst,
                    int64_t dst_stride_n, int64_t dst_stride_h, int64_t dst_stride_d,
                    void* stream);
 
+/* Gather of token rows out of the block-structured (vLLM) cache layouts into
+ * token-granular rows dest[n, H, D]; slot = src_slots[i], b = slot / block_size,
+ * o = slot % block_size:
+ *   K [num_blocks, H, D/x, block_size, x]:
+ *       dest[dest_idx[i], h, c*x + e] = k_cache[b, h, c, o, e]
+ *   V [num_blocks, H, D, block_size]:
+ *       dest[dest_idx[i], h, d]       = v_cache[b, h, d, o]
+ * Replace move_tokens_from_blocked_k_cache / move_tokens_from_blocked_v_cache
+ * and their Triton kernels (parrot/engine/builtin/kernels/tokens_moving.py:
+ * 104-218 and 222-313).  All strides are in elements and free; the fast path
+ * needs unit-stride x (K), contiguous destination head rows and 16-byte
+ * aligned destination rows, anything else takes an element-wise path.
+ * dest_idx entries must be unique; slots must lie inside the cache (not
+ * checked, as in the reference).  Bit-exact copy; elem_bytes in {1,2,4,8}. */
+int ph_gather_blocked_k(const void* k_cache, void* dest,
+                        const void* src_slots, const void* dest_idx, int index_type,
+                        int64_t n, int64_t num_heads, int64_t head_dim,
+                        int64_t block_size, int64_t x, int elem_bytes,
+                        int64_t stride_n, int64_t stride_h, int64_t stride_c,
+                        int64_t stride_b, int64_t stride_x,
+                        int64_t dst_stride_n, int64_t dst_stride_h, int64_t dst_stride_d,
+                        void* stream);
+int ph_gather_blocked_v(const void* v_cache, void* dest,
+                        const void* src_slots, const void* dest_idx, int index_type,
+                        int64_t n, int64_t num_heads, int64_t head_dim,
+                        int64_t block_size, int elem_bytes,
+                        int64_t stride_n, int64_t stride_h, int64_t stride_d, int64_t stride_b,
+                        int64_t dst_stride_n, int64_t dst_stride_h, int64_t dst_stride_d,
+                        void* stream);
+
 /* KV append: k_cache[slot[t]] = k[t], v_cache[slot[t]] = v[t] in ONE launch.
  * Replaces vllm_reshape_and_cache -> cache_ops.reshape_and_cache
  * (parrot/engine/builtin/kernels/vllm/reshape_and_cache.py:9-22,

@@ -22,6 +22,11 @@ Pinning status (what independent check fails if this file has a plausible bug):
                                    test_attention.py:127-130), q_len==1 reduces
                                    to decode, parent==0 reduces to causal.
   * ref_move_tokens/ref_kv_append -- pinned: python-loop copy, untouched rows.
+  * ref_move_from_blocked_k / ref_move_from_blocked_v -- pinned: element-wise
+                                   python loops over the flat cache buffer with the
+                                   layout's offset formula; the permuted view that
+                                   turns a blocked cache into token-granular rows;
+                                   block_size 1 reduces to ref_move_tokens.
   * ref_rope_neox / ref_rotary_embedding -- pinned: HF rotate_half form
                                    (3rdparty/vllm/tests/kernels/test_pos_encoding.py:10-24),
                                    norm preservation, position 0 identity,
@@ -218,6 +223,42 @@ def ref_move_tokens(
     assert dest_storage.shape[1:] == src_storage.shape[1:]
     rows = src_storage.index_select(0, src_indices.long())
     dest_storage.index_copy_(0, dest_indices.long(), rows)
+
+
+def ref_move_from_blocked_k(
+    blocked_k_cache: torch.Tensor,  # [num_blocks, H, D/x, block_size, x]
+    dest_storage: torch.Tensor,  # [rows, H, D]
+    src_slot_indices: torch.Tensor,  # [n]
+    dest_indices: torch.Tensor,  # [n]
+) -> None:
+    """``dest[dest_idx[i], h, c*x + e] = K[slot // bs, h, c, slot % bs, e]`` in place
+    (parrot/engine/builtin/kernels/tokens_moving.py:135-160: ``block_id = src_index // block_size``,
+    ``block_offset = src_index % block_size``, the head row viewed as ``[D/x, x]``, :177-181)."""
+    assert src_slot_indices.shape == dest_indices.shape
+    num_heads, cols, block_size, x = blocked_k_cache.shape[1:]
+    assert dest_storage.shape[1] == num_heads and dest_storage.shape[2] == cols * x
+    slots = src_slot_indices.long()
+    blk = torch.div(slots, block_size, rounding_mode="floor")
+    off = slots - blk * block_size
+    rows = blocked_k_cache[blk, :, :, off, :]  # [n, H, D/x, x]
+    dest_storage.index_copy_(0, dest_indices.long(), rows.reshape(rows.shape[0], num_heads, cols * x))
+
+
+def ref_move_from_blocked_v(
+    blocked_v_cache: torch.Tensor,  # [num_blocks, H, D, block_size]
+    dest_storage: torch.Tensor,  # [rows, H, D]
+    src_slot_indices: torch.Tensor,
+    dest_indices: torch.Tensor,
+) -> None:
+    """``dest[dest_idx[i], h, d] = V[slot // bs, h, d, slot % bs]`` in place
+    (parrot/engine/builtin/kernels/tokens_moving.py:248-270)."""
+    assert src_slot_indices.shape == dest_indices.shape
+    block_size = blocked_v_cache.shape[3]
+    assert dest_storage.shape[1:] == blocked_v_cache.shape[1:3]
+    slots = src_slot_indices.long()
+    blk = torch.div(slots, block_size, rounding_mode="floor")
+    off = slots - blk * block_size
+    dest_storage.index_copy_(0, dest_indices.long(), blocked_v_cache[blk, :, :, off])
 
 
 def ref_kv_append(

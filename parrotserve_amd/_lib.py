@@ -26,6 +26,8 @@ SIGNATURES: Dict[str, Tuple[object, List[object]]] = {
     "ph_abi_version": (I, []),
     "ph_move_tokens": (I, [P, P, P, P, I, L, L, L, I, L, L, L, L, L, L, P]),
     "ph_kv_append": (I, [P, P, P, P, P, I, L, L, L, I, L, L, L, P]),
+    "ph_gather_blocked_k": (I, [P, P, P, P, I, L, L, L, L, L, I, L, L, L, L, L, L, L, L, P]),
+    "ph_gather_blocked_v": (I, [P, P, P, P, I, L, L, L, L, I, L, L, L, L, L, L, L, P]),
     "ph_rms_norm": (I, [P, P, P, F, L, L, L, L, I, I, P]),
     "ph_rope_neox": (I, [P, P, P, P, L, L, L, L, L, L, L, I, P]),
     "ph_rotary_embedding": (I, [P, P, P, L, L, L, L, L, L, I, P]),

@@ -128,25 +128,56 @@ def discontinuous_move_tokens(src_storage, dest_storage, src_indices, dest_indic
     check(rc, "discontinuous_move_tokens")
 
 
-def _move_from_cache(cache, dest_storage, src_slot_indices, dest_indices, name):
-    if cache.dim() != 3:
-        raise ValueError(
-            f"{name}: only the token-granular cache layout [slots, H, D] is supported "
-            f"(got a {cache.dim()}-d cache; the blocked vLLM layouts are not used by this build)")
-    discontinuous_move_tokens(cache, dest_storage, src_slot_indices, dest_indices)
+def _gather_checks(cache, dest_storage, src_slot_indices, dest_indices):
+    assert src_slot_indices.shape == dest_indices.shape, "src_indices and dest_indices must have the same shape"
+    assert dest_storage.shape[0] >= dest_indices.shape[0], "dest_storage is too small"
+    assert cache.dtype == dest_storage.dtype, "storage dtype mismatch"
+    assert src_slot_indices.dtype == dest_indices.dtype, "index dtype mismatch"
+    _require_gpu(cache, dest_storage, src_slot_indices, dest_indices)
 
 
 def move_tokens_from_blocked_k_cache(blocked_k_cache, dest_storage, src_slot_indices, dest_indices):
-    """Gather token rows of the K cache by slot id into ``dest_storage``
-    (parrot/engine/builtin/kernels/tokens_moving.py:104-218).  With
-    ``block_size == 1`` the blocked K layout degenerates to ``[slots, H, D]``,
-    the only layout accepted here."""
-    _move_from_cache(blocked_k_cache, dest_storage, src_slot_indices, dest_indices, "move_tokens_from_blocked_k_cache")
+    """Gather token rows of a blocked K cache ``[num_blocks, H, D/x, block_size, x]`` by slot id
+    (``slot = block * block_size + offset``) into ``dest_storage [n, H, D]``
+    (parrot/engine/builtin/kernels/tokens_moving.py:104-218).  A 3-d cache is the token-granular layout
+    ``[slots, H, D]`` (the blocked layout at ``block_size == 1``) and takes the plain token move."""
+    if blocked_k_cache.dim() == 3:
+        return discontinuous_move_tokens(blocked_k_cache, dest_storage, src_slot_indices, dest_indices)
+    if blocked_k_cache.dim() != 5:
+        raise ValueError(f"move_tokens_from_blocked_k_cache: expected a 5-d or 3-d cache, got {blocked_k_cache.dim()}-d")
+    _gather_checks(blocked_k_cache, dest_storage, src_slot_indices, dest_indices)
+    num_heads, cols, block_size, x = blocked_k_cache.shape[1:]
+    assert dest_storage.dim() == 3 and dest_storage.shape[1] == num_heads and dest_storage.shape[2] == cols * x, \
+        "storage shape mismatch"
+    src_slot_indices = src_slot_indices.contiguous()
+    dest_indices = dest_indices.contiguous()
+    c = blocked_k_cache
+    rc = _lib.load().ph_gather_blocked_k(
+        _ptr(c), _ptr(dest_storage), _ptr(src_slot_indices), _ptr(dest_indices), _index_code(src_slot_indices),
+        src_slot_indices.shape[0], num_heads, cols * x, block_size, x, c.element_size(),
+        c.stride(0), c.stride(1), c.stride(2), c.stride(3), c.stride(4),
+        dest_storage.stride(0), dest_storage.stride(1), dest_storage.stride(2), _stream())
+    check(rc, "move_tokens_from_blocked_k_cache")
 
 
 def move_tokens_from_blocked_v_cache(blocked_v_cache, dest_storage, src_slot_indices, dest_indices):
-    """V twin of the above (tokens_moving.py:222-313)."""
-    _move_from_cache(blocked_v_cache, dest_storage, src_slot_indices, dest_indices, "move_tokens_from_blocked_v_cache")
+    """V twin of the above for ``[num_blocks, H, D, block_size]`` (tokens_moving.py:222-313)."""
+    if blocked_v_cache.dim() == 3:
+        return discontinuous_move_tokens(blocked_v_cache, dest_storage, src_slot_indices, dest_indices)
+    if blocked_v_cache.dim() != 4:
+        raise ValueError(f"move_tokens_from_blocked_v_cache: expected a 4-d or 3-d cache, got {blocked_v_cache.dim()}-d")
+    _gather_checks(blocked_v_cache, dest_storage, src_slot_indices, dest_indices)
+    num_heads, head_dim, block_size = blocked_v_cache.shape[1:]
+    assert tuple(dest_storage.shape[1:]) == (num_heads, head_dim), "storage shape mismatch"
+    src_slot_indices = src_slot_indices.contiguous()
+    dest_indices = dest_indices.contiguous()
+    c = blocked_v_cache
+    rc = _lib.load().ph_gather_blocked_v(
+        _ptr(c), _ptr(dest_storage), _ptr(src_slot_indices), _ptr(dest_indices), _index_code(src_slot_indices),
+        src_slot_indices.shape[0], num_heads, head_dim, block_size, c.element_size(),
+        c.stride(0), c.stride(1), c.stride(2), c.stride(3),
+        dest_storage.stride(0), dest_storage.stride(1), dest_storage.stride(2), _stream())
+    check(rc, "move_tokens_from_blocked_v_cache")
 
 
 def kv_append(key, value, key_cache, value_cache, slot_mapping):

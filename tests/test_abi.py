@@ -76,6 +76,17 @@ def test_argument_validation_needs_no_gpu():
                               0, None) == _lib.PH_ERR_ARG  # unknown index type
     assert lib.ph_rope_append(None, None, None, None, None, None, None, None, 0, 0, 2, 2, 128, 128, 256, 256, 256, 256,
                               0, None) == _lib.PH_OK       # no tokens
+    # gathers out of the block-structured layouts
+    gk = lambda n, D, x, eb, idx=0: lib.ph_gather_blocked_k(None, None, None, None, idx, n, 2, D, 16, x, eb, 4096, 2048,
+                                                            128, 8, 1, 256, 128, 1, None)
+    assert gk(4, 128, 8, 2) == _lib.PH_ERR_ARG       # null pointers
+    assert gk(0, 128, 8, 2) == _lib.PH_OK            # nothing to move
+    assert gk(4, 128, 7, 2) == _lib.PH_ERR_ARG       # x does not divide the head size
+    assert gk(4, 128, 8, 3) == _lib.PH_ERR_DTYPE
+    assert gk(4, 128, 8, 2, idx=5) == _lib.PH_ERR_ARG
+    gv = lambda n, bs: lib.ph_gather_blocked_v(None, None, None, None, 0, n, 2, 128, bs, 2, 4096, 2048, 16, 1, 256, 128,
+                                               1, None)
+    assert gv(4, 16) == _lib.PH_ERR_ARG and gv(0, 16) == _lib.PH_OK and gv(4, 0) == _lib.PH_ERR_ARG
     assert lib.ph_suffix_tables_append(None, 64, None, None, None, -1, None) == _lib.PH_ERR_ARG
     assert lib.ph_suffix_tables_append(None, 64, None, None, None, 0, None) == _lib.PH_OK
     assert lib.ph_suffix_tables_append(None, 64, None, None, None, 3, None) == _lib.PH_ERR_ARG

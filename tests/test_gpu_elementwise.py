@@ -2,8 +2,8 @@
 import pytest
 import torch
 
-from oracle.ref_ops import (ref_cos_sin_cache, ref_kv_append, ref_move_tokens, ref_rms_norm, ref_rope_neox,
-                            ref_rotary_embedding)
+from oracle.ref_ops import (ref_cos_sin_cache, ref_kv_append, ref_move_from_blocked_k, ref_move_from_blocked_v,
+                            ref_move_tokens, ref_rms_norm, ref_rope_neox, ref_rotary_embedding)
 
 pytestmark = pytest.mark.gpu
 
@@ -51,6 +51,93 @@ def test_move_tokens_strided_storages(dev):
     assert torch.equal(_bits(d.cpu()), _bits(want))
 
 
+def _blocked_inputs(seed, nblk, H, D, bs, x, n, rows, dtype, idx_dtype, runs):
+    g = torch.Generator().manual_seed(seed)
+    kc = torch.randn(nblk, H, D // x, bs, x, generator=g).to(dtype)
+    vc = torch.randn(nblk, H, D, bs, generator=g).to(dtype)
+    if runs:  # whole blocks in order (a context that owns its blocks), then a random tail
+        blocks = torch.randperm(nblk, generator=g)[: n // bs]
+        slots = (blocks[:, None] * bs + torch.arange(bs)[None, :]).reshape(-1)
+        slots = torch.cat([slots, torch.randint(0, nblk * bs, (n - slots.numel(),), generator=g)])
+    else:
+        slots = torch.randint(0, nblk * bs, (n,), generator=g)
+    di = torch.randperm(rows, generator=g)[:n]
+    dst0 = torch.randn(rows, H, D, generator=g).to(dtype)
+    return kc, vc, slots.to(idx_dtype), di.to(idx_dtype), dst0
+
+
+@pytest.mark.parametrize("runs", [True, False])
+@pytest.mark.parametrize("H,D,bs,x,dtype,idx_dtype", [
+    (32, 128, 16, 8, torch.float16, torch.int64),   # the vLLM layout at 16-bit elements
+    (40, 128, 16, 8, torch.bfloat16, torch.int32),
+    (96, 128, 16, 8, torch.float16, torch.int64),   # tokens_moving.py:365-420 (H 96, block 16, x 8)
+    (5, 64, 8, 4, torch.float32, torch.int64),      # 16-byte units of 4-byte elements, head count not a multiple of 4
+    (3, 256, 32, 8, torch.float16, torch.int32),    # 512-byte head rows
+    (2, 512, 4, 8, torch.float16, torch.int64),     # 1 KB head rows: one head per LDS round
+    (3, 24, 4, 2, torch.float16, torch.int64),      # 3-unit... head rows of 48 bytes, not a power of two: element path
+    (2, 20, 3, 5, torch.float16, torch.int32),      # odd everything: element path
+])
+def test_move_from_blocked_caches_bit_exact(dev, H, D, bs, x, dtype, idx_dtype, runs):
+    from parrotserve_amd import kernels
+
+    nblk, n, rows = 24, 203, 300
+    kc, vc, slots, di, dst0 = _blocked_inputs(21, nblk, H, D, bs, x, n, rows, dtype, idx_dtype, runs)
+    want_k, want_v = dst0.clone(), dst0.clone()
+    ref_move_from_blocked_k(kc, want_k, slots, di)
+    ref_move_from_blocked_v(vc, want_v, slots, di)
+    dk, dv = dst0.to(dev), dst0.to(dev)
+    kernels.move_tokens_from_blocked_k_cache(kc.to(dev), dk, slots.to(dev), di.to(dev))
+    kernels.move_tokens_from_blocked_v_cache(vc.to(dev), dv, slots.to(dev), di.to(dev))
+    assert torch.equal(_bits(dk.cpu()), _bits(want_k))
+    assert torch.equal(_bits(dv.cpu()), _bits(want_v))
+
+
+def test_move_from_blocked_strided_views_and_empty(dev):
+    """Free strides (tokens_moving.py:182-200 passes every stride): a head slice of a larger cache, a strided
+    destination; and an empty index list is a no-op."""
+    from parrotserve_amd import kernels
+
+    g = torch.Generator().manual_seed(22)
+    big_k = torch.randn(10, 6, 4, 8, 8, generator=g).half()
+    big_v = torch.randn(10, 6, 32, 8, generator=g).half()
+    kc, vc = big_k[:, 1:5], big_v[:, 1:5]               # heads 1..4 of 6
+    big_dst = torch.randn(50, 4, 64, generator=g).half()
+    dview = lambda t: t[:, :, 16:48]                    # [50, 4, 32], head stride 64
+    slots = torch.randint(0, 80, (33,), generator=g)
+    di = torch.randperm(50, generator=g)[:33]
+    want_k, want_v = big_dst.clone(), big_dst.clone()
+    ref_move_from_blocked_k(kc, dview(want_k), slots, di)
+    ref_move_from_blocked_v(vc, dview(want_v), slots, di)
+    dk, dv = big_dst.to(dev), big_dst.to(dev)
+    kernels.move_tokens_from_blocked_k_cache(big_k.to(dev)[:, 1:5], dview(dk), slots.to(dev), di.to(dev))
+    kernels.move_tokens_from_blocked_v_cache(big_v.to(dev)[:, 1:5], dview(dv), slots.to(dev), di.to(dev))
+    assert torch.equal(_bits(dk.cpu()), _bits(want_k))
+    assert torch.equal(_bits(dv.cpu()), _bits(want_v))
+    empty = torch.zeros(0, dtype=torch.int64, device=dev)
+    before = dk.clone()
+    kernels.move_tokens_from_blocked_k_cache(big_k.to(dev)[:, 1:5], dview(dk), empty, empty)
+    assert torch.equal(dk, before)
+
+
+def test_move_from_blocked_equals_token_move_at_scale(dev):
+    """65,536 tokens at 32 x 128: the blocked gathers against the plain token move on the permuted caches."""
+    from parrotserve_amd import kernels
+
+    g = torch.Generator().manual_seed(23)
+    nblk, H, D, bs, x, n = 8192, 32, 128, 16, 8, 65536
+    rows = torch.randn(nblk * bs, H, D, generator=g).half().to(dev)   # token-granular truth
+    kc = rows.view(nblk, bs, H, D // x, x).permute(0, 2, 3, 1, 4).contiguous()
+    vc = rows.view(nblk, bs, H, D).permute(0, 2, 3, 1).contiguous()
+    slots = torch.randint(0, nblk * bs, (n,), generator=g).to(dev)
+    di = torch.randperm(n, generator=g).to(dev)
+    want = torch.zeros(n, H, D, dtype=torch.float16, device=dev)
+    kernels.discontinuous_move_tokens(rows, want, slots, di)
+    for cache, fn in ((kc, kernels.move_tokens_from_blocked_k_cache), (vc, kernels.move_tokens_from_blocked_v_cache)):
+        got = torch.zeros_like(want)
+        fn(cache, got, slots, di)
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+
+
 def test_move_tokens_reference_selftest_shape(dev):
     """tokens_moving.py:316-362: H 96 x D 128 fp16, random src rows to every second dest row (scaled-down count)."""
     from parrotserve_amd import kernels
@@ -79,8 +166,10 @@ def test_move_empty_and_blocked_names(dev):
     assert torch.equal(dst.cpu(), src.cpu().flip(0))
     kernels.move_tokens_from_blocked_v_cache(src, dst, idx, idx)
     assert torch.equal(dst.cpu(), src.cpu())
-    with pytest.raises(ValueError):
-        kernels.move_tokens_from_blocked_k_cache(torch.zeros(2, 2, 2, 4, 8, device=dev).half(), dst, idx, idx)
+    with pytest.raises(ValueError):  # neither the 5-d blocked K layout nor token-granular rows
+        kernels.move_tokens_from_blocked_k_cache(torch.zeros(2, 2, 16, 4, device=dev).half(), dst, idx, idx)
+    with pytest.raises(AssertionError):  # head shape of the cache and of the destination differ
+        kernels.move_tokens_from_blocked_k_cache(torch.zeros(2, 2, 4, 4, 8, device=dev).half(), dst, idx, idx)
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])

@@ -4,8 +4,8 @@ import math
 import pytest
 import torch
 
-from oracle.ref_ops import (ref_cos_sin_cache, ref_kv_append, ref_move_tokens, ref_rms_norm, ref_rope_neox,
-                            ref_rotary_embedding)
+from oracle.ref_ops import (ref_cos_sin_cache, ref_kv_append, ref_move_from_blocked_k, ref_move_from_blocked_v,
+                            ref_move_tokens, ref_rms_norm, ref_rope_neox, ref_rotary_embedding)
 
 
 def test_move_tokens_python_loop():
@@ -35,6 +35,63 @@ def test_move_tokens_strided_dest_like_reference_selftest():
     di = torch.arange(0, 128, 2)
     ref_move_tokens(src, dst, si, di)
     assert torch.equal(dst[::2], src[si]) and (dst[1::2] == 0).all()
+
+
+def _blocked_case(seed, nblk=5, H=3, D=8, bs=4, x=2, n=11, rows=30):
+    g = torch.Generator().manual_seed(seed)
+    kc = torch.randn(nblk, H, D // x, bs, x, generator=g).half()
+    vc = torch.randn(nblk, H, D, bs, generator=g).half()
+    slots = torch.randint(0, nblk * bs, (n,), generator=g)
+    di = torch.randperm(rows, generator=g)[:n]
+    dst0 = torch.randn(rows, H, D, generator=g).half()
+    return kc, vc, slots, di, dst0
+
+
+def test_move_from_blocked_flat_offset_loops():
+    """Element-wise loops over the flat buffers with each layout's offset formula (K [nb,H,D/x,bs,x], V [nb,H,D,bs])."""
+    nblk, H, D, bs, x = 5, 3, 8, 4, 2
+    kc, vc, slots, di, dst0 = _blocked_case(3, nblk, H, D, bs, x)
+    kflat, vflat = kc.reshape(-1), vc.reshape(-1)
+    want_k, want_v = dst0.clone(), dst0.clone()
+    for i in range(slots.numel()):
+        b, o = divmod(int(slots[i]), bs)
+        for h in range(H):
+            for d in range(D):
+                want_k[int(di[i]), h, d] = kflat[(((b * H + h) * (D // x) + d // x) * bs + o) * x + d % x]
+                want_v[int(di[i]), h, d] = vflat[((b * H + h) * D + d) * bs + o]
+    got_k, got_v = dst0.clone(), dst0.clone()
+    ref_move_from_blocked_k(kc, got_k, slots, di)
+    ref_move_from_blocked_v(vc, got_v, slots, di)
+    assert torch.equal(got_k.view(torch.int16), want_k.view(torch.int16))
+    assert torch.equal(got_v.view(torch.int16), want_v.view(torch.int16))
+    untouched = [r for r in range(dst0.shape[0]) if r not in set(di.tolist())]
+    assert torch.equal(got_k[untouched], dst0[untouched]) and torch.equal(got_v[untouched], dst0[untouched])
+
+
+def test_move_from_blocked_equals_move_on_the_token_granular_view():
+    """Permuting a blocked cache to [num_blocks * block_size, H, D] makes the gather an ordinary token move."""
+    kc, vc, slots, di, dst0 = _blocked_case(4, nblk=6, H=2, D=16, bs=8, x=4, n=20, rows=40)
+    nblk, H, cols, bs, x = kc.shape
+    k_rows = kc.permute(0, 3, 1, 2, 4).reshape(nblk * bs, H, cols * x)
+    v_rows = vc.permute(0, 3, 1, 2).reshape(nblk * bs, H, cols * x)
+    for blocked, rows, fn in ((kc, k_rows, ref_move_from_blocked_k), (vc, v_rows, ref_move_from_blocked_v)):
+        got, want = dst0.clone(), dst0.clone()
+        fn(blocked, got, slots, di)
+        ref_move_tokens(rows, want, slots, di)
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+
+
+def test_move_from_blocked_block_size_one_is_the_token_move():
+    g = torch.Generator().manual_seed(5)
+    rows = torch.randn(12, 2, 8, generator=g).half()
+    slots = torch.randint(0, 12, (7,), generator=g)
+    di = torch.randperm(9, generator=g)[:7]
+    want = torch.zeros(9, 2, 8).half()
+    ref_move_tokens(rows, want, slots, di)
+    got_k, got_v = torch.zeros(9, 2, 8).half(), torch.zeros(9, 2, 8).half()
+    ref_move_from_blocked_k(rows.view(12, 2, 2, 1, 4), got_k, slots, di)
+    ref_move_from_blocked_v(rows.view(12, 2, 8, 1), got_v, slots, di)
+    assert torch.equal(got_k, want) and torch.equal(got_v, want)
 
 
 def test_kv_append_roundtrip_and_noncontiguous_source():
