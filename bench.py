@@ -396,6 +396,8 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run the move kernel as a plain 1 GiB copy (known traffic, to scale the profiler's "
                          "FETCH_SIZE / WRITE_SIZE counters) and exit")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="only run config 4's prefill kernel a few times (for profiler counter passes) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs the hot path on ONE GPU; --gpus must be 1 "
@@ -409,6 +411,22 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     lib = _lib.load()
+
+    if args.prefill_only:
+        # config 4's prefill with parent context alone, a few launches (for counter collection on that kernel)
+        c4 = synth.config4()
+        T, H4, D4 = c4.q.shape
+        kc4, vc4 = synth.pool_to_device(c4.k_rows, c4.v_rows, c4.used_slots, c4.pool_slots, dev)
+        ctx = [c4.used_slots[torch.cat([p, n])].tolist() for p, n in zip(c4.parent_lists, c4.new_lists)]
+        ptab = kernels.PrefillTables.build(c4.q_lens, ctx, dev)
+        qc = c4.q.to(dev)
+        o4 = torch.empty_like(qc)
+        t_pre = _time_gpu(torch, lambda: kernels.prefill_attention(qc, kc4, vc4, ptab, out=o4), iters=3, warmup=1, inner=4)
+        par = c4.parent_lists[0].numel()
+        flops = 4 * H4 * D4 * sum(n * par + n * (n + 1) // 2 for n in c4.q_lens)
+        print(json.dumps({"c4_prefill_only": {"tokens": T, "ms": t_pre * 1e3, "flops": flops,
+                                              "TFLOP/s": flops / t_pre / 1e12}}))
+        return
 
     if args.copy_calibration:
         rows = 131072  # x 8 KiB = 1 GiB read + 1 GiB written per launch
@@ -463,6 +481,18 @@ def main():
 
     t_step = timed(step, args.steps, args.warmup)
     t_warm = timed(lambda i: kernels.decode_attention(qs[0], kc, vc, tables[0], out=out), args.steps, args.warmup)
+
+    # spread of single steps inside the same rotation (an event between steps; the events themselves cost the
+    # stream about a microsecond per step, so these sit a little above ms_per_step)
+    n_pc = min(args.steps, 400)
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(n_pc + 1)]
+    marks[0].record()
+    for i in range(n_pc):
+        step(i)
+        marks[i + 1].record()
+    torch.cuda.synchronize()
+    per_step = sorted(marks[i].elapsed_time(marks[i + 1]) * 1e3 for i in range(n_pc))
+    pct = {k: per_step[min(n_pc - 1, int(q * n_pc))] for k, q in (("p10", 0.1), ("p50", 0.5), ("p90", 0.9))}
 
     # per-kernel durations inside the same rotation: each kernel's own dispatch begin/end (start/stop events
     # attached to its launch on the launch stream), the quantity a kernel trace reports
@@ -525,6 +555,7 @@ def main():
             "avg_launch_us": t_suffix * 1e6,
         },
         "merge_us": t_merge * 1e6,
+        "step_us_percentiles": pct,
         "warm_single_kv_set": {"value": B / t_warm, "ms_per_step": t_warm * 1e3},
     }
     if not fused:
