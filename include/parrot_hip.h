@@ -193,6 +193,11 @@ int ph_rotary_embedding(void* state, const void* cos, const void* sin,
  *                 then a copy of its first item's request, first token, count,
  *                 0, 0, 0) -- one record read starts a piece;
  *   req_item_cu:  int32 [B+1], request b owns items [cu[b], cu[b+1]).
+ *   num_items may be the capacity of the items array rather than the count
+ *   in use (only items named by lane_rec / req_item_cu are touched, and at
+ *   most num_lanes + B - 1 can be): it sizes the workspace only.  A caller
+ *   that replays a captured graph while contexts grow keeps the pointers,
+ *   num_items and num_lanes fixed and rewrites the arrays in place.
  * workspace: at least ph_decode_workspace_bytes(...) bytes, 256-byte aligned
  *   (num_items = plan->num_items, or 0 without a plan).
  */

@@ -348,7 +348,8 @@ class DecodeTables:
     max_suffix_len: int = 0
     chunk_tokens: int = 0  # 0 = let the library choose
     # balanced suffix plan (needs the lengths on the host): device int32 arrays + the host struct
-    plan_items: Optional[torch.Tensor] = None  # [num_items, 4]
+    plan_buffer: Optional[torch.Tensor] = None  # the three arrays below, back to back
+    plan_items: Optional[torch.Tensor] = None  # [lanes + B, 4], the first rows in use
     plan_lane_item_cu: Optional[torch.Tensor] = None  # lane records [num_lanes, 8]
     plan_req_item_cu: Optional[torch.Tensor] = None  # [B + 1]
     plan: Optional[_lib.SuffixPlan] = None
@@ -362,28 +363,39 @@ class DecodeTables:
         return self.suffix_slots.numel()
 
     def set_plan(self, lens: Sequence[int], num_lanes: int, device) -> None:
-        """Cut the batch's suffix token stream into ``num_lanes`` near-equal pieces (see ph_suffix_plan)."""
+        """Cut the batch's suffix token stream into ``num_lanes`` near-equal pieces (see ph_suffix_plan).
+
+        The device arrays have a fixed layout for a given (lanes, batch) -- the item array is sized for the most
+        items a cut can produce, lanes + batch -- and are rewritten in place when the lengths change, so the
+        plan's pointers and counts (and with them the workspace layout) stay what a captured graph recorded."""
         items, lane_cu, req_cu = plan_suffix_items(lens, num_lanes)
         if items.shape[0] == 0:
             return
         lanes = lane_cu.shape[0] - 1
         n_items = items.shape[0]
+        cap = lanes + req_cu.shape[0] - 1
         # one host buffer, one upload: items | lane records | per-request item offsets
-        o_rec = n_items * 4
+        o_rec = cap * 4
         o_cu = o_rec + lanes * 8
         buf = np.zeros(o_cu + req_cu.shape[0], dtype=np.int32)
-        buf[:o_rec] = items.reshape(-1)
+        buf[: n_items * 4] = items.reshape(-1)
         rec = buf[o_rec:o_cu].reshape(lanes, 8)
         rec[:, 0] = lane_cu[:-1]
         rec[:, 1] = lane_cu[1:] - lane_cu[:-1]
         first = np.minimum(lane_cu[:-1], n_items - 1)
         rec[:, 2:5] = items[first, 0:3]
         buf[o_cu:] = req_cu
+        old = self.plan_buffer
+        if old is not None and old.numel() == buf.shape[0] and old.device == torch.device(device) and \
+                self.plan is not None and self.plan.num_lanes == lanes:
+            old.copy_(torch.from_numpy(buf))  # ordered on the current stream behind the kernels still reading it
+            return
         dev_buf = torch.from_numpy(buf).to(device)
-        self.plan_items = dev_buf[:o_rec].view(n_items, 4)
+        self.plan_buffer = dev_buf
+        self.plan_items = dev_buf[:o_rec].view(cap, 4)
         self.plan_lane_item_cu = dev_buf[o_rec:o_cu].view(lanes, 8)
         self.plan_req_item_cu = dev_buf[o_cu:]
-        self.plan = _lib.SuffixPlan(self.plan_items.data_ptr(), n_items, self.plan_lane_item_cu.data_ptr(),
+        self.plan = _lib.SuffixPlan(self.plan_items.data_ptr(), cap, self.plan_lane_item_cu.data_ptr(),
                                     lanes, self.plan_req_item_cu.data_ptr())
 
     @staticmethod

@@ -376,6 +376,64 @@ def test_decode_attention_replays_from_a_captured_graph(dev):
     torch.testing.assert_close(out_static.cpu().float(), ref.float(), **TOL[torch.float16])
 
 
+def test_captured_decode_step_replays_while_contexts_grow(dev):
+    """One decode step recorded once, replayed over six iterations in which every request gains a token: the slot
+    tables are patched and the suffix plan rewritten in place between replays (fixed pointers, counts and workspace
+    layout), and each replay must equal the eager result on tables built from scratch for that iteration."""
+    from parrotserve_amd import kernels, synth, table_cache
+
+    g = torch.Generator().manual_seed(29)
+    B, H, D, P = 40, 8, 128, 700
+    lens = torch.randint(1, 100, (B,), generator=g).tolist()
+    case = synth.make_decode_case("grow", 29, torch.float16, 1, B, P, lens, H, D, 1 << 14)
+    kc, vc = synth.pool_to_device(case.k_rows, case.v_rows, case.used_slots, case.pool_slots, dev)
+    prefix = case.pool_lists(case.prefix_lists)
+    suffix = [list(l) for l in case.pool_lists(case.suffix_lists)]
+    used = set(case.used_slots.tolist())
+    spare = [s for s in range(case.pool_slots) if s not in used][: 6 * B]
+    tables = kernels.DecodeTables.build(prefix, case.group_req_cu, suffix, dev, num_heads=H, head_dim=D)
+    table_cache._widen(tables, max(lens) + 8, dev)          # room for the tokens to come
+    lanes = tables.plan.num_lanes
+    q_static = case.q.to(dev)
+    out_static = torch.empty_like(q_static)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        kernels.decode_attention(q_static, kc, vc, tables, out=out_static)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        kernels.decode_attention(q_static, kc, vc, tables, out=out_static)
+    plan_ptrs = (tables.plan.items, tables.plan.num_items, tables.plan.lane_rec, tables.plan.num_lanes)
+    gq = torch.Generator(device=dev).manual_seed(6)
+    for it in range(6):
+        new = spare[it * B:(it + 1) * B]
+        new_dev = torch.tensor(new, dtype=torch.int32, device=dev)
+        kc[new_dev.long()] = torch.randn((B, H, D), generator=gq, device=dev, dtype=torch.float16)
+        vc[new_dev.long()] = torch.randn((B, H, D), generator=gq, device=dev, dtype=torch.float16)
+        for b in range(B):
+            suffix[b].append(new[b])
+        kernels.suffix_tables_append(tables.suffix_slots, tables.suffix_lens, None, new_dev)
+        tables.max_suffix_len += 1
+        tables.set_plan([len(l) for l in suffix], lanes, dev)
+        assert (tables.plan.items, tables.plan.num_items, tables.plan.lane_rec, tables.plan.num_lanes) == plan_ptrs
+        q_new = torch.randn(q_static.shape, generator=gq, device=dev, dtype=torch.float16)
+        fresh = kernels.DecodeTables.build(prefix, case.group_req_cu, suffix, dev, num_heads=H, head_dim=D)
+        fresh.set_plan([len(l) for l in suffix], lanes, dev)  # the same cuts, so the same summation order
+        eager = kernels.decode_attention(q_new, kc, vc, fresh)
+        torch.cuda.synchronize()
+        q_static.copy_(q_new)
+        out_static.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        torch.testing.assert_close(out_static.float(), eager.float(), **TOL[torch.float16])
+        assert torch.equal(out_static, eager), f"iteration {it}: the replay differs from the eager result"
+    full = [prefix[0] + l for l in suffix]
+    ref = ref_decode_attention(q_static.cpu(), kc.cpu(), vc.cpu(), [torch.tensor(l) for l in full])
+    torch.testing.assert_close(out_static.cpu().float(), ref.float(), **TOL[torch.float16])
+
+
 @pytest.mark.parametrize("seed", range(12))
 def test_randomized_grouped_decode_shapes(dev, seed):
     """Seeded random batches: 1-3 prefix groups of 1-140 requests, prefixes of 1-1500 tokens (not multiples of
