@@ -36,8 +36,6 @@ struct GatherArgs {
                    // everything is 16-byte aligned, so 16 / unit-size consecutive slots can share one load
 };
 
-namespace {
-
 constexpr int kG = 16;    // list entries per workgroup
 constexpr int kPad = 16;  // bytes appended to every LDS row (spreads the transposed accesses over the banks)
 
@@ -181,6 +179,8 @@ __global__ __launch_bounds__(256) void gather_generic_kernel(GatherArgs a) {
     }
   }
 }
+
+namespace {
 
 bool is_pow2(int64_t v) { return v > 0 && (v & (v - 1)) == 0; }
 
