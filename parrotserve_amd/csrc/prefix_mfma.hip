@@ -65,6 +65,11 @@ __device__ __forceinline__ void lds_dma16(const void* gptr, uint32_t lds_addr) {
   else
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(lds_addr) : "memory");
 }
+// 4 bytes per lane the same way: used only to pull cache lines towards L2 ahead of the row loads (the data
+// lands in an LDS area nobody reads, so no register waits for it)
+__device__ __forceinline__ void lds_dma4(const void* gptr, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(gptr), "s"(lds_addr) : "memory");
+}
 // LDS byte address of a generic pointer into shared memory, as a wave-uniform scalar
 __device__ __forceinline__ uint32_t lds_addr_of(const char* p) {
   return __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)p);
@@ -457,7 +462,8 @@ __global__ __launch_bounds__(256, 1) void prefix_mfma_kernel(PrefixArgs a, int m
 constexpr int kWin = 4096;                        // tokens per slot window
 constexpr int kWinOff = 8 * kStage;               // LDS offset of the window (behind the 128 KB of stages)
 constexpr int kMlOff = kWinOff + kWin * 4;        // (m, l, true max) of eight waves for the fold
-constexpr int kTile8Lds = kMlOff + 8 * 3 * 256;
+constexpr int kPfOff = kMlOff + 8 * 3 * 256;    // landing area of the cache-line touches (256 bytes per wave)
+constexpr int kTile8Lds = kPfOff + 8 * 256;
 
 // max over the two 32-lane halves of the wave: lane l gets max(x[l], x[l ^ 32]).  One lane-swap instruction
 // (lanes 32..63 of the first register trade places with lanes 0..31 of the second) instead of a trip
@@ -509,6 +515,13 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
   // decode reads every prefix row once per launch (streaming policy); prefill tiles are re-read by the
   // other query tiles of the chunk and should stay in L2
   constexpr bool NTLOAD = !CAUSAL;
+  // Decode: the LDS ring holds one step beyond the one being multiplied, which is too little to cover the
+  // memory latency (the ring cannot grow: it is all of LDS).  So every thread also touches one 128-byte line
+  // of the step after that (128 tokens x K and V x 2 lines = 512 lines) with a 4-byte load: the step's rows
+  // are then on their way to L2 a whole step before the ring has room for them, and the row loads that
+  // follow find them there.  Issued behind the step's row loads, so their completion is still counted
+  // exactly (one younger load per step).
+  constexpr bool PREFETCH = !CAUSAL && A == 1 && STEP * TQ == 128;
   constexpr float kSlack = 8.f;
   float16_t oacc[4];
   float m = -INFINITY, lsum = 0.f, mtrue = -INFINITY;
@@ -543,6 +556,7 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
     gbase[i] = isv ? reinterpret_cast<const char*>(vc + (int64_t)head * kPD + ((c ^ (4 * tl)) * 8))
                    : reinterpret_cast<const char*>(kc + (int64_t)head * kPD + ((c ^ ((4 * (r0 + i) + tl) & 15)) * 8));
   const uint32_t dst0 = lds_addr_of(gl) + sub0 * kStage + (isv ? kVtOff : 0) + r0 * 1024;
+  const uint32_t pf_lds = lds_addr_of(smem + kPfOff) + w8 * 256;
   // rows of the group's tile that starts at token tb, into ring stage `stage`
   auto fetch_rows = [&](int tb, int stage) {
     uint32_t sl[LPT];
@@ -614,7 +628,7 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
     // Tile `it` of this group has landed once at most the (A - 1) LPT loads issued after it are outstanding
     // (near the end fewer were issued, so everything is awaited); the barrier publishes all parts of the
     // tile and tells everyone that the stage read in the previous step is free again.
-    if (it + A - 1 < my_iters) wait_vmcnt<(A - 1) * LPT>(); else wait_vmcnt<0>();
+    if (it + A - 1 < my_iters) wait_vmcnt<(A - 1) * LPT + (PREFETCH ? 1 : 0)>(); else wait_vmcnt<0>();
     __syncthreads();
     {
       const int front = s0 + STEP * TQ * (it + A);           // first token of the step being staged
@@ -624,6 +638,14 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
         __syncthreads();
       }
       if (it > 0 && it + A < my_iters) fetch_rows(front + STEP * g, (stage + A) % NST);
+      if constexpr (PREFETCH) {
+        // token (of all four groups) and line of the step after `front`, clamped into the list and the window
+        const int pt = min(min(front + STEP * TQ + (int)(threadIdx.x >> 2), s1 - 1), win0 + kWin - 1);
+        const uint32_t slot = (uint32_t)win[pt - win0];
+        const char* base = reinterpret_cast<const char*>((threadIdx.x & 2) ? vc : kc) + (int64_t)head * (kPD * 2) +
+                           (threadIdx.x & 1) * 128;
+        lds_dma4(base + (uint64_t)slot * row_bytes, pf_lds);
+      }
     }
     if (it >= my_iters || tb > wave_last) continue;           // wave-uniform
     float16_t sacc[SUB];
