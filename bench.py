@@ -561,11 +561,30 @@ def main():
         "step_us_percentiles": pct,
         "warm_single_kv_set": {"value": B / t_warm, "ms_per_step": t_warm * 1e3},
     }
-    if not fused:
+    if fused:
+        # the prefix phase on its own (the same batch with empty suffixes: prefix kernel, then merge), for its
+        # matrix-core figures; in the step proper it runs inside the fused launch
+        ptabs = [kernels.DecodeTables.build([perm[l * n_used:(l + 1) * n_used][p].tolist() for p in case.prefix_lists],
+                                            case.group_req_cu, [[] for _ in range(B)], dev) for l in range(NL)]
+        for i in range(8):
+            kernels.decode_attention(qs[i % NL], kc, vc, ptabs[i % NL], out=out)
+        sets = [ev.create(6) for _ in range(64)]
+        for i, s6 in enumerate(sets):
+            lib.ph_arm_kernel_events(s6)
+            kernels.decode_attention(qs[i % NL], kc, vc, ptabs[i % NL], out=out)
+        torch.cuda.synchronize()
+        lib.ph_arm_kernel_events(None)
+        tp = [ev.elapsed_ms(s6[0], s6[1]) for s6 in sets]
+        for s6 in sets:
+            ev.destroy(s6)
+        if all(v is not None for v in tp):
+            t_prefix = sum(tp) / len(tp) * 1e-3
+        del ptabs
+    if t_prefix is not None:
         prefix_tflops = prefix_flops / t_prefix / 1e12
         prefix_bound_tflops = min(MFMA_F16_PEAK_TFLOPS, B * HBM_PEAK_GBS / 1e3)  # AI = B FLOP per KV byte
         result["prefix_phase"] = {
-            "kernel": "prefix_mfma8_kernel",
+            "kernel": "prefix_mfma8_kernel" + (" (run on its own: empty suffixes)" if fused else ""),
             "avg_launch_us": t_prefix * 1e6,
             "tflops": prefix_tflops,
             "frac_mfma_peak": prefix_tflops / MFMA_F16_PEAK_TFLOPS,
