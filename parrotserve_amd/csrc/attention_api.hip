@@ -48,7 +48,10 @@ static DecodePlan plan_decode(int64_t B, int64_t H, int64_t groups, int64_t max_
     // One workgroup per CU at a time (the kernel uses most of the register file), so pick the
     // split count whose workgroup total wastes the least of a whole number of 256-wide rounds.
     // Cost model: rounds x (tokens per split + a fixed prologue/epilogue worth ~96 tokens).
-    const int64_t mtiles = cdiv(cdiv(B, groups), kPrefixQueryTile);
+    // the kernel takes 64-, 128- or 256-query tiles by the largest group; the mean group size stands in here
+    const int64_t per_group = cdiv(B, groups);
+    const int64_t qtile = per_group <= 64 ? kPrefixQueryTile : per_group <= 128 ? 2 * kPrefixQueryTile : 4 * kPrefixQueryTile;
+    const int64_t mtiles = cdiv(per_group, qtile);
     const int64_t base = groups * H * (mtiles > 0 ? mtiles : 1);
     const int64_t max_splits = cdiv(max_prefix, 4 * kPrefixTile);
     int64_t splits = 1, best = -1;

@@ -829,9 +829,10 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
 
 // Shared-prefix phase, eight waves: one unit of work = (split, head, group x 64-query tile z), run by the
 // whole workgroup; writes one (O, m, l) part per request of the tile.
-template <typename E, typename Mid = NoMid>
+template <typename E, int TQ, typename Mid = NoMid>
 __device__ __forceinline__ void prefix_unit8(const PrefixArgs& a, int split, int head, int z, int mtiles, char* smem,
                                              Mid mid = Mid()) {
+  constexpr int QB = 8 / TQ, QT = 32 * QB, NDB = 4 / TQ;  // query blocks, queries per tile, dim blocks per wave
   const int g = z / mtiles, mt = z - g * mtiles;
   int r0 = 0, r1 = a.B, poff = 0, plen = a.fixed_prefix_len;
   if (a.prefix_cu) {
@@ -840,8 +841,8 @@ __device__ __forceinline__ void prefix_unit8(const PrefixArgs& a, int split, int
     poff = a.prefix_cu[g];
     plen = a.prefix_cu[g + 1] - poff;
   }
-  const int qbase = r0 + mt * 64;
-  const int nq = min(64, r1 - qbase);
+  const int qbase = r0 + mt * QT;
+  const int nq = min(QT, r1 - qbase);
   if (nq <= 0) {
     mid();
     return;
@@ -866,19 +867,22 @@ __device__ __forceinline__ void prefix_unit8(const PrefixArgs& a, int split, int
   wk.s0 = s0;
   wk.s1 = s1;
   wk.causal_off = 0;
-  float16_t of[1];
+  float16_t of[NDB];
   float m, l;
-  attn_tile8<E, false, 4>(wk, a.kc, a.vc, a.row_stride, head, a.scale_log2e, smem, of, m, l, mid);
-  const int lane = threadIdx.x & 63, w8 = threadIdx.x >> 6, tq = w8 >> 1, qh = w8 & 1, h = lane >> 5, ql = lane & 31;
+  attn_tile8<E, false, TQ>(wk, a.kc, a.vc, a.row_stride, head, a.scale_log2e, smem, of, m, l, mid);
+  const int lane = threadIdx.x & 63, w8 = threadIdx.x >> 6, tq = w8 / QB, qh = w8 % QB, h = lane >> 5, ql = lane & 31;
   const int q = 32 * qh + ql;
   if (q < nq) {
     const float inv = 1.f / l;
     const int64_t pr = ((int64_t)split * a.B + qbase + q) * a.H + head;
-    float* op = a.opart + pr * kPD + 32 * tq + 4 * h;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      float4_t v = {of[0][4 * j] * inv, of[0][4 * j + 1] * inv, of[0][4 * j + 2] * inv, of[0][4 * j + 3] * inv};
-      *reinterpret_cast<float4_t*>(op + 8 * j) = v;
+    for (int nd = 0; nd < NDB; ++nd) {
+      float* op = a.opart + pr * kPD + 32 * (NDB * tq + nd) + 4 * h;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float4_t v = {of[nd][4 * j] * inv, of[nd][4 * j + 1] * inv, of[nd][4 * j + 2] * inv, of[nd][4 * j + 3] * inv};
+        *reinterpret_cast<float4_t*>(op + 8 * j) = v;
+      }
     }
     if (h == 0 && tq == 0) {
       a.ml[pr * 2] = m;
@@ -887,10 +891,10 @@ __device__ __forceinline__ void prefix_unit8(const PrefixArgs& a, int split, int
   }
 }
 
-template <typename E>
+template <typename E, int TQ>
 __global__ __launch_bounds__(512) void prefix_mfma8_kernel(PrefixArgs a, int mtiles) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  prefix_unit8<E>(a, blockIdx.x, blockIdx.y, blockIdx.z, mtiles, smem);
+  prefix_unit8<E, TQ>(a, blockIdx.x, blockIdx.y, blockIdx.z, mtiles, smem);
 }
 
 // Prefix and suffix phases of one decode step in one launch.  Workgroup b owns the prefix units b,
@@ -901,7 +905,7 @@ __global__ __launch_bounds__(512) void prefix_mfma8_kernel(PrefixArgs a, int mti
 // more), then the prefix main loop on tiles that landed long ago, then the fold.  Against two launches this
 // removes one launch, hides the prefix prologue behind the suffix stream and keeps the memory system busy
 // from the first microseconds.  The merge stays a separate launch: it needs every part.
-template <typename E>
+template <typename E, int TQ>
 __global__ __launch_bounds__(512) void decode_fused_kernel(PrefixArgs pa, int mtiles, int n_units, ItemArgs ia) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   constexpr int HPW = kWave / (kPD / 8);
@@ -927,12 +931,12 @@ __global__ __launch_bounds__(512) void decode_fused_kernel(PrefixArgs pa, int mt
     const int u = blockIdx.x;
     const int split = u % pa.n_splits;
     const int rest = u / pa.n_splits;
-    prefix_unit8<E>(pa, split, rest % pa.H, rest / pa.H, mtiles, smem, suffix);
+    prefix_unit8<E, TQ>(pa, split, rest % pa.H, rest / pa.H, mtiles, smem, suffix);
     for (int v = u + gridDim.x; v < n_units; v += gridDim.x) {
       __syncthreads();  // the fold scratch of the last unit is the staging ring of the next
       const int sp = v % pa.n_splits;
       const int rs = v / pa.n_splits;
-      prefix_unit8<E>(pa, sp, rs % pa.H, rs / pa.H, mtiles, smem);
+      prefix_unit8<E, TQ>(pa, sp, rs % pa.H, rs / pa.H, mtiles, smem);
     }
   } else {
     suffix();
@@ -998,6 +1002,17 @@ __global__ void prefill_tiles_kernel(const int32_t* q_cu, int num_chunks, int32_
   tile_cu[num_chunks] = acc;
 }
 
+template <typename E, int TQ>
+static void launch_prefix8(const PrefixArgs& a, int num_groups, int max_group_reqs, hipStream_t st,
+                           const KernelEvents& ev) {
+  constexpr int QT = 32 * (8 / TQ);
+  const int mtiles = (max_group_reqs + QT - 1) / QT;
+  dim3 grid(a.n_splits, a.H, num_groups * mtiles), block(512);
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefix_mfma8_kernel<E, TQ>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kTile8Lds);
+  PH_LAUNCH_TIMED((prefix_mfma8_kernel<E, TQ>), grid, block, kTile8Lds, st, ev, a, mtiles);
+}
+
 template <typename E>
 static int launch_prefix_t(const PrefixArgs& a, int num_groups, int max_group_reqs, hipStream_t st) {
   const KernelEvents ev = take_kernel_events(0);
@@ -1006,12 +1021,12 @@ static int launch_prefix_t(const PrefixArgs& a, int num_groups, int max_group_re
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefix_mfma_kernel<E, 1>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, tile_lds_bytes<1>());
     PH_LAUNCH_TIMED((prefix_mfma_kernel<E, 1>), grid, block, tile_lds_bytes<1>(), st, ev, a, 1);
-  } else {                     // eight waves, 64-query tiles
-    const int mtiles = (max_group_reqs + 63) / 64;
-    dim3 grid(a.n_splits, a.H, num_groups * mtiles), block(512);
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefix_mfma8_kernel<E>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, kTile8Lds);
-    PH_LAUNCH_TIMED((prefix_mfma8_kernel<E>), grid, block, kTile8Lds, st, ev, a, mtiles);
+  } else if (max_group_reqs <= 64) {   // eight waves, 64-query tiles
+    launch_prefix8<E, 4>(a, num_groups, max_group_reqs, st, ev);
+  } else if (max_group_reqs <= 128) {  // 128-query tiles: the prefix is read once for up to 128 requests
+    launch_prefix8<E, 2>(a, num_groups, max_group_reqs, st, ev);
+  } else {                             // 256-query tiles
+    launch_prefix8<E, 1>(a, num_groups, max_group_reqs, st, ev);
   }
   return launch_status();
 }
@@ -1038,10 +1053,11 @@ static int launch_prefill_t(const PrefillArgs& a, int64_t num_tokens, hipStream_
   return launch_prefill_tq<E, 4, 1>(a, num_tokens, st);
 }
 
-template <typename E>
-static int launch_fused_t(const PrefixArgs& a, const ItemArgs& ia, int num_groups, int max_group_reqs, int cus,
-                          hipStream_t st) {
-  const int mtiles = (max_group_reqs + 63) / 64;
+template <typename E, int TQ>
+static int launch_fused_tq(const PrefixArgs& a, const ItemArgs& ia, int num_groups, int max_group_reqs, int cus,
+                           hipStream_t st) {
+  constexpr int QT = 32 * (8 / TQ);
+  const int mtiles = (max_group_reqs + QT - 1) / QT;
   const int n_units = a.n_splits * a.H * num_groups * mtiles;
   const int hgroups = (ia.H + 3) / 4;
   const int wave_slots = ia.num_lanes * hgroups;
@@ -1049,12 +1065,21 @@ static int launch_fused_t(const PrefixArgs& a, const ItemArgs& ia, int num_group
   const int unit_grid = n_units < cus ? n_units : cus;
   if (grid < unit_grid) grid = unit_grid;
   if (grid <= 0) return PH_OK;
-  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&decode_fused_kernel<E>),
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&decode_fused_kernel<E, TQ>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, kTile8Lds);
   const KernelEvents ev = take_kernel_events(1);
-  PH_LAUNCH_TIMED((decode_fused_kernel<E>), dim3(grid), dim3(512), kTile8Lds, st, ev, a, mtiles,
+  PH_LAUNCH_TIMED((decode_fused_kernel<E, TQ>), dim3(grid), dim3(512), kTile8Lds, st, ev, a, mtiles,
                         n_units, ia);
   return launch_status();
+}
+
+// query tile by the largest group: 64, 128 or 256 requests share each K/V tile of the prefix
+template <typename E>
+static int launch_fused_t(const PrefixArgs& a, const ItemArgs& ia, int num_groups, int max_group_reqs, int cus,
+                          hipStream_t st) {
+  if (max_group_reqs <= 64) return launch_fused_tq<E, 4>(a, ia, num_groups, max_group_reqs, cus, st);
+  if (max_group_reqs <= 128) return launch_fused_tq<E, 2>(a, ia, num_groups, max_group_reqs, cus, st);
+  return launch_fused_tq<E, 1>(a, ia, num_groups, max_group_reqs, cus, st);
 }
 
 // One launch for the prefix and suffix phases: head size 128, groups of more than 32 requests (the

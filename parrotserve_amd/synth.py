@@ -55,9 +55,14 @@ def _randn(gen, shape, dtype):
 
 
 def make_decode_case(name: str, seed: int, dtype: torch.dtype, groups: int, reqs_per_group: int, prefix_len: int,
-                     suffix_lens: Sequence[int], num_heads: int, head_dim: int, pool_slots: int) -> DecodeCase:
+                     suffix_lens: Sequence[int], num_heads: int, head_dim: int, pool_slots: int,
+                     group_sizes: Sequence[int] = ()) -> DecodeCase:
+    """``groups`` prefix groups of ``reqs_per_group`` requests each, or of ``group_sizes[g]`` requests when given
+    (``reqs_per_group`` is then ignored)."""
     gen = torch.Generator().manual_seed(seed)
-    B = groups * reqs_per_group
+    if group_sizes:
+        assert len(group_sizes) == groups
+    B = int(sum(group_sizes)) if group_sizes else groups * reqs_per_group
     assert len(suffix_lens) == B
     n_used = groups * prefix_len + int(sum(suffix_lens))
     assert n_used <= pool_slots
@@ -75,7 +80,14 @@ def make_decode_case(name: str, seed: int, dtype: torch.dtype, groups: int, reqs
     q = _randn(gen, (B, num_heads, head_dim), dtype)
     k = _randn(gen, (n_used, num_heads, head_dim), dtype)
     v = _randn(gen, (n_used, num_heads, head_dim), dtype)
-    gcu = [g * reqs_per_group for g in range(groups + 1)] if prefix_len > 0 else []
+    if group_sizes:
+        gcu = [0]
+        for n in group_sizes:
+            gcu.append(gcu[-1] + int(n))
+    else:
+        gcu = [g * reqs_per_group for g in range(groups + 1)]
+    if prefix_len <= 0:
+        gcu = []
     return DecodeCase(name, dtype, q, k, v, used, pool_slots, prefix_lists if prefix_len > 0 else [], gcu,
                       suffix_lists)
 

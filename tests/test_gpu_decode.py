@@ -376,6 +376,30 @@ def test_decode_attention_replays_from_a_captured_graph(dev):
     torch.testing.assert_close(out_static.cpu().float(), ref.float(), **TOL[torch.float16])
 
 
+@pytest.mark.parametrize("sizes", [[100], [128], [129], [200, 40], [257], [300, 70, 3]])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_large_groups_take_wider_query_tiles(dev, sizes, dtype):
+    """Groups of more than 64 requests share each prefix tile among 128 or 256 queries (one read of the prefix
+    per group instead of one per 64 requests); mixed with smaller groups, partial last tiles, both element types."""
+    from parrotserve_amd import kernels, synth
+
+    g = torch.Generator().manual_seed(31 + sum(sizes))
+    B = sum(sizes)
+    lens = torch.randint(0, 40, (B,), generator=g).tolist()
+    case = synth.make_decode_case("wide", 31, dtype, len(sizes), B, 333, lens, 3, 128, 1 << 14, group_sizes=sizes)
+    kc, vc = synth.pool_to_device(case.k_rows, case.v_rows, case.used_slots, case.pool_slots, dev)
+    tables = kernels.DecodeTables.build(case.pool_lists(case.prefix_lists), case.group_req_cu,
+                                        case.pool_lists(case.suffix_lists), dev, num_heads=3, head_dim=128)
+    out = kernels.decode_attention(case.q.to(dev), kc, vc, tables).cpu()
+    ref = ref_decode_attention(case.q, case.k_rows, case.v_rows, case.full_lists())
+    torch.testing.assert_close(out.float(), ref.float(), **TOL[dtype])
+    # the same batch without the balanced plan: prefix kernel on its own launch
+    plain = kernels.DecodeTables.build(case.pool_lists(case.prefix_lists), case.group_req_cu,
+                                       case.pool_lists(case.suffix_lists), dev, num_heads=3, head_dim=128, balanced=False)
+    out2 = kernels.decode_attention(case.q.to(dev), kc, vc, plain).cpu()
+    torch.testing.assert_close(out2.float(), ref.float(), **TOL[dtype])
+
+
 def test_captured_decode_step_replays_while_contexts_grow(dev):
     """One decode step recorded once, replayed over six iterations in which every request gains a token: the slot
     tables are patched and the suffix plan rewritten in place between replays (fixed pointers, counts and workspace
