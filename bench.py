@@ -399,6 +399,9 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run the move kernel as a plain 1 GiB copy (known traffic, to scale the profiler's "
                          "FETCH_SIZE / WRITE_SIZE counters) and exit")
+    ap.add_argument("--e2e-only", action="store_true",
+                    help="only run the 13B-shape decode experiment (fused per-layer ops) and exit (for a kernel trace "
+                         "of a whole engine iteration)")
     ap.add_argument("--prefill-only", action="store_true",
                     help="only run config 4's prefill kernel a few times (for profiler counter passes) and exit")
     args = ap.parse_args()
@@ -414,6 +417,10 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     lib = _lib.load()
+
+    if args.e2e_only:
+        print(json.dumps({"e2e_decode_13b_fused_ops": e2e_decode(torch, dev, fused_ops=True)}))
+        return
 
     if args.prefill_only:
         # config 4's prefill with parent context alone, a few launches (for counter collection on that kernel)
