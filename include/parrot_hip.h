@@ -179,13 +179,20 @@ int ph_rotary_embedding(void* state, const void* cos, const void* sin,
  *                 (the kernel prefetches slot ids before it knows a list's
  *                 length and clamps those reads to this bound);
  *   suffix_lens:  int32 [B] (DEVICE); max_suffix_len: host upper bound.
- * chunk_tokens: suffix split size (multiple of 16), 0 = choose.
+ * chunk_tokens: suffix split size of the plain (request, chunk) grid form
+ *   (multiple of 16); 0 = leave the decomposition to the library.
  * plan (HOST struct of DEVICE pointers, may be NULL): a caller that knows the
  *   suffix lengths on the host (the reference builds them from Python lists,
  *   attn_func.py:523-531) cuts the batch's suffix token stream into num_lanes
  *   near-equal pieces; a piece is one or more items (request, first token,
  *   token count).  The suffix phase then runs one wave set per piece, every wave
  *   moving the same number of bytes, instead of one per fixed-size chunk.
+ *   With plan == NULL and chunk_tokens == 0 the library builds the same plan
+ *   itself, on the device, at the start of the call (ph_suffix_plan_build into
+ *   the workspace; up to 8192 requests, a few microseconds per call) -- a
+ *   caller that runs many layers per iteration saves that by building the plan
+ *   once and passing it.  plan == NULL with chunk_tokens > 0, or more than
+ *   8192 requests, runs the grid form.
  *   items:        int32 [num_items][4] = request, first token, count, 0, in
  *                 request order (a request's items are consecutive, its tokens
  *                 ascending and covered exactly once);
@@ -329,6 +336,18 @@ int ph_rope_append(const int64_t* positions, void* q, void* k, const void* v,
  * untouched (the caller widens the table first).  All pointers DEVICE. */
 int ph_suffix_tables_append(int32_t* table, int64_t table_stride, int32_t* lens, const int32_t* rows,
                             const int32_t* new_slots, int64_t n, void* stream);
+
+/* Balanced suffix plan built on the device from the length vector alone (the
+ * three arrays of ph_suffix_plan; see ph_decode_attention): one small launch
+ * per iteration in place of host-side list work and an upload.  items must
+ * hold num_lanes + num_reqs entries of 4 ints, lane_rec num_lanes entries of
+ * 8, req_item_cu num_reqs + 1.  The stream is cut into
+ * min(num_lanes, ceil(total / 16)) pieces; records of the remaining lanes are
+ * empty.  num_reqs <= 8192; the lengths must sum to less than 2^31.  The
+ * reference has no counterpart (its kernels take fixed-size blocks per
+ * request, attention_post_kernels.cu:74-110). */
+int ph_suffix_plan_build(const int32_t* suffix_lens, int64_t num_reqs, int64_t num_lanes,
+                         int32_t* items, int32_t* lane_rec, int32_t* req_item_cu, void* stream);
 
 /* ------------------------------------------------------------------------ */
 /* Instrumentation (no counterpart in the reference, which times whole

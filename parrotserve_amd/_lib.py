@@ -40,6 +40,7 @@ SIGNATURES: Dict[str, Tuple[object, List[object]]] = {
     "ph_rope_append": (I, [P, P, P, P, P, P, P, P, I, L, L, L, L, L, L, L, L, L, I, P]),
     "ph_suffix_tables_append": (I, [P, L, P, P, P, L, P]),
     "ph_arm_kernel_events": (I, [P]),
+    "ph_suffix_plan_build": (I, [P, L, L, P, P, P, P]),
     "ph_prefill_workspace_bytes": (Z, [L, L, L, L]),
     "ph_prefill_attention": (I, [P, P, P, P, L, L, L, L, I, L, L, L, F, P, P, P, L, L, P, Z, P]),
 }

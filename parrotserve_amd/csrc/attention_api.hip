@@ -11,6 +11,7 @@ struct DecodePlan {
   int split_tokens;  // prefix tokens per part
   int n_splits;      // prefix parts
   int64_t items;     // suffix items (balanced form), 0 in the grid form
+  int dev_lanes;     // lanes of a plan the library builds on the device into the workspace (0: the caller's plan or none)
   int parts() const { return n_chunks + n_splits; }
   // partial rows (one row = one head's (O, m, l)): [parts][B][H] then [items][H]
   size_t rows(int64_t B, int64_t H) const { return (size_t)parts() * B * H + (size_t)items * H; }
@@ -22,11 +23,34 @@ static int64_t cdiv(int64_t x, int64_t m) { return (x + m - 1) / m; }
 constexpr int kPrefixTile = 64;        // tokens per LDS tile of the MFMA kernel
 constexpr int kPrefixQueryTile = 64;   // queries per workgroup of the MFMA kernel
 
+// compute units of the current device (cached per device id)
+static int device_cus() {
+  static int cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
+
+// plan_head_dim > 0: a caller without a plan of its own that leaves the chunk size to the library gets the
+// balanced form from a plan built on the device (up to kPlanMaxReqs requests); an explicit chunk size keeps the
+// plain (request, chunk) grid.
 static DecodePlan plan_decode(int64_t B, int64_t H, int64_t groups, int64_t max_prefix, int64_t max_suffix,
-                              int64_t chunk_tokens, int64_t num_items = 0) {
+                              int64_t chunk_tokens, int64_t num_items = 0, int64_t plan_head_dim = 0) {
   DecodePlan p{};
   p.items = num_items;
   if (num_items > 0) {
+    p.chunk = 32;
+    p.n_chunks = 0;
+  } else if (max_suffix > 0 && chunk_tokens <= 0 && plan_head_dim >= 8 && B <= kPlanMaxReqs) {
+    const int64_t heads_per_wave = 64 / (plan_head_dim / 8) > 0 ? 64 / (plan_head_dim / 8) : 1;
+    const int64_t lanes = (int64_t)device_cus() * 4 * 2 / cdiv(H, heads_per_wave);  // two waves per SIMD
+    p.dev_lanes = (int)(lanes > 0 ? lanes : 1);
+    p.items = p.dev_lanes + B;  // capacity: a cut at every lane mark and every request boundary
     p.chunk = 32;
     p.n_chunks = 0;
   } else if (max_suffix > 0) {
@@ -72,18 +96,32 @@ static DecodePlan plan_decode(int64_t B, int64_t H, int64_t groups, int64_t max_
 
 static size_t plan_bytes(const DecodePlan& p, int64_t B, int64_t H, int64_t D) {
   const size_t rows = p.rows(B, H);
-  return round_up((int64_t)(rows * D * sizeof(float)), 256) + round_up((int64_t)(rows * 2 * sizeof(float)), 256);
+  size_t n = round_up((int64_t)(rows * D * sizeof(float)), 256) + round_up((int64_t)(rows * 2 * sizeof(float)), 256);
+  if (p.dev_lanes > 0)
+    n += round_up(p.items * 16, 256) + round_up((int64_t)p.dev_lanes * 32, 256) + round_up((B + 1) * 4, 256);
+  return n;
 }
 
 struct Carve {
   float* opart;
   float* ml;
+  int32_t *items, *lane_rec, *req_item_cu;  // the device-built plan (dev_lanes > 0)
 };
 static Carve carve(void* ws, const DecodePlan& p, int64_t B, int64_t H, int64_t D) {
   const size_t rows = p.rows(B, H);
-  Carve c;
-  c.opart = (float*)ws;
-  c.ml = (float*)((char*)ws + round_up((int64_t)(rows * D * sizeof(float)), 256));
+  Carve c{};
+  char* at = (char*)ws;
+  c.opart = (float*)at;
+  at += round_up((int64_t)(rows * D * sizeof(float)), 256);
+  c.ml = (float*)at;
+  at += round_up((int64_t)(rows * 2 * sizeof(float)), 256);
+  if (p.dev_lanes > 0) {
+    c.items = (int32_t*)at;
+    at += round_up(p.items * 16, 256);
+    c.lane_rec = (int32_t*)at;
+    at += round_up((int64_t)p.dev_lanes * 32, 256);
+    c.req_item_cu = (int32_t*)at;
+  }
   return c;
 }
 
@@ -169,19 +207,6 @@ extern "C" const char* ph_status_string(int status) {
 
 extern "C" int ph_abi_version(void) { return 1; }
 
-// compute units of the current device (cached per device id)
-static int device_cus() {
-  static int cached[64];
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-  if (cached[dev] == 0) {
-    int n = 0;
-    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-    cached[dev] = n;
-  }
-  return cached[dev];
-}
-
 static hipEvent_t g_kernel_events[6];
 static bool g_events_armed = false;
 
@@ -206,7 +231,7 @@ extern "C" size_t ph_decode_workspace_bytes(int64_t num_reqs, int64_t num_heads,
                                             int64_t chunk_tokens, int64_t num_items) {
   if (num_reqs <= 0 || num_heads <= 0 || head_dim <= 0) return 0;
   const DecodePlan p =
-      plan_decode(num_reqs, num_heads, num_groups, max_prefix_len, max_suffix_len, chunk_tokens, num_items);
+      plan_decode(num_reqs, num_heads, num_groups, max_prefix_len, max_suffix_len, chunk_tokens, num_items, head_dim);
   return plan_bytes(p, num_reqs, num_heads, head_dim);
 }
 
@@ -229,16 +254,25 @@ extern "C" int ph_decode_attention(void* out, const void* q, const void* k_cache
   const bool has_suffix = max_suffix_len > 0;
   if (has_prefix && (!prefix_slots || !prefix_cu || !group_req_cu || !group_req_cu_host)) return PH_ERR_ARG;
   if (has_suffix && (!suffix_slots || !suffix_lens || suffix_slots_count <= 0)) return PH_ERR_ARG;
-  const bool planned = has_suffix && plan != nullptr && plan->num_items > 0;
+  bool planned = has_suffix && plan != nullptr && plan->num_items > 0;
   if (planned && (!plan->items || !plan->lane_rec || !plan->req_item_cu || plan->num_lanes <= 0 ||
                   plan->num_items > (int64_t)1 << 30))
     return PH_ERR_ARG;
   const DecodePlan p = plan_decode(num_reqs, num_heads, has_prefix ? num_groups : 0, max_prefix_len, max_suffix_len,
-                                   chunk_tokens, planned ? plan->num_items : 0);
-  if (plan_bytes(p, B, H, D) > workspace_bytes || (p.parts() > 0 && !workspace)) return PH_ERR_WORKSPACE;
+                                   chunk_tokens, planned ? plan->num_items : 0, head_dim);
+  if (plan_bytes(p, B, H, D) > workspace_bytes || ((p.parts() > 0 || p.items > 0) && !workspace))
+    return PH_ERR_WORKSPACE;
   if (((uintptr_t)workspace & 255u) != 0) return PH_ERR_ALIGN;
   const Carve ws = carve(workspace, p, B, H, D);
   hipStream_t st = (hipStream_t)stream;
+  ph_suffix_plan own_plan{};
+  if (!planned && p.dev_lanes > 0) {  // no plan from the caller: one is built on the device first
+    rc = launch_suffix_plan(suffix_lens, B, p.dev_lanes, ws.items, ws.lane_rec, ws.req_item_cu, st);
+    if (rc != PH_OK) return rc;
+    own_plan = ph_suffix_plan{ws.items, p.items, ws.lane_rec, p.dev_lanes, ws.req_item_cu};
+    plan = &own_plan;
+    planned = true;
+  }
   const float sl2 = scale * kLog2e;
   bool fuse = false;  // prefix and suffix phases in one launch
   PrefixArgs fused_pa{};
@@ -416,12 +450,34 @@ extern "C" int ph_suffix_post_attention(void* out, const float* prev_m, const fl
   if (max_suffix_len < 0 || !prev_m || !prev_l) return PH_ERR_ARG;
   const bool has_suffix = max_suffix_len > 0;
   if (has_suffix && (!suffix_slots || !suffix_lens || suffix_slots_count <= 0)) return PH_ERR_ARG;
-  const DecodePlan p = plan_decode(num_reqs, num_heads, 0, 0, max_suffix_len, chunk_tokens);
-  if (plan_bytes(p, B, H, D) > workspace_bytes || (p.parts() > 0 && !workspace)) return PH_ERR_WORKSPACE;
+  const DecodePlan p = plan_decode(num_reqs, num_heads, 0, 0, max_suffix_len, chunk_tokens, 0, head_dim);
+  if (plan_bytes(p, B, H, D) > workspace_bytes || ((p.parts() > 0 || p.items > 0) && !workspace))
+    return PH_ERR_WORKSPACE;
   if (((uintptr_t)workspace & 255u) != 0) return PH_ERR_ALIGN;
   const Carve ws = carve(workspace, p, B, H, D);
   hipStream_t st = (hipStream_t)stream;
-  if (has_suffix) {
+  if (has_suffix && p.dev_lanes > 0) {  // balanced form on a plan built on the device
+    rc = launch_suffix_plan(suffix_lens, B, p.dev_lanes, ws.items, ws.lane_rec, ws.req_item_cu, st);
+    if (rc != PH_OK) return rc;
+    ItemArgs ia{};
+    ia.q = (const uint16_t*)q;
+    ia.q_stride = q_stride;
+    ia.kc = (const uint16_t*)k_cache;
+    ia.vc = (const uint16_t*)v_cache;
+    ia.row_stride = cache_stride_n;
+    ia.slots = suffix_slots;
+    ia.offsets = suffix_offsets;
+    ia.table_stride = suffix_table_stride;
+    ia.items = reinterpret_cast<const int4*>(ws.items);
+    ia.lane_rec = reinterpret_cast<const int4*>(ws.lane_rec);
+    ia.num_lanes = p.dev_lanes;
+    ia.opart = ws.opart;
+    ia.ml = ws.ml;
+    ia.H = H;
+    ia.scale_log2e = scale * kLog2e;
+    rc = launch_items(ia, dtype, D, st);
+    if (rc != PH_OK) return rc;
+  } else if (has_suffix) {
     PartialArgs sa{};
     sa.q = (const uint16_t*)q;
     sa.q_stride = q_stride;
@@ -459,6 +515,8 @@ extern "C" int ph_suffix_post_attention(void* out, const float* prev_m, const fl
   ma.baseB = 0;
   ma.lens = has_suffix ? suffix_lens : nullptr;
   ma.chunk = p.chunk;
+  ma.req_item_cu = has_suffix && p.dev_lanes > 0 ? ws.req_item_cu : nullptr;
+  ma.item_base = 0;
   ma.prev_m = prev_m;
   ma.prev_l = prev_l;
   return launch_merge(ma, dtype, D, st);

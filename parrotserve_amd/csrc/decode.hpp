@@ -109,6 +109,10 @@ int launch_prefill_mfma(const PrefillArgs& a, int dtype, int D, int64_t num_toke
 int launch_items(const ItemArgs& a, int dtype, int D, hipStream_t st);
 int launch_merge(const MergeArgs& a, int dtype, int D, hipStream_t st);
 int launch_clear_ml(float* ml, int64_t entries, hipStream_t st);
+// balanced suffix plan written on the device from the length vector (tables.hip); arrays as in ph_suffix_plan
+constexpr int kPlanMaxReqs = 8192;
+int launch_suffix_plan(const int32_t* lens, int B, int lanes, int32_t* items, int32_t* lane_rec, int32_t* req_item_cu,
+                       hipStream_t st);
 // MFMA shared-prefix kernel: grid (split, head, group x m-tile).
 int launch_prefix_mfma(const PrefixArgs& a, int dtype, int D, int num_groups, int max_group_reqs, hipStream_t st);
 bool prefix_mfma_supported(int dtype, int D);

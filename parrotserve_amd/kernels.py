@@ -398,6 +398,27 @@ class DecodeTables:
         self.plan = _lib.SuffixPlan(self.plan_items.data_ptr(), cap, self.plan_lane_item_cu.data_ptr(),
                                     lanes, self.plan_req_item_cu.data_ptr())
 
+    def plan_on_device(self, num_lanes: int, device) -> None:
+        """The balanced plan written by the library from the device length vector (``ph_suffix_plan_build``): no
+        host-side list work, no upload.  ``num_lanes`` is the lane capacity (``suffix_lane_capacity``); the planner
+        uses as many of them as the token count warrants.  The arrays keep their place from call to call."""
+        B = self.num_reqs
+        cap = num_lanes + B
+        o_rec = cap * 4
+        o_cu = o_rec + num_lanes * 8
+        n = o_cu + B + 1
+        buf = self.plan_buffer
+        if buf is None or buf.numel() != n or self.plan is None or self.plan.num_lanes != num_lanes or \
+                self.plan.num_items != cap:
+            buf = torch.zeros(n, dtype=torch.int32, device=device)
+            self.plan_buffer = buf
+            self.plan_items = buf[:o_rec].view(cap, 4)
+            self.plan_lane_item_cu = buf[o_rec:o_cu].view(num_lanes, 8)
+            self.plan_req_item_cu = buf[o_cu:]
+            self.plan = _lib.SuffixPlan(self.plan_items.data_ptr(), cap, self.plan_lane_item_cu.data_ptr(),
+                                        num_lanes, self.plan_req_item_cu.data_ptr())
+        suffix_plan_build(self.suffix_lens, num_lanes, self.plan_items, self.plan_lane_item_cu, self.plan_req_item_cu)
+
     @staticmethod
     def build(prefix_lists: Sequence[Sequence[int]], group_req_cu: Sequence[int],
               suffix_lists: Sequence[Sequence[int]], device, num_heads: int = 32, head_dim: int = 128,
@@ -449,7 +470,10 @@ class DecodeTables:
                 chunk *= 2
             t.chunk_tokens = chunk
             if balanced:
-                t.set_plan(lens, suffix_lanes(device, num_heads, head_dim, total), device)
+                if B <= PLAN_MAX_REQS and t.suffix_offsets is None:
+                    t.plan_on_device(suffix_lane_capacity(device, num_heads, head_dim), device)
+                else:
+                    t.set_plan(lens, suffix_lanes(device, num_heads, head_dim, total), device)
         return t
 
 
@@ -476,6 +500,28 @@ def suffix_tables_append(table: torch.Tensor, lens: torch.Tensor, rows: Optional
     assert rows is None or (rows.dtype == torch.int32 and rows.numel() == new_slots.numel())
     check(_lib.load().ph_suffix_tables_append(_ptr(table), table.stride(0), _ptr(lens), _ptr(rows), _ptr(new_slots),
                                               new_slots.numel(), _stream()), "suffix_tables_append")
+
+
+def suffix_plan_build(lens: torch.Tensor, num_lanes: int, items: torch.Tensor, lane_rec: torch.Tensor,
+                      req_item_cu: torch.Tensor) -> None:
+    """The balanced suffix plan written on the device from the device length vector (``ph_suffix_plan_build``):
+    ``items [num_lanes + B, 4]``, ``lane_rec [num_lanes, 8]``, ``req_item_cu [B + 1]``, all int32."""
+    _require_gpu(lens, items, lane_rec, req_item_cu)
+    B = lens.numel()
+    assert lens.dtype == items.dtype == lane_rec.dtype == req_item_cu.dtype == torch.int32
+    assert items.numel() >= (num_lanes + B) * 4 and lane_rec.numel() >= num_lanes * 8 and req_item_cu.numel() >= B + 1
+    check(_lib.load().ph_suffix_plan_build(_ptr(lens), B, num_lanes, _ptr(items), _ptr(lane_rec), _ptr(req_item_cu),
+                                           _stream()), "suffix_plan_build")
+
+
+PLAN_MAX_REQS = 8192  # batch size up to which the library plans on the device
+
+
+def suffix_lane_capacity(device, num_heads: int, head_dim: int) -> int:
+    """Lanes of the device-built plan: one launch-wide round of waves at two waves per SIMD (see suffix_lanes)."""
+    heads_per_wave = max(1, 64 // max(1, head_dim // 8))
+    hgroups = (num_heads + heads_per_wave - 1) // heads_per_wave
+    return max(1, _cu_count(device) * 4 * 2 // hgroups)
 
 
 def suffix_lanes(device, num_heads: int, head_dim: int, total_tokens: int) -> int:

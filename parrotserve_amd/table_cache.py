@@ -7,7 +7,8 @@ same batch nothing changes except that every Generate job's context gained the
 one slot of the token being generated, so the device tables of the previous
 iteration are patched instead: O(batch) host work, one upload of the new slots,
 one tiny kernel (``ph_suffix_tables_append``), and a fresh balanced suffix plan
-(its cut points move with the lengths).
+(its cut points move with the lengths) that a second tiny kernel writes from
+the device length vector (``ph_suffix_plan_build``).
 
 A batch qualifies when it consists of Generate jobs only, bound to the same
 context objects in the same order as the cached iteration, each context exactly
@@ -90,8 +91,11 @@ class DecodeTableCache:
         c.slot_mapping = torch.from_numpy(np.asarray(new_slots, dtype=np.int32)).to(device)
         kernels.suffix_tables_append(t.suffix_slots, t.suffix_lens, c.rows, c.slot_mapping)
         t.max_suffix_len = need
-        total = int(c.lens_host.sum())
-        t.set_plan(c.lens_host, kernels.suffix_lanes(device, c.num_heads, c.head_dim, total), device)
+        if t.num_reqs <= kernels.PLAN_MAX_REQS:  # the cut points move with the lengths: a fresh plan, built on the device
+            t.plan_on_device(kernels.suffix_lane_capacity(device, c.num_heads, c.head_dim), device)
+        else:
+            total = int(c.lens_host.sum())
+            t.set_plan(c.lens_host, kernels.suffix_lanes(device, c.num_heads, c.head_dim, total), device)
         self.hits += 1
         return c
 

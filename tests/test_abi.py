@@ -87,6 +87,10 @@ def test_argument_validation_needs_no_gpu():
     gv = lambda n, bs: lib.ph_gather_blocked_v(None, None, None, None, 0, n, 2, 128, bs, 2, 4096, 2048, 16, 1, 256, 128,
                                                1, None)
     assert gv(4, 16) == _lib.PH_ERR_ARG and gv(0, 16) == _lib.PH_OK and gv(4, 0) == _lib.PH_ERR_ARG
+    assert lib.ph_suffix_plan_build(None, 4, 256, None, None, None, None) == _lib.PH_ERR_ARG      # null pointers
+    assert lib.ph_suffix_plan_build(None, 0, 256, None, None, None, None) == _lib.PH_OK           # no requests
+    assert lib.ph_suffix_plan_build(None, 8193, 256, None, None, None, None) == _lib.PH_ERR_ARG   # beyond the device planner
+    assert lib.ph_suffix_plan_build(None, 4, 0, None, None, None, None) == _lib.PH_ERR_ARG
     assert lib.ph_suffix_tables_append(None, 64, None, None, None, -1, None) == _lib.PH_ERR_ARG
     assert lib.ph_suffix_tables_append(None, 64, None, None, None, 0, None) == _lib.PH_OK
     assert lib.ph_suffix_tables_append(None, 64, None, None, None, 3, None) == _lib.PH_ERR_ARG

@@ -251,8 +251,10 @@ def test_incremental_tables_match_full_rebuild_over_a_decode_loop(dev, name, n_g
         assert ti.suffix_slots.shape[1] >= w
         cols = torch.arange(w, device=dev)[None, :] < tf.suffix_lens[:, None]
         assert torch.equal(torch.where(cols, ti.suffix_slots[:, :w], 0), torch.where(cols, tf.suffix_slots, 0))
-        assert torch.equal(ti.plan_items, tf.plan_items) and torch.equal(ti.plan_lane_item_cu, tf.plan_lane_item_cu)
         assert torch.equal(ti.plan_req_item_cu, tf.plan_req_item_cu)
+        n_items = int(tf.plan_req_item_cu[-1])  # rows of the item array in use (the rest keeps older contents)
+        assert torch.equal(ti.plan_items[:n_items], tf.plan_items[:n_items])
+        assert torch.equal(ti.plan_lane_item_cu, tf.plan_lane_item_cu)
         assert (st_i.decode_perm is None) == (st_f.decode_perm is None)
         if st_i.decode_perm is not None:
             assert torch.equal(st_i.decode_perm[0], st_f.decode_perm[0])
@@ -263,3 +265,37 @@ def test_incremental_tables_match_full_rebuild_over_a_decode_loop(dev, name, n_g
             o_f = attn_full(q, k, v, st_f)  # appends the same rows again: idempotent
             assert torch.equal(o_i, o_f)
     assert Inc.table_cache.hits == 39 and Inc.table_cache.rebuilds == 1
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_device_suffix_plan_equals_the_host_plan(dev, seed):
+    """ph_suffix_plan_build against the numpy planner: same items, lane records and per-request offsets, for ragged
+    batches with empty requests, fewer tokens than lanes, one request, and lengths that are multiples of the cut."""
+    from parrotserve_amd import kernels
+
+    g = torch.Generator().manual_seed(50 + seed)
+    B = [1, 2, 7, 64, 64, 200, 333, 1000, 5, 8192][seed]
+    hi = [5000, 40, 3, 512, 16, 2000, 100, 64, 8192, 30][seed]
+    lens = torch.randint(0, hi + 1, (B,), generator=g)
+    if seed in (2, 6):
+        lens[torch.rand(B, generator=g) < 0.4] = 0
+    if seed == 4:
+        lens[:] = 16
+    lanes_cap = [256, 256, 256, 256, 512, 128, 2048, 37, 256, 256][seed]
+    total = int(lens.sum())
+    items = torch.full(((lanes_cap + B), 4), -1, dtype=torch.int32, device=dev)
+    rec = torch.full((lanes_cap, 8), -1, dtype=torch.int32, device=dev)
+    rcu = torch.full((B + 1,), -1, dtype=torch.int32, device=dev)
+    kernels.suffix_plan_build(lens.to(torch.int32).to(dev), lanes_cap, items, rec, rcu)
+    lanes = max(1, min(lanes_cap, (total + 15) // 16))
+    h_items, h_lane_cu, h_rcu = kernels.plan_suffix_items(lens.tolist(), lanes)
+    n = h_items.shape[0]
+    assert torch.equal(rcu.cpu(), torch.from_numpy(h_rcu))
+    assert torch.equal(items[:n].cpu(), torch.from_numpy(h_items))
+    rec = rec.cpu()
+    eff = h_lane_cu.shape[0] - 1
+    if n:
+        assert torch.equal(rec[:eff, 0], torch.from_numpy(h_lane_cu[:-1]))
+        assert torch.equal(rec[:eff, 1], torch.from_numpy(h_lane_cu[1:] - h_lane_cu[:-1]))
+        assert torch.equal(rec[:eff, 2:5], torch.from_numpy(h_items[h_lane_cu[:-1], 0:3]))
+    assert (rec[eff:, 1] == 0).all()  # lanes beyond the cut count own nothing

@@ -400,9 +400,30 @@ def test_large_groups_take_wider_query_tiles(dev, sizes, dtype):
     torch.testing.assert_close(out2.float(), ref.float(), **TOL[dtype])
 
 
+@pytest.mark.parametrize("groups,B,P", [(1, 48, 600), (2, 20, 300), (0, 37, 0)])
+def test_library_plans_for_callers_without_a_plan(dev, groups, B, P):
+    """No plan from the caller and the chunk size left to the library (0): the library builds the balanced plan on
+    the device inside the call (workspace from the same query) -- one large group (single-launch path), small
+    groups (prefix kernel + balanced suffix) and a ragged batch without any prefix."""
+    from parrotserve_amd import kernels, synth
+
+    g = torch.Generator().manual_seed(41 + B)
+    n = max(1, groups) * B
+    lens = torch.randint(0, 300, (n,), generator=g).tolist()
+    case = synth.make_decode_case("noplan", 41, torch.float16, max(1, groups), B, P if groups else 0, lens, 5, 128, 1 << 15)
+    kc, vc = synth.pool_to_device(case.k_rows, case.v_rows, case.used_slots, case.pool_slots, dev)
+    tables = kernels.DecodeTables.build(case.pool_lists(case.prefix_lists), case.group_req_cu,
+                                        case.pool_lists(case.suffix_lists), dev, num_heads=5, head_dim=128, balanced=False)
+    assert tables.plan is None
+    tables.chunk_tokens = 0
+    out = kernels.decode_attention(case.q.to(dev), kc, vc, tables).cpu()
+    ref = ref_decode_attention(case.q, case.k_rows, case.v_rows, case.full_lists())
+    torch.testing.assert_close(out.float(), ref.float(), **TOL[torch.float16])
+
+
 def test_captured_decode_step_replays_while_contexts_grow(dev):
     """One decode step recorded once, replayed over six iterations in which every request gains a token: the slot
-    tables are patched and the suffix plan rewritten in place between replays (fixed pointers, counts and workspace
+    tables are patched and the suffix plan rebuilt in place (on the device) between replays (fixed pointers, counts and workspace
     layout), and each replay must equal the eager result on tables built from scratch for that iteration."""
     from parrotserve_amd import kernels, synth, table_cache
 
@@ -417,7 +438,7 @@ def test_captured_decode_step_replays_while_contexts_grow(dev):
     spare = [s for s in range(case.pool_slots) if s not in used][: 6 * B]
     tables = kernels.DecodeTables.build(prefix, case.group_req_cu, suffix, dev, num_heads=H, head_dim=D)
     table_cache._widen(tables, max(lens) + 8, dev)          # room for the tokens to come
-    lanes = tables.plan.num_lanes
+    lanes = kernels.suffix_lane_capacity(dev, H, D)
     q_static = case.q.to(dev)
     out_static = torch.empty_like(q_static)
     side = torch.cuda.Stream()
@@ -440,11 +461,10 @@ def test_captured_decode_step_replays_while_contexts_grow(dev):
             suffix[b].append(new[b])
         kernels.suffix_tables_append(tables.suffix_slots, tables.suffix_lens, None, new_dev)
         tables.max_suffix_len += 1
-        tables.set_plan([len(l) for l in suffix], lanes, dev)
+        tables.plan_on_device(lanes, dev)
         assert (tables.plan.items, tables.plan.num_items, tables.plan.lane_rec, tables.plan.num_lanes) == plan_ptrs
         q_new = torch.randn(q_static.shape, generator=gq, device=dev, dtype=torch.float16)
         fresh = kernels.DecodeTables.build(prefix, case.group_req_cu, suffix, dev, num_heads=H, head_dim=D)
-        fresh.set_plan([len(l) for l in suffix], lanes, dev)  # the same cuts, so the same summation order
         eager = kernels.decode_attention(q_new, kc, vc, fresh)
         torch.cuda.synchronize()
         q_static.copy_(q_new)
