@@ -37,28 +37,40 @@ struct PlanScratch {
   int part[kPlanThreads];
 };
 
-// exclusive prefix sums of v(0..n-1) into out[0..n] by the whole workgroup (each thread owns a run)
+// exclusive prefix sums of v(0..n-1) into out[0..n] by the whole workgroup: each thread owns a run, the thread
+// sums are scanned inside each wave with lane shuffles and across the sixteen waves by the first wave
 template <typename F>
 __device__ __forceinline__ void block_scan(F v, int n, int* out, int* part) {
-  const int t = threadIdx.x;
+  const int t = threadIdx.x, lane = t & 63, w = t >> 6;
   const int per = (n + kPlanThreads - 1) / kPlanThreads;
   const int b0 = min(t * per, n), b1 = min(b0 + per, n);
   int s = 0;
   for (int i = b0; i < b1; ++i) s += v(i);
-  part[t] = s;
-  __syncthreads();
-  for (int d = 1; d < kPlanThreads; d <<= 1) {  // Hillis-Steele over the thread sums
-    const int add = t >= d ? part[t - d] : 0;
-    __syncthreads();
-    part[t] += add;
-    __syncthreads();
+  int inc = s;  // inclusive scan over the wave
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const int up = __shfl_up(inc, d, kWave);
+    if (lane >= d) inc += up;
   }
-  int run = t > 0 ? part[t - 1] : 0;
+  if (lane == kWave - 1) part[w] = inc;
+  __syncthreads();
+  if (w == 0) {
+    constexpr int NW = kPlanThreads / kWave;
+    int ws = lane < NW ? part[lane] : 0;
+#pragma unroll
+    for (int d = 1; d < NW; d <<= 1) {
+      const int up = __shfl_up(ws, d, kWave);
+      if (lane >= d) ws += up;
+    }
+    if (lane < NW) part[lane] = ws;  // inclusive over the waves
+  }
+  __syncthreads();
+  int run = inc - s + (w > 0 ? part[w - 1] : 0);
   for (int i = b0; i < b1; ++i) {
     out[i] = run;
     run += v(i);
   }
-  if (t == kPlanThreads - 1) out[n] = part[t];
+  if (t == kPlanThreads - 1) out[n] = run;
   __syncthreads();
 }
 
