@@ -262,6 +262,37 @@ int ph_suffix_post_attention(void* out, const float* prev_m, const float* prev_l
                              int64_t max_suffix_len, int64_t chunk_tokens,
                              void* workspace, size_t workspace_bytes, void* stream);
 
+/* The other order, which the reference's extension exports as well
+ * (csrc/attention.cpp:19-32, shared_flash_decoding.py:332-376): suffix phase
+ * first, prefix phase second.
+ *
+ * ph_suffix_prev_attention: suffix phase only -- writes the normalised O
+ * (element type) and m / l as fp32 [B, H] (m in the exp2 domain, l relative to
+ * m; l == 0 where a request has no suffix).  Replaces
+ * attention_ops.single_query_cached_kv_prev_attention
+ * (csrc/attention/attention_prev_kernels.cu:74-338).
+ *
+ * ph_prefix_post_attention: prefix phase over one shared slot list, then
+ * merge with the partial that already sits in out / prev_m / prev_l; out is
+ * in/out.  Replaces triton_flash_attention(..., load_mid_results=True)
+ * (shared_flash_decoding.py:202-277,332-376). */
+int ph_suffix_prev_attention(void* out, float* m_out, float* l_out,
+                             const void* q, const void* k_cache, const void* v_cache,
+                             int64_t num_reqs, int64_t num_heads, int64_t head_dim, int dtype,
+                             int64_t q_stride, int64_t out_stride, int64_t cache_stride_n, float scale,
+                             const int32_t* suffix_slots, const int64_t* suffix_offsets,
+                             int64_t suffix_table_stride, int64_t suffix_slots_count,
+                             const int32_t* suffix_lens,
+                             int64_t max_suffix_len, int64_t chunk_tokens,
+                             void* workspace, size_t workspace_bytes, void* stream);
+
+int ph_prefix_post_attention(void* out, const float* prev_m, const float* prev_l,
+                             const void* q, const void* k_cache, const void* v_cache,
+                             int64_t num_reqs, int64_t num_heads, int64_t head_dim, int dtype,
+                             int64_t q_stride, int64_t out_stride, int64_t cache_stride_n, float scale,
+                             const int32_t* prefix_slots, int64_t prefix_len,
+                             void* workspace, size_t workspace_bytes, void* stream);
+
 /* ------------------------------------------------------------------------ */
 /* Prefill with parent context: packed ragged chunks, each causal
  * (bottom-right aligned) over ancestors' + own KV read through a slot table.

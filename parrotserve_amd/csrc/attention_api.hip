@@ -382,16 +382,18 @@ extern "C" int ph_decode_attention(void* out, const void* q, const void* k_cache
   return rc;
 }
 
-extern "C" int ph_prefix_attention(void* out, float* m_out, float* l_out, const void* q, const void* k_cache,
-                                   const void* v_cache, int64_t num_reqs, int64_t num_heads, int64_t head_dim,
-                                   int dtype, int64_t q_stride, int64_t out_stride, int64_t cache_stride_n,
-                                   float scale, const int32_t* prefix_slots, int64_t prefix_len, void* workspace,
-                                   size_t workspace_bytes, void* stream) {
+// Prefix phase over one shared slot list, merged with an optional partial already in out / prev_m / prev_l; the
+// merged m / l are exported when asked for.
+static int prefix_phase(void* out, const float* prev_m, const float* prev_l, float* m_out, float* l_out, const void* q,
+                        const void* k_cache, const void* v_cache, int64_t num_reqs, int64_t num_heads,
+                        int64_t head_dim, int dtype, int64_t q_stride, int64_t out_stride, int64_t cache_stride_n,
+                        float scale, const int32_t* prefix_slots, int64_t prefix_len, void* workspace,
+                        size_t workspace_bytes, void* stream) {
   const int B = (int)num_reqs, H = (int)num_heads, D = (int)head_dim;
   int rc = check_common(out, q, k_cache, v_cache, num_reqs, num_heads, head_dim, dtype, q_stride, out_stride,
                         cache_stride_n);
   if (rc != PH_OK || num_reqs == 0) return rc;
-  if (prefix_len < 0 || !m_out || !l_out || (prefix_len > 0 && !prefix_slots)) return PH_ERR_ARG;
+  if (prefix_len < 0 || (prefix_len > 0 && !prefix_slots)) return PH_ERR_ARG;
   const DecodePlan p = plan_decode(num_reqs, num_heads, prefix_len > 0 ? 1 : 0, prefix_len, 0, 0);
   if (plan_bytes(p, B, H, D) > workspace_bytes || (p.parts() > 0 && !workspace)) return PH_ERR_WORKSPACE;
   if (((uintptr_t)workspace & 255u) != 0) return PH_ERR_ALIGN;
@@ -429,25 +431,50 @@ extern "C" int ph_prefix_attention(void* out, float* m_out, float* l_out, const 
   ma.baseB = p.n_splits;
   ma.lens = nullptr;
   ma.chunk = p.chunk;
+  ma.prev_m = prev_m;
+  ma.prev_l = prev_l;
   ma.m_out = m_out;
   ma.l_out = l_out;
   return launch_merge(ma, dtype, D, st);
 }
 
-extern "C" int ph_suffix_post_attention(void* out, const float* prev_m, const float* prev_l, const void* q,
+extern "C" int ph_prefix_attention(void* out, float* m_out, float* l_out, const void* q, const void* k_cache,
+                                   const void* v_cache, int64_t num_reqs, int64_t num_heads, int64_t head_dim,
+                                   int dtype, int64_t q_stride, int64_t out_stride, int64_t cache_stride_n,
+                                   float scale, const int32_t* prefix_slots, int64_t prefix_len, void* workspace,
+                                   size_t workspace_bytes, void* stream) {
+  if (num_reqs > 0 && (!m_out || !l_out)) return PH_ERR_ARG;
+  return prefix_phase(out, nullptr, nullptr, m_out, l_out, q, k_cache, v_cache, num_reqs, num_heads, head_dim, dtype,
+                      q_stride, out_stride, cache_stride_n, scale, prefix_slots, prefix_len, workspace,
+                      workspace_bytes, stream);
+}
+
+extern "C" int ph_prefix_post_attention(void* out, const float* prev_m, const float* prev_l, const void* q,
                                         const void* k_cache, const void* v_cache, int64_t num_reqs,
                                         int64_t num_heads, int64_t head_dim, int dtype, int64_t q_stride,
                                         int64_t out_stride, int64_t cache_stride_n, float scale,
-                                        const int32_t* suffix_slots, const int64_t* suffix_offsets,
-                                        int64_t suffix_table_stride, int64_t suffix_slots_count,
-                                        const int32_t* suffix_lens,
-                                        int64_t max_suffix_len, int64_t chunk_tokens, void* workspace,
+                                        const int32_t* prefix_slots, int64_t prefix_len, void* workspace,
                                         size_t workspace_bytes, void* stream) {
+  if (num_reqs > 0 && (!prev_m || !prev_l)) return PH_ERR_ARG;
+  return prefix_phase(out, prev_m, prev_l, nullptr, nullptr, q, k_cache, v_cache, num_reqs, num_heads, head_dim,
+                      dtype, q_stride, out_stride, cache_stride_n, scale, prefix_slots, prefix_len, workspace,
+                      workspace_bytes, stream);
+}
+
+// Suffix phase, merged with an optional partial already in out / prev_m / prev_l; the merged m / l are exported
+// when asked for.
+static int suffix_phase(void* out, const float* prev_m, const float* prev_l, float* m_out, float* l_out, const void* q,
+                        const void* k_cache, const void* v_cache, int64_t num_reqs, int64_t num_heads,
+                        int64_t head_dim, int dtype, int64_t q_stride, int64_t out_stride, int64_t cache_stride_n,
+                        float scale, const int32_t* suffix_slots, const int64_t* suffix_offsets,
+                        int64_t suffix_table_stride, int64_t suffix_slots_count, const int32_t* suffix_lens,
+                        int64_t max_suffix_len, int64_t chunk_tokens, void* workspace, size_t workspace_bytes,
+                        void* stream) {
   const int B = (int)num_reqs, H = (int)num_heads, D = (int)head_dim;
   int rc = check_common(out, q, k_cache, v_cache, num_reqs, num_heads, head_dim, dtype, q_stride, out_stride,
                         cache_stride_n);
   if (rc != PH_OK || num_reqs == 0) return rc;
-  if (max_suffix_len < 0 || !prev_m || !prev_l) return PH_ERR_ARG;
+  if (max_suffix_len < 0) return PH_ERR_ARG;
   const bool has_suffix = max_suffix_len > 0;
   if (has_suffix && (!suffix_slots || !suffix_lens || suffix_slots_count <= 0)) return PH_ERR_ARG;
   const DecodePlan p = plan_decode(num_reqs, num_heads, 0, 0, max_suffix_len, chunk_tokens, 0, head_dim);
@@ -519,7 +546,39 @@ extern "C" int ph_suffix_post_attention(void* out, const float* prev_m, const fl
   ma.item_base = 0;
   ma.prev_m = prev_m;
   ma.prev_l = prev_l;
+  ma.m_out = m_out;
+  ma.l_out = l_out;
   return launch_merge(ma, dtype, D, st);
+}
+
+extern "C" int ph_suffix_post_attention(void* out, const float* prev_m, const float* prev_l, const void* q,
+                                        const void* k_cache, const void* v_cache, int64_t num_reqs,
+                                        int64_t num_heads, int64_t head_dim, int dtype, int64_t q_stride,
+                                        int64_t out_stride, int64_t cache_stride_n, float scale,
+                                        const int32_t* suffix_slots, const int64_t* suffix_offsets,
+                                        int64_t suffix_table_stride, int64_t suffix_slots_count,
+                                        const int32_t* suffix_lens,
+                                        int64_t max_suffix_len, int64_t chunk_tokens, void* workspace,
+                                        size_t workspace_bytes, void* stream) {
+  if (num_reqs > 0 && (!prev_m || !prev_l)) return PH_ERR_ARG;
+  return suffix_phase(out, prev_m, prev_l, nullptr, nullptr, q, k_cache, v_cache, num_reqs, num_heads, head_dim,
+                      dtype, q_stride, out_stride, cache_stride_n, scale, suffix_slots, suffix_offsets,
+                      suffix_table_stride, suffix_slots_count, suffix_lens, max_suffix_len, chunk_tokens, workspace,
+                      workspace_bytes, stream);
+}
+
+extern "C" int ph_suffix_prev_attention(void* out, float* m_out, float* l_out, const void* q, const void* k_cache,
+                                        const void* v_cache, int64_t num_reqs, int64_t num_heads, int64_t head_dim,
+                                        int dtype, int64_t q_stride, int64_t out_stride, int64_t cache_stride_n,
+                                        float scale, const int32_t* suffix_slots, const int64_t* suffix_offsets,
+                                        int64_t suffix_table_stride, int64_t suffix_slots_count,
+                                        const int32_t* suffix_lens, int64_t max_suffix_len, int64_t chunk_tokens,
+                                        void* workspace, size_t workspace_bytes, void* stream) {
+  if (num_reqs > 0 && (!m_out || !l_out)) return PH_ERR_ARG;
+  return suffix_phase(out, nullptr, nullptr, m_out, l_out, q, k_cache, v_cache, num_reqs, num_heads, head_dim, dtype,
+                      q_stride, out_stride, cache_stride_n, scale, suffix_slots, suffix_offsets, suffix_table_stride,
+                      suffix_slots_count, suffix_lens, max_suffix_len, chunk_tokens, workspace, workspace_bytes,
+                      stream);
 }
 
 extern "C" size_t ph_prefill_workspace_bytes(int64_t num_tokens, int64_t num_heads, int64_t head_dim,

@@ -288,6 +288,29 @@ def test_prefix_and_post_entry_points(dev, dtype, B, P, H):
     torch.cuda.synchronize()
     ref = ref_decode_attention(case.q, case.k_rows, case.v_rows, case.full_lists())
     torch.testing.assert_close(out.cpu().float(), ref.float(), **TOL[dtype])
+    # the other order (shared_flash_decoding.py:332-376): suffix phase first with its (m, l) exported, then the
+    # prefix phase merged on top
+    out2 = torch.zeros_like(q)
+    m2 = torch.empty_like(m)
+    l2 = torch.empty_like(l)
+    rc = lib.ph_suffix_prev_attention(out2.data_ptr(), m2.data_ptr(), l2.data_ptr(), q.data_ptr(), kc.data_ptr(),
+                                      vc.data_ptr(), B, H, D, code, q.stride(0), out2.stride(0), kc.stride(0), scale,
+                                      table.data_ptr(), None, table.stride(0), table.numel(), lens.data_ptr(),
+                                      width, 0, ws.data_ptr(), nbytes, st)
+    assert rc == 0
+    torch.cuda.synchronize()
+    so_ref, sm_ref, sl_ref = ref_partial(case.q, case.k_rows, case.v_rows, case.suffix_lists, scale)
+    has = torch.tensor([len(x) > 0 for x in suffix])
+    torch.testing.assert_close(out2.cpu().float()[has], so_ref.float()[has], **TOL[dtype])
+    torch.testing.assert_close(m2.cpu()[has], sm_ref[has], atol=1e-3, rtol=1e-4)
+    torch.testing.assert_close(l2.cpu()[has], sl_ref[has], atol=1e-3, rtol=2e-2 if dtype == torch.bfloat16 else 5e-3)
+    assert (l2.cpu()[~has] == 0).all()  # no suffix: an empty partial
+    rc = lib.ph_prefix_post_attention(out2.data_ptr(), m2.data_ptr(), l2.data_ptr(), q.data_ptr(), kc.data_ptr(),
+                                      vc.data_ptr(), B, H, D, code, q.stride(0), out2.stride(0), kc.stride(0), scale,
+                                      pslots.data_ptr(), P, ws.data_ptr(), nbytes, st)
+    assert rc == 0
+    torch.cuda.synchronize()
+    torch.testing.assert_close(out2.cpu().float(), ref.float(), **TOL[dtype])
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
