@@ -351,6 +351,7 @@ def config5_layer(torch, dev):
     st.num_generation_jobs = B
     st.slot_mapping = case.new_slots.to(torch.int32).to(dev)
     st.fill_tables = None
+    st.fill_decode_tables = None
     st.decode_perm = None
     st.decode_tables = kernels.DecodeTables.build(dec.pool_lists(dec.prefix_lists), dec.group_req_cu,
                                                   dec.pool_lists(dec.suffix_lists), dev, num_heads=H, head_dim=D)

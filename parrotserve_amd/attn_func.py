@@ -141,6 +141,49 @@ def build_iteration_tables(jobs: Sequence[Any], grouping: str = "lca") -> Iterat
     return t
 
 
+def forked_fill_tables(jobs: Sequence[Any], min_parent_len: int, max_own_len: int):
+    """Fill jobs forked from common parents, as a shared-prefix *decode* problem: every new token is a request,
+    the parent's whole context is the prefix its group shares, and its suffix is its own context up to itself
+    (the causal part).  The parent's K/V is then read once per group of up to 256 new tokens instead of once per
+    chunk, which is what the prefix phase exists for.  Worth it for short chunks over long shared parents (the
+    forked prompts of the reference's experiments: tens of tokens over thousands); returns None otherwise, i.e.
+    unless every Fill of the iteration has a parent of at least ``min_parent_len`` tokens that it shares with a
+    neighbouring Fill, and an own context of at most ``max_own_len`` tokens.
+    Returns (prefix slot lists, token offsets of the groups, per-token suffix slot lists)."""
+    fills = [j for j in jobs if isinstance(j, Fill)]
+    if len(fills) < 2:
+        return None
+    prefix_lists: List[List[int]] = []
+    gcu = [0]
+    suffix_lists: List[List[int]] = []
+    last_parent = None
+    members = 0
+    for job in fills:
+        parent = job.context.parent_context
+        plen = parent.get_context_len() if parent is not None else 0
+        slots = job.context.get_context_slot_ids()
+        own = slots[plen:]
+        n = len(job.token_ids)
+        if parent is None or plen < min_parent_len or len(own) > max_own_len:
+            return None
+        if parent is not last_parent:
+            if last_parent is not None:
+                if members < 2:
+                    return None
+                gcu.append(len(suffix_lists))
+            prefix_lists.append(slots[:plen])
+            last_parent = parent
+            members = 0
+        members += 1
+        first = len(own) - n
+        for r in range(n):
+            suffix_lists.append(own[: first + r + 1])
+    if members < 2:
+        return None
+    gcu.append(len(suffix_lists))
+    return prefix_lists, gcu, suffix_lists
+
+
 # --------------------------------------------------------------------------- #
 # the plug-in
 # --------------------------------------------------------------------------- #
@@ -166,6 +209,10 @@ class HipSharedPrefixAttn(AttnFunc):
     # device tables of the last decode-only batch, patched in place while the same batch keeps generating
     table_cache = DecodeTableCache()
     incremental = True
+    # Fill jobs forked from a shared parent run as a shared-prefix decode over their new tokens when the parent is
+    # at least this long and every chunk's own context at most that long (see forked_fill_tables); 0 switches it off
+    forked_fill_min_parent = 256
+    forked_fill_max_own = 64
 
     @classmethod
     def init_iteration_state(cls, iteration_state, builtin_config, jobs, num_heads: int, head_size: int):
@@ -178,6 +225,7 @@ class HipSharedPrefixAttn(AttnFunc):
             st.flash_context_len = cached.flash_context_len
             st.slot_mapping = cached.slot_mapping
             st.fill_tables = None
+            st.fill_decode_tables = None
             st.decode_tables = cached.tables
             st.decode_perm = cached.decode_perm
             return
@@ -189,8 +237,16 @@ class HipSharedPrefixAttn(AttnFunc):
         st.flash_context_len = tabs.flash_context_len
         st.slot_mapping = torch.from_numpy(np.asarray(tabs.slot_mapping, dtype=np.int32)).to(device)
         st.fill_tables = None
+        st.fill_decode_tables = None
         if tabs.fill_q_lens:
-            st.fill_tables = kernels.PrefillTables.build(tabs.fill_q_lens, tabs.fill_slot_lists, device)
+            forked = None
+            if cls.forked_fill_min_parent > 0 and head_size == 128:
+                forked = forked_fill_tables(jobs, cls.forked_fill_min_parent, cls.forked_fill_max_own)
+            if forked is not None:
+                st.fill_decode_tables = kernels.DecodeTables.build(*forked, device, num_heads=num_heads,
+                                                                   head_dim=head_size)
+            else:
+                st.fill_tables = kernels.PrefillTables.build(tabs.fill_q_lens, tabs.fill_slot_lists, device)
         st.decode_tables = None
         st.decode_perm = None
         if tabs.num_generates:
@@ -230,7 +286,10 @@ class HipSharedPrefixAttn(AttnFunc):
             q = q.contiguous()
         output = torch.empty((T, self.num_heads, self.head_dim), dtype=q.dtype, device=q.device)
         nf = st.num_total_fill_tokens
-        if nf > 0:
+        if nf > 0 and st.fill_decode_tables is not None:  # forked Fills: the parent is a shared prefix of their tokens
+            kernels.decode_attention(q[:nf], k_cache, v_cache, st.fill_decode_tables, scale=self.scaling,
+                                     out=output[:nf])
+        elif nf > 0:
             kernels.prefill_attention(q[:nf], k_cache, v_cache, st.fill_tables, scale=self.scaling, out=output[:nf])
         if st.num_generation_jobs > 0:
             q_gen = q[nf:]

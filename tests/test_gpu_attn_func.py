@@ -299,3 +299,84 @@ def test_device_suffix_plan_equals_the_host_plan(dev, seed):
         assert torch.equal(rec[:eff, 1], torch.from_numpy(h_lane_cu[1:] - h_lane_cu[:-1]))
         assert torch.equal(rec[:eff, 2:5], torch.from_numpy(h_items[h_lane_cu[:-1], 0:3]))
     assert (rec[eff:, 1] == 0).all()  # lanes beyond the cut count own nothing
+
+
+@pytest.mark.parametrize("name", ["xformers_fill_shared_prompts_generate", "hip_shared_prefix"])
+@pytest.mark.parametrize("n_parents,chunks,own_prev", [(1, 9, 0), (3, 4, 0), (2, 70, 5)])
+def test_forked_fills_run_as_shared_prefix_decode(dev, name, n_parents, chunks, own_prev):
+    """Fill jobs forked from shared parents (short chunks over long parents): the plug-in hands their new tokens to
+    the shared-prefix decode path; results against the oracle's prefill with parent context, for one and several
+    parents, for more than 256 new tokens under one parent (two query tiles), for chunks that continue an own
+    context, and mixed with Generate jobs in the same iteration."""
+    from parrotserve_amd import mem
+    from parrotserve_amd.attn_func import BuiltinConfig
+    from parrotserve_amd.context import BlockContext, RecyclePool
+    from parrotserve_amd.iter_state import IterationState
+    from parrotserve_amd.primitive_job import Fill, Generate
+
+    H, D, slots = 4, 128, 8192
+    pool = RecyclePool(pool_size=slots)
+    g = torch.Generator().manual_seed(70 + chunks)
+    fills, gens, cid = [], [], 0
+    for pi in range(n_parents):
+        parent = BlockContext(cid, None, pool, 1)
+        cid += 1
+        parent.allocate(300 + 41 * pi)
+        for c in range(chunks):
+            child = BlockContext(cid, parent, pool, 1)
+            cid += 1
+            n = int(torch.randint(1, 12, (1,), generator=g))
+            child.allocate(own_prev + n)  # an own context of own_prev older tokens, then the chunk
+            job = Fill(0, cid, child.context_id, parent.context_id, token_ids=list(range(n)))
+            job.context = child
+            fills.append(job)
+        child = BlockContext(cid, parent, pool, 1)
+        cid += 1
+        child.allocate(7)
+        job = Generate(0, cid, child.context_id, parent.context_id, sampling_config=None)
+        job.context = child
+        gens.append(job)
+    jobs = fills + gens
+    cfg = BuiltinConfig(num_kv_cache_blocks=slots, attn_func=name, dtype=torch.float16, device=dev)
+    cfg.attn_func.table_cache.clear()
+    store = mem.init_model_cache_storage(1, slots, H, D, torch.float16, dev)
+    kc_cpu = torch.randn(slots, H, D, generator=g).half()
+    vc_cpu = torch.randn(slots, H, D, generator=g).half()
+    store.k_cache[0].copy_(kc_cpu)
+    store.v_cache[0].copy_(vc_cpu)
+    st = IterationState(jobs, _Cfg(H, H * D), cfg)
+    assert st.fill_decode_tables is not None and st.fill_tables is None  # the forked form was chosen
+    n_new = [len(j.token_ids) if isinstance(j, Fill) else 1 for j in jobs]
+    T = sum(n_new)
+    qkv = torch.randn(T, 3 * H * D, generator=g).half()
+    q, k, v = (t.view(T, H, D) for t in qkv.chunk(3, dim=-1))
+    kc_ref, vc_ref = kc_cpu.clone(), vc_cpu.clone()
+    pos = 0
+    for j, n in zip(jobs, n_new):
+        sl = torch.tensor(j.context.get_context_slot_ids())
+        kc_ref[sl[-n:]] = k[pos:pos + n]
+        vc_ref[sl[-n:]] = v[pos:pos + n]
+        pos += n
+    ref = torch.zeros(T, H, D, dtype=torch.float16)
+    pos = 0
+    for j, n in zip(jobs, n_new):
+        sl = torch.tensor(j.context.get_context_slot_ids())
+        if isinstance(j, Fill):
+            ref[pos:pos + n] = ref_prefill_with_parent(q[pos:pos + n], kc_ref, vc_ref, [n], [sl])
+        else:
+            ref[pos:pos + 1] = ref_decode_attention(q[pos:pos + 1], kc_ref, vc_ref, [sl])
+        pos += n
+    attn = cfg.attn_func(layer_idx=0, scaling=D ** -0.5, num_heads=H, head_dim=D)
+    q_d, k_d, v_d = (t.view(T, H, D) for t in qkv.to(dev).chunk(3, dim=-1))
+    out = attn(q_d, k_d, v_d, st)
+    torch.testing.assert_close(out.cpu().view(T, H, D).float(), ref.float(), **TOL)
+    # the same iteration with the forked form switched off takes the prefill kernel and agrees
+    class Plain(cfg.attn_func):
+        forked_fill_min_parent = 0
+    cfg2 = BuiltinConfig(num_kv_cache_blocks=slots, attn_func=Plain, dtype=torch.float16, device=dev)
+    st2 = IterationState(jobs, _Cfg(H, H * D), cfg2)
+    assert st2.fill_decode_tables is None and st2.fill_tables is not None
+    out2 = Plain(layer_idx=0, scaling=D ** -0.5, num_heads=H, head_dim=D)(q_d, k_d, v_d, st2)
+    torch.testing.assert_close(out2.cpu().view(T, H, D).float(), ref.float(), **TOL)
+    cfg.attn_func.table_cache.clear()
+    mem.Model_Cache = None

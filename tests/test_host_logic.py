@@ -279,3 +279,38 @@ def test_table_cache_host_side_hits_only_on_the_same_batch_one_token_later():
     assert cache.advance_host([g] + jobs[1:]) is None and unchanged()
     # and the unchanged batch still qualifies
     assert cache.advance_host(jobs) == [j.context.token_kv_block_ids[-1] for j in jobs]
+
+
+def test_forked_fill_tables_grouping_rules():
+    """Forked Fills as a shared-prefix decode problem: groups by neighbouring common parent, per-token suffix lists
+    = the own context up to the token; refused for lone chunks, short parents, long own contexts, parentless Fills."""
+    from parrotserve_amd.attn_func import forked_fill_tables
+    from parrotserve_amd.context import BlockContext, RecyclePool
+    from parrotserve_amd.primitive_job import Fill, Generate
+
+    pool = RecyclePool(pool_size=4096)
+
+    def fork(parent, own_prev, n, cid):
+        c = BlockContext(cid, parent, pool, 1)
+        c.allocate(own_prev + n)
+        j = Fill(0, cid, cid, parent.context_id if parent is not None else -1, token_ids=list(range(n)))
+        j.context = c
+        return j
+
+    pa = BlockContext(100, None, pool, 1)
+    pa.allocate(50)
+    pb = BlockContext(101, None, pool, 1)
+    pb.allocate(40)
+    jobs = [fork(pa, 0, 3, 1), fork(pa, 2, 2, 2), fork(pb, 0, 1, 3), fork(pb, 0, 4, 4)]
+    prefix, gcu, suffix = forked_fill_tables(jobs, 32, 16)
+    assert prefix == [pa.get_context_slot_ids(), pb.get_context_slot_ids()] and gcu == [0, 5, 10]
+    own1 = jobs[1].context.token_kv_block_ids
+    assert suffix[0] == jobs[0].context.token_kv_block_ids[:1] and suffix[2] == jobs[0].context.token_kv_block_ids[:3]
+    assert suffix[3] == own1[:3] and suffix[4] == own1[:4]  # two older own tokens are visible to the chunk's first token
+    assert [len(x) for x in suffix[5:]] == [1, 1, 2, 3, 4]
+    assert forked_fill_tables(jobs, 45, 16) is None            # parent b is shorter than 45
+    assert forked_fill_tables(jobs, 32, 3) is None             # an own context of 4 tokens
+    assert forked_fill_tables(jobs[:3], 32, 16) is None        # the last parent has a single chunk
+    assert forked_fill_tables([jobs[0], jobs[2], jobs[1], jobs[3]], 32, 16) is None  # same parent, not neighbours
+    assert forked_fill_tables([jobs[0]], 32, 16) is None
+    assert forked_fill_tables([fork(None, 0, 5, 7), fork(None, 0, 5, 8)], 0, 16) is None  # no parent
