@@ -97,27 +97,35 @@ def build_iteration_tables(jobs: Sequence[Any], grouping: str = "lca") -> Iterat
     several prompt groups can share the iteration."""
     assert grouping in ("lca", "parent")
     P = get_shared_context_len(jobs) if grouping == "lca" else 0
-    slots0 = jobs[0].context.get_context_slot_ids()
+    slots0 = jobs[0].context.get_context_slot_ids() if P > 0 else []
     t = IterationTables(P, slots0[:P], [], [], [], [], [], [], [], [], [], 0)
-    gen_full: List[List[int]] = []
+    gen_full: List[List[int]] = []    # "lca": every Generate job's whole context
+    gen_own: List[List[int]] = []     # "parent": only what lies beyond the fork parent (the job's own tokens)
     gen_parent: List[Any] = []
     for job in jobs:
-        slots = job.context.get_context_slot_ids()
         if isinstance(job, Fill):
+            slots = job.context.get_context_slot_ids()
             n = len(job.token_ids)
             t.num_fill_tokens.append(n)
             t.fill_q_lens.append(n)
             t.fill_kv_lens.append(len(slots))
             t.fill_slots.extend(slots)
             t.fill_slot_lists.append(slots)
+            t.slot_mapping.extend(slots[-n:])
         elif isinstance(job, Generate):
-            n = 1
             t.num_generates += 1
-            gen_full.append(slots)
-            gen_parent.append(job.context.parent_context)
+            if grouping == "lca":
+                slots = job.context.get_context_slot_ids()
+                gen_full.append(slots)
+                t.slot_mapping.append(slots[-1])
+            else:
+                # the parent's list is taken once per group below, not copied into every job's list
+                own = list(job.context.token_kv_block_ids)
+                gen_own.append(own)
+                gen_parent.append(job.context.parent_context)
+                t.slot_mapping.append(own[-1])
         else:
             raise TypeError(f"unknown job type {type(job)}")
-        t.slot_mapping.extend(slots[-n:])
     if grouping == "lca":
         for slots in gen_full:
             t.paged_block_tables.append(slots[P:])
@@ -126,16 +134,18 @@ def build_iteration_tables(jobs: Sequence[Any], grouping: str = "lca") -> Iterat
             t.groups.append((t.flash_block_table, list(range(len(gen_full)))))
     else:
         by_parent: Dict[int, int] = {}
-        for i, (slots, parent) in enumerate(zip(gen_full, gen_parent)):
-            plen = parent.get_context_len() if parent is not None else 0
-            t.paged_block_tables.append(slots[plen:])
-            t.paged_context_lens.append(len(slots) - plen)
-            if plen == 0:
+        for i, (own, parent) in enumerate(zip(gen_own, gen_parent)):
+            t.paged_block_tables.append(own)
+            t.paged_context_lens.append(len(own))
+            if parent is None:
                 continue
             g = by_parent.get(id(parent))
             if g is None:
+                prefix = parent.get_context_slot_ids()
+                if not prefix:
+                    continue
                 by_parent[id(parent)] = len(t.groups)
-                t.groups.append((slots[:plen], [i]))
+                t.groups.append((prefix, [i]))
             else:
                 t.groups[g][1].append(i)
     return t
