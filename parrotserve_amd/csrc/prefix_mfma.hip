@@ -516,12 +516,16 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
   // other query tiles of the chunk and should stay in L2
   constexpr bool NTLOAD = !CAUSAL;
   // Decode: the LDS ring holds one step beyond the one being multiplied, which is too little to cover the
-  // memory latency (the ring cannot grow: it is all of LDS).  So every thread also touches one 128-byte line
-  // of the step after that (128 tokens x K and V x 2 lines = 512 lines) with a 4-byte load: the step's rows
-  // are then on their way to L2 a whole step before the ring has room for them, and the row loads that
-  // follow find them there.  Issued behind the step's row loads, so their completion is still counted
-  // exactly (one younger load per step).
+  // memory latency (the ring cannot grow: it is all of LDS).  When the workgroup's share is at most two steps
+  // longer than the ring, every thread also touches one 128-byte line of the step after the one being staged
+  // (128 tokens x K and V x 2 lines = 512 lines) with a 4-byte load during the first two steps: the rows of
+  // the steps beyond the ring are then on their way to L2 a whole step before the ring has room for them, and
+  // the row loads that follow find them there.  Issued behind the step's row loads, so their completion is
+  // still counted exactly (one younger load per step).  Longer shares run in a bandwidth-bound steady state
+  // where the extra requests cost more than the earlier start gains (measured on cold K/V: 2 % slower with
+  // them at 11 steps per workgroup, 1 % faster at 4), so they go without.
   constexpr bool PREFETCH = !CAUSAL && A == 1 && STEP * TQ == 128;
+  constexpr int kPfSteps = 2;
   constexpr float kSlack = 8.f;
   float16_t oacc[4];
   float m = -INFINITY, lsum = 0.f, mtrue = -INFINITY;
@@ -557,6 +561,7 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
                    : reinterpret_cast<const char*>(kc + (int64_t)head * kPD + ((c ^ ((4 * (r0 + i) + tl) & 15)) * 8));
   const uint32_t dst0 = lds_addr_of(gl) + sub0 * kStage + (isv ? kVtOff : 0) + r0 * 1024;
   const uint32_t pf_lds = lds_addr_of(smem + kPfOff) + w8 * 256;
+  const int pf_steps = (PREFETCH && (s1 - s0 + STEP * TQ - 1) / (STEP * TQ) <= NST + kPfSteps) ? kPfSteps : 0;
   // rows of the group's tile that starts at token tb, into ring stage `stage`
   auto fetch_rows = [&](int tb, int stage) {
     uint32_t sl[LPT];
@@ -628,7 +633,13 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
     // Tile `it` of this group has landed once at most the (A - 1) LPT loads issued after it are outstanding
     // (near the end fewer were issued, so everything is awaited); the barrier publishes all parts of the
     // tile and tells everyone that the stage read in the previous step is free again.
-    if (it + A - 1 < my_iters) wait_vmcnt<(A - 1) * LPT + (PREFETCH ? 1 : 0)>(); else wait_vmcnt<0>();
+    if (it + A - 1 >= my_iters) {
+      wait_vmcnt<0>();
+    } else if (PREFETCH && pf_steps > 0 && it >= 1 && it <= pf_steps) {
+      wait_vmcnt<(A - 1) * LPT + 1>();  // the line touches issued behind the last row loads may still be out
+    } else {
+      wait_vmcnt<(A - 1) * LPT>();
+    }
     __syncthreads();
     {
       const int front = s0 + STEP * TQ * (it + A);           // first token of the step being staged
@@ -638,7 +649,7 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
         __syncthreads();
       }
       if (it > 0 && it + A < my_iters) fetch_rows(front + STEP * g, (stage + A) % NST);
-      if constexpr (PREFETCH) {
+      if (PREFETCH && it < pf_steps) {
         // token (of all four groups) and line of the step after `front`, clamped into the list and the window
         const int pt = min(min(front + STEP * TQ + (int)(threadIdx.x >> 2), s1 - 1), win0 + kWin - 1);
         const uint32_t slot = (uint32_t)win[pt - win0];
