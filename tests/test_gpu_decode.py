@@ -61,6 +61,30 @@ def test_config2_full_size(dev):
     _check(case, dev)
 
 
+def test_config5_full_size_attention(dev):
+    """Config 5's attention at full size (4 groups x 32 branches, prefix 6000, suffix U[32,1024], 40x128, seed 4):
+    the grouped shared-prefix path equals the non-shared ragged path over every request's whole context (two
+    independent kernel paths on the GPU), and eight sampled requests equal the oracle."""
+    from parrotserve_amd import kernels, synth
+
+    gen = torch.Generator().manual_seed(4)
+    s = torch.randint(32, 1025, (128,), generator=gen).tolist()  # the draw of synth.config5
+    case = synth.make_decode_case("C5", 4, torch.float16, 4, 32, 6000, s, 40, 128, 1 << 18)
+    kc, vc = synth.pool_to_device(case.k_rows, case.v_rows, case.used_slots, case.pool_slots, dev)
+    q = case.q.to(dev)
+    shared = kernels.DecodeTables.build(case.pool_lists(case.prefix_lists), case.group_req_cu,
+                                        case.pool_lists(case.suffix_lists), dev, num_heads=40, head_dim=128)
+    out = kernels.decode_attention(q, kc, vc, shared)
+    full = case.full_lists()
+    plain = kernels.DecodeTables.build([], [], [case.used_slots[l].tolist() for l in full], dev, num_heads=40,
+                                       head_dim=128)
+    out_plain = kernels.decode_attention(q, kc, vc, plain)
+    torch.testing.assert_close(out.float(), out_plain.float(), **TOL[torch.float16])
+    pick = [0, 31, 32, 50, 64, 95, 100, 127]
+    ref = ref_decode_attention(case.q[pick], case.k_rows, case.v_rows, [full[i] for i in pick])
+    torch.testing.assert_close(out[pick].cpu().float(), ref.float(), **TOL[torch.float16])
+
+
 def test_multi_group_prefixes(dev):
     """Config-5 style: several prefix groups in one batch (scaled down)."""
     from parrotserve_amd import synth
