@@ -154,6 +154,37 @@ def test_config3_ragged_decode_scaled(dev):
     _check(case, dev)
 
 
+def test_config3_full_size_properties(dev):
+    """Config 3 at full size (B 256, ctx log-uniform[128,8192], 32x128, 4M-slot pool of device-generated rows):
+    the balanced form and the plain grid form agree, a value cache of ones gives ones (softmax weights sum to one
+    over every ragged list), and the four shortest requests equal the oracle on their own rows."""
+    from parrotserve_amd import kernels, synth
+
+    pool = 1 << 22
+    case = synth.config3(batch=256, pool_slots=pool)
+    lists = case.pool_lists(case.suffix_lists)
+    assert len(lists) == 256 and sum(len(l) for l in lists) > 300000
+    gen = torch.Generator(device=dev).manual_seed(3)
+    kc = torch.randn((pool, 32, 128), generator=gen, device=dev, dtype=torch.float16)
+    vc = torch.randn((pool, 32, 128), generator=gen, device=dev, dtype=torch.float16)
+    q = case.q.to(dev)
+    balanced = kernels.DecodeTables.build([], [], lists, dev)
+    grid = kernels.DecodeTables.build([], [], lists, dev, balanced=False)
+    out = kernels.decode_attention(q, kc, vc, balanced)
+    out_grid = kernels.decode_attention(q, kc, vc, grid)
+    torch.testing.assert_close(out.float(), out_grid.float(), **TOL[torch.float16])
+    short = sorted(range(256), key=lambda i: len(lists[i]))[:4]
+    for i in short:
+        rows = torch.tensor(lists[i], device=dev)
+        ref = ref_decode_attention(case.q[i:i + 1], kc[rows].cpu(), vc[rows].cpu(), [torch.arange(len(lists[i]))])
+        torch.testing.assert_close(out[i:i + 1].cpu().float(), ref.float(), **TOL[torch.float16])
+    vc.fill_(1.0)
+    ones = kernels.decode_attention(q, kc, vc, balanced)
+    torch.testing.assert_close(ones.float(), torch.ones_like(ones).float(), atol=2e-3, rtol=0)
+    del kc, vc
+    torch.cuda.empty_cache()  # 69 GB of pool rows
+
+
 def test_reference_named_entry_points(dev):
     """flash_paged_attention / paged_flash_attention / vllm_paged_attention with the
     reference's argument lists (padded 2-D tables, int32 lens)."""
