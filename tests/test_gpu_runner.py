@@ -31,13 +31,16 @@ def _set_weights(model, seed):
     return w
 
 
-@pytest.mark.parametrize("attn_func,fused", [("xformers_fill_shared_prompts_generate", False),
-                                             ("hip_shared_prefix", False), ("hip_shared_prefix", True)])
-def test_shared_prompt_generation_loop_matches_flat_oracle(dev, attn_func, fused):
+@pytest.mark.parametrize("attn_func,fused,forked", [("xformers_fill_shared_prompts_generate", False, False),
+                                                    ("hip_shared_prefix", False, False),
+                                                    ("hip_shared_prefix", True, False),
+                                                    ("hip_shared_prefix", True, True)])
+def test_shared_prompt_generation_loop_matches_flat_oracle(dev, attn_func, fused, forked, monkeypatch):
     """The scenario of the reference's decode benchmark (benchmark/bench_kernel.py:11-66), small: one shared
     Fill, B forked Fills, then Generate iterations on the forked contexts.  Every hidden state handed to the
     sampler must equal the oracle's hidden state of the same token in the branch's flat sequence, and every
-    sampled token the oracle's arg-max wherever its margin is clear of fp16 noise."""
+    sampled token the oracle's arg-max wherever its margin is clear of fp16 noise.  ``forked``: the B forked Fills run
+    as a shared-prefix decode over their new tokens instead of through the prefill kernel."""
     from parrotserve_amd.attn_func import BuiltinConfig
     from parrotserve_amd.primitive_job import Fill, Generate
     from parrotserve_amd.runner import BuiltinRunner, LlamaConfig, SamplingConfig
@@ -47,6 +50,8 @@ def test_shared_prompt_generation_loop_matches_flat_oracle(dev, attn_func, fused
     mc = LlamaConfig(vocab_size=V, hidden_size=N, intermediate_size=Fdim, num_hidden_layers=L, num_attention_heads=H,
                      rms_norm_eps=1e-6, max_position_embeddings=256, fused_ops=fused)
     cfg = BuiltinConfig(num_kv_cache_blocks=2048, attn_func=attn_func, dtype=torch.float16, device=dev)
+    if forked:  # the forked Fills of this scenario (5-7 tokens over the 40-token parent) take the shared-prefix path
+        monkeypatch.setattr(cfg.attn_func, "forked_fill_min_parent", 16)
     cfg.attn_func.table_cache.clear()
     hits0 = cfg.attn_func.table_cache.hits
     runner = BuiltinRunner(mc, cfg, dummy_weights=False)
