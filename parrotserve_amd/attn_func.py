@@ -151,14 +151,17 @@ def build_iteration_tables(jobs: Sequence[Any], grouping: str = "lca") -> Iterat
     return t
 
 
-def forked_fill_tables(jobs: Sequence[Any], min_parent_len: int, max_own_len: int):
+def forked_fill_tables(jobs: Sequence[Any], min_parent_len: int, max_own_len: int, pay_ratio: int = 4):
     """Fill jobs forked from common parents, as a shared-prefix *decode* problem: every new token is a request,
     the parent's whole context is the prefix its group shares, and its suffix is its own context up to itself
     (the causal part).  The parent's K/V is then read once per group of up to 256 new tokens instead of once per
     chunk, which is what the prefix phase exists for.  Worth it for short chunks over long shared parents (the
     forked prompts of the reference's experiments: tens of tokens over thousands); returns None otherwise, i.e.
     unless every Fill of the iteration has a parent of at least ``min_parent_len`` tokens that it shares with a
-    neighbouring Fill, and an own context of at most ``max_own_len`` tokens.
+    neighbouring Fill, and an own context of at most ``max_own_len`` tokens -- and unless it pays: the suffix phase
+    reads a token's own context once per *token* (no reuse across the chunk's queries), so the (query, own key)
+    pairs it adds must stay well under the parent rows it saves (``1 / pay_ratio`` of them: chunks of about
+    sqrt(P / 2) tokens over a P-token parent at the most).
     Returns (prefix slot lists, token offsets of the groups, per-token suffix slot lists)."""
     fills = [j for j in jobs if isinstance(j, Fill)]
     if len(fills) < 2:
@@ -168,6 +171,8 @@ def forked_fill_tables(jobs: Sequence[Any], min_parent_len: int, max_own_len: in
     suffix_lists: List[List[int]] = []
     last_parent = None
     members = 0
+    own_pairs = 0      # (query, own key) pairs the suffix phase would read
+    parent_rows = 0    # parent rows read chunk by chunk
     for job in fills:
         parent = job.context.parent_context
         plen = parent.get_context_len() if parent is not None else 0
@@ -188,9 +193,15 @@ def forked_fill_tables(jobs: Sequence[Any], min_parent_len: int, max_own_len: in
         first = len(own) - n
         for r in range(n):
             suffix_lists.append(own[: first + r + 1])
+        own_pairs += n * first + n * (n + 1) // 2
+        parent_rows += plen
     if members < 2:
         return None
     gcu.append(len(suffix_lists))
+    # parent rows read as a shared prefix: once per 256 new tokens of a group
+    shared_rows = sum(len(p) * ((gcu[g + 1] - gcu[g] + 255) // 256) for g, p in enumerate(prefix_lists))
+    if pay_ratio * own_pairs > parent_rows - shared_rows:
+        return None
     return prefix_lists, gcu, suffix_lists
 
 
@@ -223,6 +234,7 @@ class HipSharedPrefixAttn(AttnFunc):
     # at least this long and every chunk's own context at most that long (see forked_fill_tables); 0 switches it off
     forked_fill_min_parent = 256
     forked_fill_max_own = 64
+    forked_fill_pay_ratio = 4
 
     @classmethod
     def init_iteration_state(cls, iteration_state, builtin_config, jobs, num_heads: int, head_size: int):
@@ -251,7 +263,8 @@ class HipSharedPrefixAttn(AttnFunc):
         if tabs.fill_q_lens:
             forked = None
             if cls.forked_fill_min_parent > 0 and head_size == 128:
-                forked = forked_fill_tables(jobs, cls.forked_fill_min_parent, cls.forked_fill_max_own)
+                forked = forked_fill_tables(jobs, cls.forked_fill_min_parent, cls.forked_fill_max_own,
+                                            cls.forked_fill_pay_ratio)
             if forked is not None:
                 st.fill_decode_tables = kernels.DecodeTables.build(*forked, device, num_heads=num_heads,
                                                                    head_dim=head_size)

@@ -52,6 +52,7 @@ def test_shared_prompt_generation_loop_matches_flat_oracle(dev, attn_func, fused
     cfg = BuiltinConfig(num_kv_cache_blocks=2048, attn_func=attn_func, dtype=torch.float16, device=dev)
     if forked:  # the forked Fills of this scenario (5-7 tokens over the 40-token parent) take the shared-prefix path
         monkeypatch.setattr(cfg.attn_func, "forked_fill_min_parent", 16)
+        monkeypatch.setattr(cfg.attn_func, "forked_fill_pay_ratio", 0)  # taken whatever it saves
     cfg.attn_func.table_cache.clear()
     hits0 = cfg.attn_func.table_cache.hits
     runner = BuiltinRunner(mc, cfg, dummy_weights=False)

@@ -298,9 +298,9 @@ def test_forked_fill_tables_grouping_rules():
         return j
 
     pa = BlockContext(100, None, pool, 1)
-    pa.allocate(50)
+    pa.allocate(80)
     pb = BlockContext(101, None, pool, 1)
-    pb.allocate(40)
+    pb.allocate(60)
     jobs = [fork(pa, 0, 3, 1), fork(pa, 2, 2, 2), fork(pb, 0, 1, 3), fork(pb, 0, 4, 4)]
     prefix, gcu, suffix = forked_fill_tables(jobs, 32, 16)
     assert prefix == [pa.get_context_slot_ids(), pb.get_context_slot_ids()] and gcu == [0, 5, 10]
@@ -308,9 +308,11 @@ def test_forked_fill_tables_grouping_rules():
     assert suffix[0] == jobs[0].context.token_kv_block_ids[:1] and suffix[2] == jobs[0].context.token_kv_block_ids[:3]
     assert suffix[3] == own1[:3] and suffix[4] == own1[:4]  # two older own tokens are visible to the chunk's first token
     assert [len(x) for x in suffix[5:]] == [1, 1, 2, 3, 4]
-    assert forked_fill_tables(jobs, 45, 16) is None            # parent b is shorter than 45
+    assert forked_fill_tables(jobs, 70, 16) is None            # parent b is shorter than 70
     assert forked_fill_tables(jobs, 32, 3) is None             # an own context of 4 tokens
     assert forked_fill_tables(jobs[:3], 32, 16) is None        # the last parent has a single chunk
     assert forked_fill_tables([jobs[0], jobs[2], jobs[1], jobs[3]], 32, 16) is None  # same parent, not neighbours
     assert forked_fill_tables([jobs[0]], 32, 16) is None
+    # it has to pay: two 12-token chunks read 2 x 78 own pairs for the 80 parent rows they save
+    assert forked_fill_tables([fork(pa, 0, 12, 20), fork(pa, 0, 12, 21)], 32, 16) is None
     assert forked_fill_tables([fork(None, 0, 5, 7), fork(None, 0, 5, 8)], 0, 16) is None  # no parent
