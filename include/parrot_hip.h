@@ -373,7 +373,7 @@ int ph_suffix_tables_append(int32_t* table, int64_t table_stride, int32_t* lens,
  * per iteration in place of host-side list work and an upload.  items must
  * hold num_lanes + num_reqs entries of 4 ints, lane_rec num_lanes entries of
  * 8, req_item_cu num_reqs + 1.  The stream is cut into
- * min(num_lanes, ceil(total / 16)) pieces; records of the remaining lanes are
+ * min(num_lanes, ceil(total / 4)) pieces; records of the remaining lanes are
  * empty.  num_reqs <= 8192; the lengths must sum to less than 2^31.  The
  * reference has no counterpart (its kernels take fixed-size blocks per
  * request, attention_post_kernels.cu:74-110). */

@@ -28,8 +28,13 @@ __global__ __launch_bounds__(256) void append_slots_kernel(int32_t* __restrict__
 //   - the first item of request b starts at cu[b];
 //   - mark l that falls strictly inside a request starts another item of that request;
 //   - lane l's record names the item that starts at cut(l) and counts the items up to cut(l + 1).
-// lanes = min(lanes_cap, ceil(total / 16), total): no piece under 16 tokens; records beyond `lanes` are empty.
+// lanes = min(lanes_cap, ceil(total / kMinPiece), total): no piece under kMinPiece tokens; records beyond `lanes`
+// are empty.
 constexpr int kPlanThreads = 1024;
+// Smallest piece: one round of the streaming body's register pipeline.  A short total is a latency problem, not a
+// bandwidth problem: spread over many lanes every wave walks the slot-id -> rows -> partial chain once, instead of
+// a few waves walking it several times in a row while the rest of the launch waits for them.
+constexpr int kMinPiece = 4;
 
 struct PlanScratch {
   int cu[kPlanMaxReqs + 1];      // token prefix sums
@@ -82,7 +87,7 @@ __global__ __launch_bounds__(kPlanThreads) void suffix_plan_kernel(const int32_t
   const int t = threadIdx.x;
   block_scan([&](int i) { return max(lens[i], 0); }, B, sh.cu, sh.part);
   const int64_t total = sh.cu[B];
-  const int lanes = (int)max((int64_t)1, min((int64_t)lanes_cap, min((total + 15) / 16, total)));
+  const int lanes = (int)max((int64_t)1, min((int64_t)lanes_cap, min((total + kMinPiece - 1) / kMinPiece, total)));
   auto cut = [&](int l) { return (int)((int64_t)l * total / lanes); };
   // first mark strictly inside request b (cut(l) > cu[b]), and one past the last (cut(l) < cu[b+1])
   auto mark_lo = [&](int b) { return (int)((((int64_t)sh.cu[b] + 1) * lanes + total - 1) / total); };

@@ -527,12 +527,13 @@ def suffix_lane_capacity(device, num_heads: int, head_dim: int) -> int:
 def suffix_lanes(device, num_heads: int, head_dim: int, total_tokens: int) -> int:
     """Pieces of the balanced suffix phase: one launch-wide round of waves at two waves per SIMD (a piece is
     streamed by one wave per 64/(head_dim/8) heads; measured: one to three waves per SIMD stream at the same rate,
-    and fewer, longer pieces pay the start-up chain less often), and no piece under 16 tokens."""
+    and fewer, longer pieces pay the start-up chain less often), and no piece under 4 tokens (one round of the
+    streaming body's register pipeline)."""
     heads_per_wave = max(1, 64 // max(1, head_dim // 8))
     hgroups = (num_heads + heads_per_wave - 1) // heads_per_wave
     cus = _cu_count(device)
     lanes = max(1, cus * 4 * 2 // hgroups)
-    return max(1, min(lanes, (total_tokens + 15) // 16))
+    return max(1, min(lanes, (total_tokens + 3) // 4))
 
 
 def plan_suffix_items(lens: Sequence[int], num_lanes: int):
