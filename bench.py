@@ -225,6 +225,7 @@ def extras(torch, dev):
     # --- config 5: full LLaMA-13B decoder layer, 4 prefix groups x 32 branches, prefix 6000 ------------------
     out["c5_layer"] = config5_layer(torch, dev)
     out["c2_iteration_tables"] = iteration_tables_cost(torch, dev)
+    out["prefix_length_sweep"] = prefix_length_sweep(torch, dev)
     out["e2e_decode_13b"] = e2e_decode(torch, dev)
     out["e2e_decode_13b_fused_ops"] = e2e_decode(torch, dev, fused_ops=True)
     # --- RMSNorm at a bandwidth-sized row count (LLaMA-13B hidden) -----------------------------------------
@@ -236,6 +237,46 @@ def extras(torch, dev):
     out["rms_norm_8192x5120"] = {"us": t * 1e6, "GB/s": nbytes / t / 1e9, "frac_hbm": nbytes / t / 1e9 / HBM_PEAK_GBS,
                                  "algorithmic_bytes": nbytes}
     return out
+
+
+def prefix_length_sweep(torch, dev):
+    """Fixed cost and steady state of the prefix + suffix launch: batch 64, 32 heads, ten-token suffixes, the shared
+    prefix swept from 512 to 32K tokens; a line through the two longest points gives the streaming rate, its
+    intercept the part of a launch that does not scale with the prefix (the chain of dependent steps)."""
+    from parrotserve_amd import _lib, kernels, synth
+
+    lib = _lib.load()
+    ev = HipEvents()
+    B, H, D = 64, 32, 128
+    res = {"batch": B, "heads": H, "suffix_len": "U[5,14]", "launch_us": {}}
+    pts = []
+    for P in (512, 2048, 8192, 16384, 32768):
+        g = torch.Generator().manual_seed(1)
+        lens = torch.randint(5, 15, (B,), generator=g).tolist()
+        case = synth.make_decode_case("sweep", 1, torch.float16, 1, B, P, lens, H, D, 1 << 18)
+        kc, vc = synth.pool_to_device(case.k_rows, case.v_rows, case.used_slots, case.pool_slots, dev)
+        tabs = kernels.DecodeTables.build(case.pool_lists(case.prefix_lists), case.group_req_cu,
+                                          case.pool_lists(case.suffix_lists), dev, num_heads=H, head_dim=D)
+        q = case.q.to(dev)
+        o = torch.empty_like(q)
+        for _ in range(5):
+            kernels.decode_attention(q, kc, vc, tabs, out=o)
+        sets = [ev.create(6) for _ in range(30)]
+        for s6 in sets:
+            lib.ph_arm_kernel_events(s6)
+            kernels.decode_attention(q, kc, vc, tabs, out=o)
+        torch.cuda.synchronize()
+        t = sorted(ev.elapsed_ms(s6[2], s6[3]) for s6 in sets)[15] * 1e3
+        for s6 in sets:
+            ev.destroy(s6)
+        res["launch_us"][str(P)] = t
+        pts.append((2 * P * H * D * 2 / 1e6, t))
+        del kc, vc, tabs
+    (x0, y0), (x1, y1) = pts[-2], pts[-1]
+    slope = (y1 - y0) / (x1 - x0)  # microseconds per MB of K/V
+    res["steady_state_GB/s"] = 1e3 / slope
+    res["fixed_us"] = y1 - slope * x1
+    return res
 
 
 def iteration_tables_cost(torch, dev):
