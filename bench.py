@@ -236,7 +236,41 @@ def extras(torch, dev):
     nbytes = 2 * xs[0].numel() * 2 + 5120 * 2
     out["rms_norm_8192x5120"] = {"us": t * 1e6, "GB/s": nbytes / t / 1e9, "frac_hbm": nbytes / t / 1e9 / HBM_PEAK_GBS,
                                  "algorithmic_bytes": nbytes}
+    out["sampler_64x32000"] = sampler_cost(torch, dev)
     return out
+
+
+def sampler_cost(torch, dev):
+    """Temperature + top-p + draw for a batch of 64 rows of 32,000 fp16 logits (everything in Sampler.forward after
+    the logits GEMM): the one-launch kernel, and beside it the reference's own sequence of library calls
+    (models/sampler.py:33-64: div, sort, softmax, cumsum, mask, argsort, gather, softmax, multinomial) timed on the
+    same GPU with the same inputs."""
+    from parrotserve_amd import kernels
+
+    B, V = 64, 32000
+    g = torch.Generator(device=dev).manual_seed(1)
+    logits = (torch.randn((B, V), device=dev, generator=g) * 4).half()
+    temp = torch.full((B,), 0.8, device=dev)
+    top_p = torch.full((B,), 0.9, device=dev)
+    u = torch.rand(B, device=dev, generator=g)
+
+    def library_sequence(filtered):
+        x = logits.clone()
+        x.div_(temp.unsqueeze(-1))
+        if filtered:
+            sorted_logits, idx = x.sort(dim=-1, descending=True)
+            probs = sorted_logits.softmax(dim=-1)
+            mask = (probs.cumsum(dim=-1) - probs) > top_p.unsqueeze(-1)
+            sorted_logits[mask] = -float("inf")
+            x = torch.gather(sorted_logits, dim=-1, index=torch.argsort(idx, dim=-1))
+        return torch.multinomial(torch.softmax(x, dim=-1, dtype=torch.float), num_samples=1, replacement=True)
+
+    res = {"rows": B, "vocab": V, "dtype": "f16"}
+    res["kernel_top_p_us"] = _time_gpu(torch, lambda: kernels.sample_top_p(logits, temp, top_p, u)) * 1e6
+    res["kernel_plain_draw_us"] = _time_gpu(torch, lambda: kernels.sample_top_p(logits, temp, None, u)) * 1e6
+    res["library_sequence_top_p_us"] = _time_gpu(torch, lambda: library_sequence(True), iters=10, inner=3) * 1e6
+    res["library_sequence_plain_draw_us"] = _time_gpu(torch, lambda: library_sequence(False), iters=10, inner=3) * 1e6
+    return res
 
 
 def prefix_length_sweep(torch, dev):
@@ -444,6 +478,8 @@ def main():
     ap.add_argument("--e2e-only", action="store_true",
                     help="only run the 13B-shape decode experiment (fused per-layer ops) and exit (for a kernel trace "
                          "of a whole engine iteration)")
+    ap.add_argument("--sampler-only", action="store_true",
+                    help="only time the token sampler (kernel and the reference's library-call sequence) and exit")
     ap.add_argument("--prefill-only", action="store_true",
                     help="only run config 4's prefill kernel a few times (for profiler counter passes) and exit")
     args = ap.parse_args()
@@ -460,6 +496,9 @@ def main():
     dev = torch.device("cuda:0")
     lib = _lib.load()
 
+    if args.sampler_only:
+        print(json.dumps({"sampler_64x32000": sampler_cost(torch, dev)}))
+        return
     if args.e2e_only:
         print(json.dumps({"e2e_decode_13b_fused_ops": e2e_decode(torch, dev, fused_ops=True)}))
         return

@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-typedef enum { PH_F16 = 0, PH_BF16 = 1 } ph_dtype;
+typedef enum { PH_F16 = 0, PH_BF16 = 1, PH_F32 = 2 /* ph_sample_top_p only */ } ph_dtype;
 typedef enum { PH_IDX_I32 = 0, PH_IDX_I64 = 1 } ph_index_type;
 
 enum {
@@ -379,6 +379,32 @@ int ph_suffix_tables_append(int32_t* table, int64_t table_stride, int32_t* lens,
  * request, attention_post_kernels.cu:74-110). */
 int ph_suffix_plan_build(const int32_t* suffix_lens, int64_t num_reqs, int64_t num_lanes,
                          int32_t* items, int32_t* lane_rec, int32_t* req_item_cu, void* stream);
+
+/* ------------------------------------------------------------------------ */
+/* Token sampler: temperature, top-p filter and one draw per row, in one launch.
+ * Replaces the body of Sampler.forward after the logits GEMM
+ * (parrot/engine/builtin/models/sampler.py:33-64: division by the
+ * temperature in the logits' element type, descending sort, soft-max,
+ * cumulative sum, mask, gather back through an arg-sort, soft-max,
+ * torch.multinomial).  Per row r:
+ *   x = logits[r] / temperature[r]   (rounded to the element type; skipped at 1)
+ *   token i survives iff the soft-max mass of the tokens sorted before it
+ *   (descending x, equal values by ascending id) is <= top_p[r];
+ *   out_ids[r] = the first id whose cumulative surviving mass, in ascending id
+ *   order, exceeds uniform[r] * (surviving mass).
+ * The filter is found by bisection over the element type's ordered bit
+ * patterns instead of a sort.  uniform[r] in [0, 1) comes from the caller's
+ * random generator, so the draw is reproducible from the inputs; the
+ * distribution of the drawn token is that of the reference, the mapping from
+ * a seed to a token is not (that one is torch.multinomial's).
+ * temperature == NULL means 1 for every row, top_p == NULL means 1 (no
+ * filter); a temperature <= 0 selects the most likely token.  logits
+ * [rows, vocab] with row_stride elements between rows, dtype PH_F16, PH_BF16
+ * or PH_F32; temperature, top_p, uniform: float32 [rows]; out_ids int64 [rows].
+ * All pointers DEVICE. */
+int ph_sample_top_p(const void* logits, int64_t row_stride, const float* temperature,
+                    const float* top_p, const float* uniform, int64_t* out_ids, int64_t rows,
+                    int64_t vocab, int dtype, void* stream);
 
 /* ------------------------------------------------------------------------ */
 /* Instrumentation (no counterpart in the reference, which times whole

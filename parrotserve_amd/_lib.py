@@ -14,7 +14,7 @@ from typing import Dict, List, Tuple
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(PKG_DIR, "libparrot_hip.so")
 
-PH_F16, PH_BF16 = 0, 1
+PH_F16, PH_BF16, PH_F32 = 0, 1, 2
 PH_IDX_I32, PH_IDX_I64 = 0, 1
 PH_OK, PH_ERR_DTYPE, PH_ERR_HEAD_DIM, PH_ERR_ALIGN, PH_ERR_ARG, PH_ERR_WORKSPACE, PH_ERR_LAUNCH = range(7)
 
@@ -43,6 +43,7 @@ SIGNATURES: Dict[str, Tuple[object, List[object]]] = {
     "ph_suffix_tables_append": (I, [P, L, P, P, P, L, P]),
     "ph_arm_kernel_events": (I, [P]),
     "ph_suffix_plan_build": (I, [P, L, L, P, P, P, P]),
+    "ph_sample_top_p": (I, [P, L, P, P, P, P, L, L, I, P]),
     "ph_prefill_workspace_bytes": (Z, [L, L, L, L]),
     "ph_prefill_attention": (I, [P, P, P, P, L, L, L, L, I, L, L, L, F, P, P, P, L, L, P, Z, P]),
 }

@@ -14,7 +14,7 @@ from concurrent.futures import ThreadPoolExecutor
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libparrot_hip.so")
-SOURCES = ["move_tokens.hip", "gather_blocked.hip", "norm_rope.hip", "fused.hip", "tables.hip", "decode.hip", "prefix_mfma.hip", "attention_api.hip"]
+SOURCES = ["move_tokens.hip", "gather_blocked.hip", "norm_rope.hip", "fused.hip", "sampler.hip", "tables.hip", "decode.hip", "prefix_mfma.hip", "attention_api.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950",

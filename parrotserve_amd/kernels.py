@@ -265,6 +265,31 @@ def silu_mul(gate: torch.Tensor, up: torch.Tensor, out: Optional[torch.Tensor] =
     return out.view(gate.shape)
 
 
+def sample_top_p(logits: torch.Tensor, temperature: Optional[torch.Tensor], top_p: Optional[torch.Tensor],
+                 uniform: torch.Tensor) -> torch.Tensor:
+    """Temperature, top-p filter and one draw per row of ``logits [B, V]`` (fp16, bf16 or fp32) in one launch: the
+    body of the reference's ``Sampler.forward`` after the logits GEMM (models/sampler.py:33-64), with the filter
+    found by bisection instead of two sorts and the draw taken from ``uniform [B]`` (float32 in [0, 1), from the
+    caller's generator) by inverse CDF over ascending token ids.  ``temperature`` / ``top_p``: float32 ``[B]`` on the
+    device, or ``None`` for 1.  Returns int64 ``[B]``."""
+    _require_gpu(logits, temperature, top_p, uniform)
+    assert logits.dim() == 2 and logits.stride(1) == 1
+    B, V = logits.shape
+    if logits.dtype == torch.float32:
+        code = _lib.PH_F32
+    else:
+        code = _dtype_code(logits)
+    for name, v in (("temperature", temperature), ("top_p", top_p), ("uniform", uniform)):
+        if v is not None and (v.dtype != torch.float32 or v.numel() != B or not v.is_contiguous()):
+            raise ValueError(f"{name} must be a contiguous float32 tensor of {B} elements")
+    out = torch.empty(B, dtype=torch.int64, device=logits.device)
+    check(_lib.load().ph_sample_top_p(_ptr(logits), logits.stride(0) if B > 1 else max(logits.stride(0), V),
+                                      _ptr(temperature) if temperature is not None else None,
+                                      _ptr(top_p) if top_p is not None else None, _ptr(uniform), _ptr(out), B, V, code,
+                                      _stream()), "sample_top_p")
+    return out
+
+
 def silu_and_mul(out: torch.Tensor, input: torch.Tensor) -> None:
     """vLLM's form (3rdparty/vllm/csrc/activation.cpp:3-6): ``input`` is ``[T, 2d]`` = gate | up."""
     d = input.shape[-1] // 2

@@ -17,7 +17,7 @@ from typing import Dict, List, Optional, Tuple
 import torch
 from torch import nn
 
-from . import mem
+from . import kernels, mem
 from .attn_func import BuiltinConfig
 from .context import BlockContext, RecyclePool
 from .iter_state import IterationState
@@ -77,7 +77,10 @@ class EngineContextManager:
 
 
 class Sampler(nn.Module):
-    """Temperature, top-p, multinomial draw over ``hidden @ lm_head.T`` (models/sampler.py:19-66)."""
+    """Temperature, top-p, one draw per row over ``hidden @ lm_head.T`` (models/sampler.py:19-66).  Everything
+    after the logits GEMM is one kernel (``ph_sample_top_p``): the reference's two sorts become a threshold search
+    and its ``torch.multinomial`` an inverse-CDF draw from ``torch.rand`` numbers, so the tokens follow torch's
+    generator (same seed, same tokens) with the reference's distribution."""
 
     def __init__(self, config: LlamaConfig, embd_weight: torch.Tensor):
         super().__init__()
@@ -89,19 +92,13 @@ class Sampler(nn.Module):
             return torch.zeros(0, dtype=torch.int64, device=hidden_states.device)
         assert hidden_states.shape[0] == len(sampling_config)
         logits = torch.matmul(hidden_states, self.embd_weight.t())
+        dev = logits.device
         temperature = [sc.temperature for sc in sampling_config]
-        if any(t != 1.0 for t in temperature):
-            logits.div_(torch.tensor(temperature, dtype=torch.float, device=logits.device).unsqueeze(-1))
         top_ps = [sc.top_p for sc in sampling_config]
-        if any(p < 1.0 for p in top_ps):
-            sorted_logits, logits_idx = logits.sort(dim=-1, descending=True)
-            tp = torch.tensor(top_ps, dtype=torch.float, device=logits.device).unsqueeze(-1)
-            sorted_probs = sorted_logits.softmax(dim=-1)
-            mask = (sorted_probs.cumsum(dim=-1) - sorted_probs) > tp
-            sorted_logits[mask] = -float("inf")
-            logits = torch.gather(sorted_logits, dim=-1, index=torch.argsort(logits_idx, dim=-1))
-        probs = torch.softmax(logits, dim=-1, dtype=torch.float)
-        return torch.multinomial(probs, num_samples=1, replacement=True).squeeze(-1)
+        t_dev = torch.tensor(temperature, dtype=torch.float, device=dev) if any(t != 1.0 for t in temperature) else None
+        p_dev = torch.tensor(top_ps, dtype=torch.float, device=dev) if any(p < 1.0 for p in top_ps) else None
+        uniform = torch.rand(logits.shape[0], dtype=torch.float, device=dev)
+        return kernels.sample_top_p(logits, t_dev, p_dev, uniform)
 
 
 def hidden_states_postprocess(hidden_states: torch.Tensor, iteration_state) -> Tuple[torch.Tensor, torch.Tensor]:

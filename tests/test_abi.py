@@ -91,6 +91,11 @@ def test_argument_validation_needs_no_gpu():
     assert lib.ph_suffix_plan_build(None, 0, 256, None, None, None, None) == _lib.PH_OK           # no requests
     assert lib.ph_suffix_plan_build(None, 8193, 256, None, None, None, None) == _lib.PH_ERR_ARG   # beyond the device planner
     assert lib.ph_suffix_plan_build(None, 4, 0, None, None, None, None) == _lib.PH_ERR_ARG
+    assert lib.ph_sample_top_p(None, 32000, None, None, None, None, 4, 32000, 0, None) == _lib.PH_ERR_ARG  # null pointers
+    assert lib.ph_sample_top_p(None, 32000, None, None, None, None, 0, 32000, 2, None) == _lib.PH_OK       # no rows
+    assert lib.ph_sample_top_p(None, 32000, None, None, None, None, 4, 32000, 7, None) == _lib.PH_ERR_DTYPE
+    assert lib.ph_sample_top_p(None, 100, None, None, None, None, 4, 32000, 0, None) == _lib.PH_ERR_ARG    # rows overlap
+    assert lib.ph_sample_top_p(None, 0, None, None, None, None, 4, 0, 0, None) == _lib.PH_ERR_ARG
     assert lib.ph_suffix_tables_append(None, 64, None, None, None, -1, None) == _lib.PH_ERR_ARG
     assert lib.ph_suffix_tables_append(None, 64, None, None, None, 0, None) == _lib.PH_OK
     assert lib.ph_suffix_tables_append(None, 64, None, None, None, 3, None) == _lib.PH_ERR_ARG
