@@ -5,17 +5,20 @@
 //           top_p -- the most likely token always stays, and so does the token on which the mass crosses top_p;
 //   :63-64  soft-max of the surviving logits, one token drawn from it.
 // The reference sorts every row twice (sort, then arg-sort of the permutation) to apply the filter.  Here the
-// filter is a threshold: with e_i = exp(x_i - max) and G(t) = sum of e_j over x_j > t, token i stays iff
-// G(x_i) + (its rank among equal values) * e_i <= top_p * sum(e).  G is monotone, so the smallest surviving value
+// filter is a threshold: with e_i = exp(x_i - max) and G(t) = sum of e_j over e_j > t, token i stays iff
+// G(e_i) + (its rank among equal values) * e_i <= top_p * sum(e).  G is monotone, so the smallest surviving value
 // is found by bisection over the ordered bit patterns of the element type (16 steps for bf16, 19 for fp16, 32
-// for fp32), each step one pass over the row's e values held in LDS (compare and add; the exponential is taken
-// once per token).  Equal values are ranked by ascending token id.
+// for fp32), each step a compare-and-add over the row's e values (the exponential is taken once per token) and
+// one block reduction.  Equal values are ranked by ascending token id.
 // The draw is the inverse-CDF draw over ascending token ids from a uniform number the caller passes, so the
 // result is a function of the inputs (the reference draws through torch.multinomial's own random stream).
 //
-// One workgroup of 1024 lanes per row; a row of up to 36 K tokens stays in LDS as fp32 between the passes,
-// longer rows are re-read and re-exponentiated in every pass (they sit in L2; slower, same result).  Sums are taken in a fixed order: per-lane strided partial sums,
-// a wave tree, then the sixteen wave sums in sequence -- the same result on every run.
+// One workgroup of 1024 lanes per row.  Two kernels, same arithmetic:
+//   sample_rows_kernel   rows on the 16-byte grid of up to 57,344 tokens: the row lives in registers;
+//   sample_top_p_kernel  any other row: e values in LDS up to 36 K tokens, longer rows are re-read and
+//                        re-exponentiated in every pass (they sit in L2; slower).
+// Sums are taken in a fixed order (per-lane partial sums, a wave tree, then the sixteen wave sums in
+// sequence): the same tokens on every run.
 #include "common.hpp"
 
 namespace ph {
