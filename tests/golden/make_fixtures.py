@@ -17,6 +17,7 @@ import torch
 HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
 
+from oracle import ref_sampler  # noqa: E402
 from oracle.ref_ops import (ref_add_rms_norm, ref_cos_sin_cache, ref_decode_attention, ref_kv_append,  # noqa: E402
                             ref_move_tokens, ref_prefill_with_parent, ref_rms_norm, ref_rope_neox, ref_silu_mul)
 
@@ -106,7 +107,24 @@ def elementwise_fixture():
              addnorm_y=bits(y_add), addnorm_h=bits(h_add), silu_mul=bits(act))
 
 
+def sampler_fixture():
+    """48 rows of 2000 fp16 logits with mixed temperatures and top-p values; only rows whose decisions are clear of
+    every rounding boundary (relative margin >= 1e-4) are kept, so any correct fp32 implementation draws these ids."""
+    g = torch.Generator().manual_seed(21)
+    B, V = 48, 2000
+    x = (torch.randn(B, V, generator=g) * 3).half()
+    temps = torch.tensor([1.0, 0.7, 1.5])[torch.randint(0, 3, (B,), generator=g)]
+    tops = torch.tensor([1.0, 0.9, 0.5, 1e-6])[torch.randint(0, 4, (B,), generator=g)]
+    u = torch.rand(B, generator=g)
+    ids, margins = ref_sampler.ref_sample(x.double().numpy(), temps.numpy(), tops.numpy(), u.numpy(), "f16")
+    keep = margins >= 1e-4
+    assert keep.sum() >= 40
+    np.savez(os.path.join(HERE, "sampler_fp16.npz"), logits=bits(x[keep]), temperature=temps.numpy()[keep],
+             top_p=tops.numpy()[keep], uniform=u.numpy()[keep], ids=ids[keep])
+
+
 if __name__ == "__main__":
+    sampler_fixture()
     decode_fixture(torch.float16, "decode_fp16.npz")
     decode_fixture(torch.bfloat16, "decode_bf16.npz")
     prefill_fixture()

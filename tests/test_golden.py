@@ -9,6 +9,8 @@ import torch
 from oracle.ref_ops import (ref_add_rms_norm, ref_decode_attention, ref_kv_append, ref_move_tokens,
                             ref_prefill_with_parent, ref_rms_norm, ref_rope_neox, ref_silu_mul)
 
+from oracle import ref_sampler
+
 GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 TOL = {torch.float16: dict(atol=2e-3, rtol=1e-2), torch.bfloat16: dict(atol=1e-2, rtol=2e-2)}
 # oracle against its own frozen output: reductions and exp may round differently on another host CPU, so
@@ -127,3 +129,20 @@ def test_gpu_prefill_and_elementwise_match_fixtures(dev):
     assert torch.equal(bits(rr), _t(e["addnorm_h"], h).view(torch.int16))
     torch.testing.assert_close(y.cpu().float(), _t(e["addnorm_y"], h).float(), **TOL[h])
     torch.testing.assert_close(kernels.silu_mul(x, r).cpu().float(), _t(e["silu_mul"], h).float(), **TOL[h])
+
+
+def test_oracle_reproduces_sampler_fixture():
+    f = _load("sampler_fp16.npz")
+    x = _t(f["logits"], torch.float16)
+    ids, margins = ref_sampler.ref_sample(x.double().numpy(), f["temperature"], f["top_p"], f["uniform"], "f16")
+    assert (ids == f["ids"]).all() and (margins >= 1e-4).all()
+
+
+@pytest.mark.gpu
+def test_gpu_sampler_matches_fixture(dev):
+    from parrotserve_amd import kernels
+
+    f = _load("sampler_fp16.npz")
+    ids = kernels.sample_top_p(_t(f["logits"], torch.float16).to(dev), _t(f["temperature"]).to(dev), _t(f["top_p"]).to(dev),
+                               _t(f["uniform"]).to(dev))
+    assert ids.cpu().tolist() == f["ids"].tolist()
