@@ -218,6 +218,34 @@ def test_reference_named_entry_points(dev):
     torch.testing.assert_close(out1.float(), ref.float(), **TOL[torch.float16])
 
 
+def test_reference_self_test_harness_shape(dev):
+    """The reference's own kernel check (kernels/shared_flash_decoding.py:417-459 and kernels/vllm/paged_attention.py:
+    81-134): 16 sequences of 1024 tokens, 48 heads of 64, contexts laid out back to back in the cache, inputs N(0, 1),
+    seed 2023, compared with its in-file formula at atol = rtol = 1e-2 -- here on the token-granular layout (a block
+    table is a slot list), against the oracle, at this build's tighter tolerance."""
+    from parrotserve_amd import kernels
+
+    torch.manual_seed(2023)
+    B, H, D, L = 16, 48, 64, 1024
+    q = torch.randn(B, H, D).half()
+    k = torch.randn(B * L + 64, H, D).half()
+    v = torch.randn(B * L + 64, H, D).half()
+    tables = torch.arange(B * L, dtype=torch.int32).reshape(B, L)
+    lens = torch.full((B,), L, dtype=torch.int32)
+    ref = ref_decode_attention(q, k, v, [tables[b].long() for b in range(B)])
+    hm = torch.arange(H, dtype=torch.int32, device=dev)
+    out = kernels.vllm_paged_attention(q.to(dev), k.to(dev), v.to(dev), hm, lens.to(dev), tables.to(dev)).cpu()
+    torch.testing.assert_close(out.float(), ref.float(), **TOL[torch.float16])
+    # the same contexts with their first 768 tokens declared as a prefix every sequence shares (sequence 0's slots)
+    P = 768
+    shared = torch.cat([tables[:1, :P].expand(B, P), tables[:, P:]], dim=1)
+    ref2 = ref_decode_attention(q, k, v, [shared[b].long() for b in range(B)])
+    for fn in (kernels.flash_paged_attention, kernels.paged_flash_attention):
+        out2 = fn(q.to(dev), k.to(dev), v.to(dev), hm, P, tables[0, :P].to(dev), (lens - P).to(dev),
+                  tables[:, P:].contiguous().to(dev)).cpu()
+        torch.testing.assert_close(out2.float(), ref2.float(), **TOL[torch.float16])
+
+
 def test_shared_equals_non_shared_property(dev):
     """Size-independent property at config-2 scale: the shared-prefix path and the
     non-shared ragged path agree (both on the GPU), and softmax weights sum to one
