@@ -47,7 +47,7 @@ static DecodePlan plan_decode(int64_t B, int64_t H, int64_t groups, int64_t max_
     p.chunk = 32;
     p.n_chunks = 0;
   } else if (max_suffix > 0 && chunk_tokens <= 0 && plan_head_dim >= 8 && B <= kPlanMaxReqs) {
-    const int64_t heads_per_wave = 64 / (plan_head_dim / 8) > 0 ? 64 / (plan_head_dim / 8) : 1;
+    const int64_t heads_per_wave = 64 / lanes_per_head((int)plan_head_dim) > 0 ? 64 / lanes_per_head((int)plan_head_dim) : 1;
     const int64_t lanes = (int64_t)device_cus() * 4 * 2 / cdiv(H, heads_per_wave);  // two waves per SIMD
     p.dev_lanes = (int)(lanes > 0 ? lanes : 1);
     p.items = p.dev_lanes + B;  // capacity: a cut at every lane mark and every request boundary
@@ -128,7 +128,7 @@ static Carve carve(void* ws, const DecodePlan& p, int64_t B, int64_t H, int64_t 
 static int check_common(const void* out, const void* q, const void* kc, const void* vc, int64_t B, int64_t H,
                         int64_t D, int dtype, int64_t q_stride, int64_t out_stride, int64_t row_stride) {
   if (dtype != PH_F16 && dtype != PH_BF16) return PH_ERR_DTYPE;
-  if (D != 64 && D != 128 && D != 256) return PH_ERR_HEAD_DIM;
+  if (D != 64 && D != 80 && D != 96 && D != 112 && D != 128 && D != 256) return PH_ERR_HEAD_DIM;
   if (B < 0 || H <= 0 || B > (1 << 24) || H > 4096) return PH_ERR_ARG;
   if (B == 0) return PH_OK;
   if (!out || !q || !kc || !vc) return PH_ERR_ARG;

@@ -155,6 +155,23 @@ KernelEvents take_kernel_events(int which);  // attention_api.hip; nulls unless 
       hipLaunchKernelGGL(kernel, grid, block, shmem, stream, __VA_ARGS__);                               \
   } while (0)
 
+// Lane mapping of the per-request decode kernels: a head's D elements are spread over LPH lanes of 8 elements
+// each, LPH the power of two >= D / 8, so that a wave holds 64 / LPH whole heads.  For D = 80, 96, 112 the lanes
+// past the head's last 8-element chunk are idle: they point at chunk 0 (a duplicate of another lane's load, no
+// extra traffic), carry a zero query and store nothing.
+constexpr int lanes_per_head(int D) {
+  int p = 1;
+  while (p * 8 < D) p <<= 1;
+  return p;
+}
+template <int D>
+struct HeadLanes {
+  static constexpr int LPH = lanes_per_head(D);
+  static constexpr int HPW = kWave / LPH;
+  static __device__ __forceinline__ bool active(int lane) { return LPH * 8 == D || (lane % LPH) * 8 < D; }
+  static __device__ __forceinline__ int chunk(int lane) { return active(lane) ? lane % LPH : 0; }
+};
+
 inline int launch_status() { return hipGetLastError() == hipSuccess ? PH_OK : PH_ERR_LAUNCH; }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

@@ -3,7 +3,8 @@
 // log-sum-exp merge.  HBM-bound (1 FLOP per KV byte): no MFMA, no LDS.
 //
 // Mapping: in the [slot, H, D] pool all heads of a token are one contiguous
-// row.  A wave owns HPW = 64 / (D/8) adjacent heads of one (request, chunk):
+// row.  A wave owns HPW = 64 / LPH adjacent heads of one (request, chunk), LPH = D/8 lanes per head
+// (rounded up to a power of two for D = 80, 96, 112, whose spare lanes idle):
 // each lane loads 8 contiguous elements (one 128-bit load), so a wave reads a
 // contiguous HPW*D*2-byte span of every token row.  The D/8 lanes of a head
 // combine their partial dot products with a butterfly; softmax runs online in
@@ -21,8 +22,8 @@ namespace ph {
 // of chunks past a request's end exit at once.  Used when the caller has no host copy of the lengths.
 template <typename E, int D, int TB, int STAGES>
 __global__ __launch_bounds__(256) void decode_partial_kernel(PartialArgs a) {
-  constexpr int LPH = D / 8;       // lanes per head
-  constexpr int HPW = kWave / LPH;  // heads per wave
+  constexpr int LPH = HeadLanes<D>::LPH;  // lanes per head
+  constexpr int HPW = HeadLanes<D>::HPW;  // heads per wave
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(blockIdx.x * 4 + (threadIdx.x >> 6));
   const int hgroups = (a.H + HPW - 1) / HPW;
@@ -59,8 +60,9 @@ __global__ __launch_bounds__(256) void decode_partial_kernel(PartialArgs a) {
   const int head = hg * HPW + lane / LPH;
   const bool head_ok = head < a.H;
   const int hclamp = head_ok ? head : a.H - 1;
-  const uint32_t lane_off = (uint32_t)(hclamp * D + (lane % LPH) * 8);  // elements inside a token row
-  const u32x4 qv = ld16(a.q + (int64_t)b * a.q_stride + lane_off);
+  const uint32_t lane_off = (uint32_t)(hclamp * D + HeadLanes<D>::chunk(lane) * 8);  // elements inside a token row
+  u32x4 qv = ld16(a.q + (int64_t)b * a.q_stride + lane_off);
+  if (!HeadLanes<D>::active(lane)) qv = u32x4{0u, 0u, 0u, 0u};
 
   if (t0 >= len) return;
   const int t1 = min(len, t0 + a.chunk);
@@ -74,7 +76,7 @@ __global__ __launch_bounds__(256) void decode_partial_kernel(PartialArgs a) {
 // so every wave of the launch moves the same number of bytes and the launch is a single round.
 template <typename E, int D, int TB, int STAGES>
 __global__ __launch_bounds__(256) void decode_items_kernel(ItemArgs a) {
-  constexpr int HPW = kWave / (D / 8);
+  constexpr int HPW = HeadLanes<D>::HPW;
   const int wave = __builtin_amdgcn_readfirstlane(blockIdx.x * 4 + (threadIdx.x >> 6));
   const int hgroups = (a.H + HPW - 1) / HPW;
   const int piece = wave / hgroups;
@@ -87,8 +89,8 @@ __global__ __launch_bounds__(256) void decode_items_kernel(ItemArgs a) {
 // then wave 0 folds the four running results through LDS and writes the output row.
 template <typename E, int D>
 __global__ __launch_bounds__(256) void merge_kernel(MergeArgs a) {
-  constexpr int LPH = D / 8;
-  constexpr int HPW = kWave / LPH;
+  constexpr int LPH = HeadLanes<D>::LPH;
+  constexpr int HPW = HeadLanes<D>::HPW;
   __shared__ float sh[3][10][kWave];
   const int lane = threadIdx.x & 63;
   const int w = threadIdx.x >> 6;
@@ -98,7 +100,7 @@ __global__ __launch_bounds__(256) void merge_kernel(MergeArgs a) {
   const int head_raw = hg * HPW + lane / LPH;
   const bool head_ok = head_raw < a.H;
   const int head = head_ok ? head_raw : a.H - 1;
-  const int dl = (lane % LPH) * 8;
+  const int dl = HeadLanes<D>::chunk(lane) * 8;
 
   float M = -INFINITY, L = 0.f;
   float acc[8];
@@ -175,13 +177,13 @@ __global__ __launch_bounds__(256) void merge_kernel(MergeArgs a) {
     for (int k = 0; k < 8; ++k) acc[k] = acc[k] * sa + sh[o][2 + k][lane] * sb;
     M = Mn;
   }
-  if (!head_ok) return;
+  if (!head_ok || !HeadLanes<D>::active(lane)) return;
   const float inv = L > 0.f ? 1.f / L : 0.f;
   u32x4 r;
 #pragma unroll
   for (int k = 0; k < 4; ++k) r[k] = pack2<E>(acc[2 * k] * inv, acc[2 * k + 1] * inv);
   st16(a.out + (int64_t)b * a.out_stride + (int64_t)head * D + dl, r);
-  if (a.m_out && dl == 0) {
+  if (a.m_out && lane % LPH == 0) {
     a.m_out[(int64_t)b * a.H + head] = M;
     a.l_out[(int64_t)b * a.H + head] = L;
   }
@@ -195,7 +197,7 @@ __global__ __launch_bounds__(256) void clear_ml_kernel(float* ml, int64_t n2) {
 
 template <typename E, int D>
 static int launch_partial_t(const PartialArgs& a, hipStream_t st) {
-  constexpr int HPW = kWave / (D / 8);
+  constexpr int HPW = HeadLanes<D>::HPW;
   const int64_t hgroups = (a.H + HPW - 1) / HPW;
   const int64_t waves = (int64_t)a.num_reqs * a.n_chunks * hgroups;
   if (waves == 0) return PH_OK;
@@ -207,7 +209,7 @@ static int launch_partial_t(const PartialArgs& a, hipStream_t st) {
 
 template <typename E, int D>
 static int launch_items_t(const ItemArgs& a, hipStream_t st) {
-  constexpr int HPW = kWave / (D / 8);
+  constexpr int HPW = HeadLanes<D>::HPW;
   const int64_t hgroups = (a.H + HPW - 1) / HPW;
   const int64_t waves = (int64_t)a.num_lanes * hgroups;
   if (waves == 0) return PH_OK;
@@ -219,7 +221,7 @@ static int launch_items_t(const ItemArgs& a, hipStream_t st) {
 
 template <typename E, int D>
 static int launch_merge_t(const MergeArgs& a, hipStream_t st) {
-  constexpr int HPW = kWave / (D / 8);
+  constexpr int HPW = HeadLanes<D>::HPW;
   const int64_t hgroups = (a.H + HPW - 1) / HPW;
   const int64_t groups = (int64_t)a.B * hgroups;
   if (groups == 0) return PH_OK;
@@ -235,10 +237,16 @@ static int launch_merge_t(const MergeArgs& a, hipStream_t st) {
       if ((D) == 128) return FN<F16, 128>(__VA_ARGS__);                 \
       if ((D) == 64) return FN<F16, 64>(__VA_ARGS__);                   \
       if ((D) == 256) return FN<F16, 256>(__VA_ARGS__);                 \
+      if ((D) == 80) return FN<F16, 80>(__VA_ARGS__);                   \
+      if ((D) == 96) return FN<F16, 96>(__VA_ARGS__);                   \
+      if ((D) == 112) return FN<F16, 112>(__VA_ARGS__);                 \
     } else {                                                            \
       if ((D) == 128) return FN<BF16, 128>(__VA_ARGS__);                \
       if ((D) == 64) return FN<BF16, 64>(__VA_ARGS__);                  \
       if ((D) == 256) return FN<BF16, 256>(__VA_ARGS__);                \
+      if ((D) == 80) return FN<BF16, 80>(__VA_ARGS__);                  \
+      if ((D) == 96) return FN<BF16, 96>(__VA_ARGS__);                  \
+      if ((D) == 112) return FN<BF16, 112>(__VA_ARGS__);                \
     }                                                                   \
     return PH_ERR_HEAD_DIM;                                             \
   } while (0)

@@ -19,7 +19,7 @@ __device__ __forceinline__ void stream_item(const uint16_t* __restrict__ kc, con
                                             int t0, int t1, u32x4 qv, uint32_t lane_off, float scale_log2e,
                                             bool head_ok, float* __restrict__ opart, float* __restrict__ ml,
                                             int64_t pr) {
-  constexpr int LPH = D / 8;
+  constexpr int LPH = HeadLanes<D>::LPH;
   const int lane = threadIdx.x & 63;
   float m = -INFINITY, l = 0.f;
   float o[8];
@@ -91,7 +91,7 @@ __device__ __forceinline__ void stream_item(const uint16_t* __restrict__ kc, con
     }
   }
 
-  if (!head_ok) return;
+  if (!head_ok || !HeadLanes<D>::active(lane)) return;
   const float inv = 1.f / l;
   float* op = opart + pr * D + (lane % LPH) * 8;
   float4_t o0 = {o[0] * inv, o[1] * inv, o[2] * inv, o[3] * inv};
@@ -109,13 +109,13 @@ __device__ __forceinline__ void stream_item(const uint16_t* __restrict__ kc, con
 // (rec0, rec1) = the piece's lane record, already loaded by the caller
 template <typename E, int D, int TB, int STAGES>
 __device__ __forceinline__ void run_piece_rec(const ItemArgs& a, int hg, int4 rec0, int4 rec1) {
-  constexpr int LPH = D / 8;
-  constexpr int HPW = kWave / LPH;
+  constexpr int LPH = HeadLanes<D>::LPH;
+  constexpr int HPW = HeadLanes<D>::HPW;
   const int lane = threadIdx.x & 63;
   const int head = hg * HPW + lane / LPH;
   const bool head_ok = head < a.H;
   const int hclamp = head_ok ? head : a.H - 1;
-  const uint32_t lane_off = (uint32_t)(hclamp * D + (lane % LPH) * 8);
+  const uint32_t lane_off = (uint32_t)(hclamp * D + HeadLanes<D>::chunk(lane) * 8);
   const int i0 = rec0.x, i1 = rec0.x + rec0.y;
   for (int it = i0; it < i1; ++it) {
     int4 meta = {rec0.z, rec0.w, rec1.x, 0};
@@ -123,7 +123,8 @@ __device__ __forceinline__ void run_piece_rec(const ItemArgs& a, int hg, int4 re
     const int b = meta.x, t0 = meta.y, t1 = meta.y + meta.z;
     const int32_t* slots = a.slots + (a.offsets ? a.offsets[b] : (int64_t)b * a.table_stride);
     const int myslot = slots[min(t0 + lane, t1 - 1)];
-    const u32x4 qv = ld16(a.q + (int64_t)b * a.q_stride + lane_off);
+    u32x4 qv = ld16(a.q + (int64_t)b * a.q_stride + lane_off);
+    if (!HeadLanes<D>::active(lane)) qv = u32x4{0u, 0u, 0u, 0u};
     stream_item<E, D, TB, STAGES>(a.kc, a.vc, a.row_stride, slots, myslot, t0, t1, qv, lane_off, a.scale_log2e,
                                   head_ok, a.opart, a.ml, (int64_t)it * a.H + hclamp);
   }

@@ -542,19 +542,27 @@ def suffix_plan_build(lens: torch.Tensor, num_lanes: int, items: torch.Tensor, l
 PLAN_MAX_REQS = 8192  # batch size up to which the library plans on the device
 
 
+def _heads_per_wave(head_dim: int) -> int:
+    """A head's elements sit on head_dim / 8 lanes, rounded up to a power of two (80, 96, 112 take 16 like 128)."""
+    lanes = 1
+    while lanes * 8 < head_dim:
+        lanes *= 2
+    return max(1, 64 // lanes)
+
+
 def suffix_lane_capacity(device, num_heads: int, head_dim: int) -> int:
     """Lanes of the device-built plan: one launch-wide round of waves at two waves per SIMD (see suffix_lanes)."""
-    heads_per_wave = max(1, 64 // max(1, head_dim // 8))
+    heads_per_wave = _heads_per_wave(head_dim)
     hgroups = (num_heads + heads_per_wave - 1) // heads_per_wave
     return max(1, _cu_count(device) * 4 * 2 // hgroups)
 
 
 def suffix_lanes(device, num_heads: int, head_dim: int, total_tokens: int) -> int:
     """Pieces of the balanced suffix phase: one launch-wide round of waves at two waves per SIMD (a piece is
-    streamed by one wave per 64/(head_dim/8) heads; measured: one to three waves per SIMD stream at the same rate,
+    streamed by one wave per `_heads_per_wave(head_dim)` heads; measured: one to three waves per SIMD stream at the same rate,
     and fewer, longer pieces pay the start-up chain less often), and no piece under 4 tokens (one round of the
     streaming body's register pipeline)."""
-    heads_per_wave = max(1, 64 // max(1, head_dim // 8))
+    heads_per_wave = _heads_per_wave(head_dim)
     hgroups = (num_heads + heads_per_wave - 1) // heads_per_wave
     cus = _cu_count(device)
     lanes = max(1, cus * 4 * 2 // hgroups)

@@ -60,7 +60,7 @@ def test_argument_validation_needs_no_gpu():
     assert lib.ph_move_tokens(None, None, None, None, 0, 0, 2, 8, 2, 16, 8, 1, 16, 8, 1, None) == _lib.PH_OK
     assert lib.ph_rms_norm(None, None, None, 1e-6, 4, 64, 64, 64, 7, 1, None) == _lib.PH_ERR_DTYPE
     # unsupported head size mirrors the reference's "Unsupported head size" check
-    rc = lib.ph_decode_attention(1, 1, 1, 1, 4, 2, 80, 0, 160, 160, 160, 1.0, 0, None, None, None, None, 0,
+    rc = lib.ph_decode_attention(1, 1, 1, 1, 4, 2, 72, 0, 144, 144, 144, 1.0, 0, None, None, None, None, 0,
                                  None, None, 0, 0, None, 0, 0, None, None, 0, None)
     assert rc == _lib.PH_ERR_HEAD_DIM
     # fused per-layer ops and the table patch

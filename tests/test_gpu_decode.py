@@ -135,8 +135,10 @@ def test_suffix_chunking_is_invisible(dev, chunk):
     _check(case, dev, chunk_tokens=chunk)
 
 
-@pytest.mark.parametrize("D,H", [(64, 12), (256, 3), (128, 5)])
+@pytest.mark.parametrize("D,H", [(64, 12), (256, 3), (128, 5), (80, 32), (80, 5), (96, 7), (112, 3)])
 def test_other_head_sizes_and_odd_head_counts(dev, D, H):
+    """Every head size the reference's kernels dispatch (csrc/attention/attention_post_kernels.cu:420-446:
+    64, 80, 96, 112, 128, 256); 80 x 32 is OPT-2.7B's shape."""
     from parrotserve_amd import synth
 
     g = torch.Generator().manual_seed(8)
@@ -269,8 +271,8 @@ def test_shared_equals_non_shared_property(dev):
 def test_unsupported_inputs_raise(dev):
     from parrotserve_amd import kernels
 
-    q = torch.zeros(2, 2, 80, dtype=torch.float16, device=dev)
-    kc = torch.zeros(8, 2, 80, dtype=torch.float16, device=dev)
+    q = torch.zeros(2, 2, 72, dtype=torch.float16, device=dev)
+    kc = torch.zeros(8, 2, 72, dtype=torch.float16, device=dev)
     t = kernels.DecodeTables.build([], [], [[0, 1], [2]], dev)
     with pytest.raises(RuntimeError, match="head size"):
         kernels.decode_attention(q, kc, kc, t)

@@ -137,7 +137,7 @@ def test_prefill_heads_not_multiple_of_eight_and_tail_tiles(dev):
         torch.testing.assert_close(out.float(), ref.float(), **TOL[torch.bfloat16])
 
 
-@pytest.mark.parametrize("D,H", [(64, 6), (256, 2)])
+@pytest.mark.parametrize("D,H", [(64, 6), (256, 2), (80, 5), (96, 3), (112, 2)])
 def test_prefill_other_head_sizes(dev, D, H):
     """Head sizes the matrix-core kernel does not cover run every query row through the per-request kernel
     over its visible slots; same results."""
