@@ -207,6 +207,10 @@ int ph_rotary_embedding(void* state, const void* cos, const void* sin,
  *   num_items and num_lanes fixed and rewrites the arrays in place.
  * workspace: at least ph_decode_workspace_bytes(...) bytes, 256-byte aligned
  *   (num_items = plan->num_items, or 0 without a plan).
+ * head_dim: 64, 80, 96, 112, 128 or 256 -- the sizes the reference's kernels
+ *   dispatch (csrc/attention/attention_post_kernels.cu:420-446); anything else
+ *   returns PH_ERR_HEAD_DIM.  The same set holds for every attention entry
+ *   point below.
  */
 typedef struct {
   const int32_t* items;
