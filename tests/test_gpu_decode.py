@@ -220,6 +220,32 @@ def test_reference_named_entry_points(dev):
     torch.testing.assert_close(out1.float(), ref.float(), **TOL[torch.float16])
 
 
+@pytest.mark.parametrize("B,grouped", [(8192, True), (8193, False), (9000, True)])
+def test_batches_around_the_device_planner_limit(dev, B, grouped):
+    """The suffix plan is written on the device for up to 8192 requests and on the host beyond; thousands of
+    requests with one to three tokens each (and a 40-token prefix every request shares) against the oracle."""
+    from parrotserve_amd import kernels
+
+    g = torch.Generator().manual_seed(5 + B)
+    H, D = 2, 128
+    lens = torch.randint(1, 4, (B,), generator=g).tolist()
+    total, P = sum(lens), (40 if grouped else 0)
+    perm = torch.randperm(total + P + 16, generator=g)
+    k = torch.randn(total + P + 16, H, D, generator=g).half()
+    v = torch.randn(total + P + 16, H, D, generator=g).half()
+    q = torch.randn(B, H, D, generator=g).half()
+    pre, pos, suf = perm[:P], P, []
+    for n in lens:
+        suf.append(perm[pos:pos + n])
+        pos += n
+    t = kernels.DecodeTables.build([pre.tolist()] if grouped else [], [0, B] if grouped else [],
+                                   [s.tolist() for s in suf], dev, num_heads=H, head_dim=D)
+    assert t.plan is not None
+    out = kernels.decode_attention(q.to(dev), k.to(dev), v.to(dev), t).cpu()
+    ref = ref_decode_attention(q, k, v, [torch.cat([pre, s]) for s in suf])
+    torch.testing.assert_close(out.float(), ref.float(), **TOL[torch.float16])
+
+
 def test_reference_self_test_harness_shape(dev):
     """The reference's own kernel check (kernels/shared_flash_decoding.py:417-459 and kernels/vllm/paged_attention.py:
     81-134): 16 sequences of 1024 tokens, 48 heads of 64, contexts laid out back to back in the cache, inputs N(0, 1),
