@@ -237,7 +237,29 @@ def extras(torch, dev):
     out["rms_norm_8192x5120"] = {"us": t * 1e6, "GB/s": nbytes / t / 1e9, "frac_hbm": nbytes / t / 1e9 / HBM_PEAK_GBS,
                                  "algorithmic_bytes": nbytes}
     out["sampler_64x32000"] = sampler_cost(torch, dev)
+    out["c2_shape_head_size_64"] = head_size_64_step(torch, dev)
     return out
+
+
+def head_size_64_step(torch, dev):
+    """Config 2's batch with 64-wide heads (32 x 64, the OPT-1.3B shape): the prefix phase runs on head pairs through
+    the 128-wide matrix-core kernel, the suffix phase and the merge at the native width.  Warm (one KV set)."""
+    from parrotserve_amd import kernels, synth
+
+    g = torch.Generator().manual_seed(1)
+    B, P, H, D = 64, 4096, 32, 64
+    s = torch.randint(16, 513, (B,), generator=g).tolist()
+    case = synth.make_decode_case("d64", 1, torch.float16, 1, B, P, s, H, D, 1 << 20)
+    kc, vc = synth.pool_to_device(case.k_rows, case.v_rows, case.used_slots, case.pool_slots, dev)
+    tables = kernels.DecodeTables.build(case.pool_lists(case.prefix_lists), case.group_req_cu,
+                                        case.pool_lists(case.suffix_lists), dev, num_heads=H, head_dim=D)
+    q = case.q.to(dev)
+    o = torch.empty_like(q)
+    t = _time_gpu(torch, lambda: kernels.decode_attention(q, kc, vc, tables, out=o))
+    nbytes = 2 * (P + sum(s)) * H * D * 2
+    return {"batch": B, "prefix": P, "sum_suffix": sum(s), "heads": H, "head_dim": D, "us": t * 1e6,
+            "GB/s": nbytes / t / 1e9, "frac_hbm": nbytes / t / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": nbytes,
+            "tokens/s/layer": B / t}
 
 
 def sampler_cost(torch, dev):

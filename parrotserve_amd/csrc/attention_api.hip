@@ -12,6 +12,7 @@ struct DecodePlan {
   int n_splits;      // prefix parts
   int64_t items;     // suffix items (balanced form), 0 in the grid form
   int dev_lanes;     // lanes of a plan the library builds on the device into the workspace (0: the caller's plan or none)
+  bool paired;       // D == 64: the prefix phase runs on head pairs through the 128-wide matrix-core kernel
   int parts() const { return n_chunks + n_splits; }
   // partial rows (one row = one head's (O, m, l)): [parts][B][H] then [items][H]
   size_t rows(int64_t B, int64_t H) const { return (size_t)parts() * B * H + (size_t)items * H; }
@@ -40,7 +41,8 @@ static int device_cus() {
 // balanced form from a plan built on the device (up to kPlanMaxReqs requests); an explicit chunk size keeps the
 // plain (request, chunk) grid.
 static DecodePlan plan_decode(int64_t B, int64_t H, int64_t groups, int64_t max_prefix, int64_t max_suffix,
-                              int64_t chunk_tokens, int64_t num_items = 0, int64_t plan_head_dim = 0) {
+                              int64_t chunk_tokens, int64_t num_items = 0, int64_t plan_head_dim = 0,
+                              bool paired = false) {
   DecodePlan p{};
   p.items = num_items;
   if (num_items > 0) {
@@ -73,10 +75,12 @@ static DecodePlan plan_decode(int64_t B, int64_t H, int64_t groups, int64_t max_
     // split count whose workgroup total wastes the least of a whole number of 256-wide rounds.
     // Cost model: rounds x (tokens per split + a fixed prologue/epilogue worth ~96 tokens).
     // the kernel takes 64-, 128- or 256-query tiles by the largest group; the mean group size stands in here
-    const int64_t per_group = cdiv(B, groups);
+    p.paired = paired;
+    const int64_t rows_b = paired ? 2 * B : B, rows_h = paired ? H / 2 : H;  // what the kernel sees
+    const int64_t per_group = cdiv(rows_b, groups);
     const int64_t qtile = per_group <= 64 ? kPrefixQueryTile : per_group <= 128 ? 2 * kPrefixQueryTile : 4 * kPrefixQueryTile;
     const int64_t mtiles = cdiv(per_group, qtile);
-    const int64_t base = groups * H * (mtiles > 0 ? mtiles : 1);
+    const int64_t base = groups * rows_h * (mtiles > 0 ? mtiles : 1);
     const int64_t max_splits = cdiv(max_prefix, 4 * kPrefixTile);
     int64_t splits = 1, best = -1;
     for (int64_t s = 1; s <= 64 && s <= (max_splits > 0 ? max_splits : 1); ++s) {
@@ -99,6 +103,9 @@ static size_t plan_bytes(const DecodePlan& p, int64_t B, int64_t H, int64_t D) {
   size_t n = round_up((int64_t)(rows * D * sizeof(float)), 256) + round_up((int64_t)(rows * 2 * sizeof(float)), 256);
   if (p.dev_lanes > 0)
     n += round_up(p.items * 16, 256) + round_up((int64_t)p.dev_lanes * 32, 256) + round_up((B + 1) * 4, 256);
+  if (p.paired)  // the widened query rows, and the head-pair partials of the prefix parts
+    n += round_up(B * H * 128 * 2, 256) + round_up((int64_t)p.n_splits * B * H * 128 * 4, 256) +
+         round_up((int64_t)p.n_splits * B * H * 2 * 4, 256);
   return n;
 }
 
@@ -106,6 +113,8 @@ struct Carve {
   float* opart;
   float* ml;
   int32_t *items, *lane_rec, *req_item_cu;  // the device-built plan (dev_lanes > 0)
+  uint16_t* q_pairs;                        // paired prefix phase: [2B][H/2][128] queries,
+  float *opart_pairs, *ml_pairs;            // [n_splits][2B][H/2] partial rows of 128 floats / (m, l)
 };
 static Carve carve(void* ws, const DecodePlan& p, int64_t B, int64_t H, int64_t D) {
   const size_t rows = p.rows(B, H);
@@ -121,8 +130,40 @@ static Carve carve(void* ws, const DecodePlan& p, int64_t B, int64_t H, int64_t 
     c.lane_rec = (int32_t*)at;
     at += round_up((int64_t)p.dev_lanes * 32, 256);
     c.req_item_cu = (int32_t*)at;
+    at += round_up((B + 1) * 4, 256);
+  }
+  if (p.paired) {
+    c.q_pairs = (uint16_t*)at;
+    at += round_up(B * H * 128 * 2, 256);
+    c.opart_pairs = (float*)at;
+    at += round_up((int64_t)p.n_splits * B * H * 128 * 4, 256);
+    c.ml_pairs = (float*)at;
   }
   return c;
+}
+
+// D == 64 with an even head count: two adjacent heads of a token row are one 128-wide row of the matrix-core
+// kernel.  Request b, head 2p + s becomes row 2b + s, pseudo-head p, whose query is the head's 64 values in
+// half s and zeros in the other half: the zeros cancel the neighbour's keys in the score, and half s of the
+// 128-wide output is exactly the head's output (the other half, the neighbour's values under this head's
+// weights, is ignored).  Twice the matrix work, the same K/V traffic -- read once per group, not once per request.
+static bool pair_heads(int64_t D, int64_t H) { return D == 64 && H % 2 == 0; }
+
+__global__ __launch_bounds__(256) void widen_queries_kernel(const uint16_t* __restrict__ q, int64_t q_stride,
+                                                            uint16_t* __restrict__ q2, int B, int H) {
+  // one 16-byte chunk per thread: 16 chunks per (row, pseudo-head), chunks 8s .. 8s+7 carry the head's values
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t total = (int64_t)2 * B * (H / 2) * 16;
+  if (i >= total) return;
+  const int c = (int)(i & 15);
+  const int64_t rp = i >> 4;
+  const int p = (int)(rp % (H / 2));
+  const int64_t row = rp / (H / 2);
+  const int s = (int)(row & 1);
+  const int64_t b = row >> 1;
+  u32x4 v = {0u, 0u, 0u, 0u};
+  if ((c >> 3) == s) v = ld16(q + b * q_stride + (int64_t)(2 * p + s) * 64 + (c & 7) * 8);
+  st16(q2 + i * 8, v);
 }
 
 static int check_common(const void* out, const void* q, const void* kc, const void* vc, int64_t B, int64_t H,
@@ -142,7 +183,22 @@ static int check_common(const void* out, const void* q, const void* kc, const vo
 // Prefix phase: matrix-core kernel for head size 128; other head sizes run the
 // per-request gather kernel once per group over the shared slot list.
 static int run_prefix(PrefixArgs& pa, int dtype, int D, int num_groups, const int32_t* group_req_cu_host,
-                      int max_group_reqs, hipStream_t st) {
+                      int max_group_reqs, hipStream_t st, const Carve* pairs = nullptr) {
+  if (pairs && pairs->q_pairs) {
+    const int64_t chunks = (int64_t)2 * pa.B * (pa.H / 2) * 16;
+    hipLaunchKernelGGL(widen_queries_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, st, pa.q, pa.q_stride,
+                       pairs->q_pairs, pa.B, pa.H);
+    if (launch_status() != PH_OK) return PH_ERR_LAUNCH;
+    PrefixArgs w = pa;
+    w.q = pairs->q_pairs;
+    w.q_stride = (int64_t)(pa.H / 2) * 128;
+    w.B = 2 * pa.B;
+    w.H = pa.H / 2;
+    w.req_shift = 1;
+    w.opart = pairs->opart_pairs;
+    w.ml = pairs->ml_pairs;
+    return launch_prefix_mfma(w, dtype, 128, num_groups, 2 * max_group_reqs, st);
+  }
   if (prefix_mfma_supported(dtype, D)) return launch_prefix_mfma(pa, dtype, D, num_groups, max_group_reqs, st);
   int rc = launch_clear_ml(pa.ml, (int64_t)pa.n_splits * pa.B * pa.H, st);
   if (rc != PH_OK) return rc;
@@ -231,7 +287,8 @@ extern "C" size_t ph_decode_workspace_bytes(int64_t num_reqs, int64_t num_heads,
                                             int64_t chunk_tokens, int64_t num_items) {
   if (num_reqs <= 0 || num_heads <= 0 || head_dim <= 0) return 0;
   const DecodePlan p =
-      plan_decode(num_reqs, num_heads, num_groups, max_prefix_len, max_suffix_len, chunk_tokens, num_items, head_dim);
+      plan_decode(num_reqs, num_heads, num_groups, max_prefix_len, max_suffix_len, chunk_tokens, num_items, head_dim,
+                  pair_heads(head_dim, num_heads));
   return plan_bytes(p, num_reqs, num_heads, head_dim);
 }
 
@@ -258,8 +315,9 @@ extern "C" int ph_decode_attention(void* out, const void* q, const void* k_cache
   if (planned && (!plan->items || !plan->lane_rec || !plan->req_item_cu || plan->num_lanes <= 0 ||
                   plan->num_items > (int64_t)1 << 30))
     return PH_ERR_ARG;
+  const bool paired = pair_heads(D, H) && prefix_mfma_supported(dtype, 128);
   const DecodePlan p = plan_decode(num_reqs, num_heads, has_prefix ? num_groups : 0, max_prefix_len, max_suffix_len,
-                                   chunk_tokens, planned ? plan->num_items : 0, head_dim);
+                                   chunk_tokens, planned ? plan->num_items : 0, head_dim, pair_heads(D, H));
   if (plan_bytes(p, B, H, D) > workspace_bytes || ((p.parts() > 0 || p.items > 0) && !workspace))
     return PH_ERR_WORKSPACE;
   if (((uintptr_t)workspace & 255u) != 0) return PH_ERR_ALIGN;
@@ -286,7 +344,7 @@ extern "C" int ph_decode_attention(void* out, const void* q, const void* k_cache
       if (r1 - r0 > max_group_reqs) max_group_reqs = r1 - r0;
     }
     if (covered != B) {  // requests outside every group: their prefix parts must read as empty
-      rc = launch_clear_ml(ws.ml, (int64_t)p.n_splits * B * H, st);
+      rc = launch_clear_ml(paired ? ws.ml_pairs : ws.ml, (int64_t)p.n_splits * B * H, st);
       if (rc != PH_OK) return rc;
     }
     PrefixArgs pa{};
@@ -312,7 +370,7 @@ extern "C" int ph_decode_attention(void* out, const void* q, const void* k_cache
       fused_groups = (int)num_groups;
       fused_max_reqs = max_group_reqs;
     } else {
-      rc = run_prefix(pa, dtype, D, (int)num_groups, group_req_cu_host, max_group_reqs, st);
+      rc = run_prefix(pa, dtype, D, (int)num_groups, group_req_cu_host, max_group_reqs, st, paired ? &ws : nullptr);
       if (rc != PH_OK) return rc;
     }
   }
@@ -372,6 +430,10 @@ extern "C" int ph_decode_attention(void* out, const void* q, const void* k_cache
   ma.B = B;
   ma.H = H;
   ma.nA = has_prefix ? p.n_splits : 0;
+  if (has_prefix && paired) {
+    ma.opart_pairs = ws.opart_pairs;
+    ma.ml_pairs = ws.ml_pairs;
+  }
   ma.baseB = p.n_splits;
   ma.lens = has_suffix ? suffix_lens : nullptr;
   ma.chunk = p.chunk;
@@ -394,7 +456,8 @@ static int prefix_phase(void* out, const float* prev_m, const float* prev_l, flo
                         cache_stride_n);
   if (rc != PH_OK || num_reqs == 0) return rc;
   if (prefix_len < 0 || (prefix_len > 0 && !prefix_slots)) return PH_ERR_ARG;
-  const DecodePlan p = plan_decode(num_reqs, num_heads, prefix_len > 0 ? 1 : 0, prefix_len, 0, 0);
+  const bool paired = pair_heads(D, H) && prefix_mfma_supported(dtype, 128);
+  const DecodePlan p = plan_decode(num_reqs, num_heads, prefix_len > 0 ? 1 : 0, prefix_len, 0, 0, 0, 0, pair_heads(D, H));
   if (plan_bytes(p, B, H, D) > workspace_bytes || (p.parts() > 0 && !workspace)) return PH_ERR_WORKSPACE;
   if (((uintptr_t)workspace & 255u) != 0) return PH_ERR_ALIGN;
   const Carve ws = carve(workspace, p, B, H, D);
@@ -417,12 +480,16 @@ static int prefix_phase(void* out, const float* prev_m, const float* prev_l, flo
     pa.B = B;
     pa.H = H;
     pa.scale_log2e = scale * kLog2e;
-    rc = run_prefix(pa, dtype, D, 1, nullptr, B, st);
+    rc = run_prefix(pa, dtype, D, 1, nullptr, B, st, paired ? &ws : nullptr);
     if (rc != PH_OK) return rc;
   }
   MergeArgs ma{};
   ma.opart = ws.opart;
   ma.ml = ws.ml;
+  if (prefix_len > 0 && paired) {
+    ma.opart_pairs = ws.opart_pairs;
+    ma.ml_pairs = ws.ml_pairs;
+  }
   ma.out = (uint16_t*)out;
   ma.out_stride = out_stride;
   ma.B = B;

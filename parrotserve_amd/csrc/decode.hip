@@ -134,14 +134,23 @@ __global__ __launch_bounds__(256) void merge_kernel(MergeArgs a) {
 #pragma unroll 2
   for (int i = w; i < total; i += 4) {
     int64_t pr;
-    if (i < a.nA)
-      pr = ((int64_t)i * a.B + b) * a.H + head;
-    else if (a.req_item_cu)
-      pr = a.item_base + (int64_t)(it0 + i - a.nA) * a.H + head;
-    else
-      pr = ((int64_t)(a.baseB + i - a.nA) * a.B + b) * a.H + head;
-    const float2 mlp = *reinterpret_cast<const float2*>(a.ml + pr * 2);
-    const float* op = a.opart + pr * D + dl;
+    const float* mlrow;
+    const float* op;
+    if (i < a.nA && a.opart_pairs) {  // D == 64: this head is one half of a 128-wide row
+      pr = ((int64_t)i * (2 * a.B) + 2 * b + (head & 1)) * (a.H >> 1) + (head >> 1);
+      mlrow = a.ml_pairs + pr * 2;
+      op = a.opart_pairs + pr * (2 * D) + (head & 1) * D + dl;
+    } else {
+      if (i < a.nA)
+        pr = ((int64_t)i * a.B + b) * a.H + head;
+      else if (a.req_item_cu)
+        pr = a.item_base + (int64_t)(it0 + i - a.nA) * a.H + head;
+      else
+        pr = ((int64_t)(a.baseB + i - a.nA) * a.B + b) * a.H + head;
+      mlrow = a.ml + pr * 2;
+      op = a.opart + pr * D + dl;
+    }
+    const float2 mlp = *reinterpret_cast<const float2*>(mlrow);
     const float4_t o0 = *reinterpret_cast<const float4_t*>(op);
     const float4_t o1 = *reinterpret_cast<const float4_t*>(op + 4);
     const bool live = mlp.y > 0.f;  // l == 0 marks an empty part (its O may be garbage)

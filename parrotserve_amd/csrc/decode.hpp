@@ -53,6 +53,11 @@ struct ItemArgs {
 struct MergeArgs {
   const float* opart;
   const float* ml;
+  // Head pairs (D = 64 only): parts [0, nA) were written by the 128-wide matrix-core kernel on a query set in which
+  // request b, head 2p + s is row 2b + s, head p, with the other head's half of the query zeroed; they live in
+  // their own buffers, rows of 128 floats [part][2B][H/2], of which dims [64 s, 64 s + 64) are this head's output.
+  const float* opart_pairs;
+  const float* ml_pairs;
   uint16_t* out;
   int64_t out_stride;
   int B, H;
@@ -77,6 +82,7 @@ struct PrefixArgs {
   const int32_t* slots;        // all groups' prefix slots
   const int32_t* prefix_cu;    // [G+1] device
   const int32_t* group_req_cu; // [G+1] device
+  int req_shift;               // request indices of group_req_cu are shifted left by this (1: every request is two rows)
   int fixed_prefix_len;        // used when prefix_cu is null: one group, all requests, slots[0 .. len)
   int split_tokens;            // tokens per split (multiple of the tile)
   int n_splits;                // parts [0, n_splits)

@@ -395,8 +395,8 @@ __global__ __launch_bounds__(256, 1) void prefix_mfma_kernel(PrefixArgs a, int m
   const int g = blockIdx.z / mtiles, mt = blockIdx.z - g * mtiles;
   int r0 = 0, r1 = a.B, poff = 0, plen = a.fixed_prefix_len;
   if (a.prefix_cu) {
-    r0 = a.group_req_cu[g];
-    r1 = a.group_req_cu[g + 1];
+    r0 = a.group_req_cu[g] << a.req_shift;
+    r1 = a.group_req_cu[g + 1] << a.req_shift;
     poff = a.prefix_cu[g];
     plen = a.prefix_cu[g + 1] - poff;
   }
@@ -847,8 +847,8 @@ __device__ __forceinline__ void prefix_unit8(const PrefixArgs& a, int split, int
   const int g = z / mtiles, mt = z - g * mtiles;
   int r0 = 0, r1 = a.B, poff = 0, plen = a.fixed_prefix_len;
   if (a.prefix_cu) {
-    r0 = a.group_req_cu[g];
-    r1 = a.group_req_cu[g + 1];
+    r0 = a.group_req_cu[g] << a.req_shift;
+    r1 = a.group_req_cu[g + 1] << a.req_shift;
     poff = a.prefix_cu[g];
     plen = a.prefix_cu[g + 1] - poff;
   }

@@ -340,27 +340,26 @@ def test_prefix_longer_than_slot_window(dev):
     _check(case, dev)
 
 
-def _split_halves_case(dtype, B, P, H, seed):
+def _split_halves_case(dtype, B, P, H, seed, D=128):
     from parrotserve_amd import synth
 
     g = torch.Generator().manual_seed(seed)
     s = torch.randint(1, 150, (B,), generator=g).tolist()
     s[0] = 0 if B > 1 else s[0]  # one request without a suffix
-    return synth.make_decode_case("halves", seed, dtype, 1, B, P, s, H, 128, 1 << 14)
+    return synth.make_decode_case("halves", seed, dtype, 1, B, P, s, H, D, 1 << 14)
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("B,P,H", [(64, 700, 8), (20, 333, 4)])
-def test_prefix_and_post_entry_points(dev, dtype, B, P, H):
+@pytest.mark.parametrize("B,P,H,D", [(64, 700, 8, 128), (20, 333, 4, 128), (40, 500, 6, 64), (7, 129, 3, 64)])
+def test_prefix_and_post_entry_points(dev, dtype, B, P, H, D):
     """The two halves exported separately, called through the C ABI the way the reference calls its Triton
     prefix kernel (O, row max and denominator out) and then its post kernel (suffix + merge in place)."""
     import ctypes
 
     from parrotserve_amd import _lib, kernels, synth
 
-    case = _split_halves_case(dtype, B, P, H, 40 + B)
+    case = _split_halves_case(dtype, B, P, H, 40 + B, D)
     lib = _lib.load()
-    D = 128
     kc, vc = synth.pool_to_device(case.k_rows, case.v_rows, case.used_slots, case.pool_slots, dev)
     q = case.q.to(dev)
     out = torch.zeros_like(q)
@@ -616,12 +615,24 @@ def test_captured_decode_step_replays_while_contexts_grow(dev):
 def test_randomized_grouped_decode_shapes(dev, seed):
     """Seeded random batches: 1-3 prefix groups of 1-140 requests, prefixes of 1-1500 tokens (not multiples of
     any tile size), suffixes of 0-90 tokens, odd head counts, a few ungrouped requests, both element types."""
+    _random_grouped_case(dev, seed, 128)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_randomized_grouped_decode_shapes_head_size_64(dev, seed):
+    """The same batches with 64-wide heads: even head counts run the prefix phase on head pairs through the
+    128-wide matrix-core kernel (twice the rows, so groups of up to 140 requests cover every tile size and more
+    than one tile), odd head counts take the per-request kernel."""
+    _random_grouped_case(dev, seed, 64)
+
+
+def _random_grouped_case(dev, seed, D):
     from parrotserve_amd import kernels
 
     g = torch.Generator().manual_seed(1000 + seed)
     ri = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))  # noqa: E731
     dtype = torch.float16 if seed % 2 == 0 else torch.bfloat16
-    H, D = ri(1, 9), 128
+    H = ri(1, 9)
     n_groups = ri(1, 3)
     sizes = [ri(1, 140) if i == 0 else ri(1, 50) for i in range(n_groups)]
     plens = [ri(1, 1500) for _ in range(n_groups)]
