@@ -257,9 +257,24 @@ def head_size_64_step(torch, dev):
     o = torch.empty_like(q)
     t = _time_gpu(torch, lambda: kernels.decode_attention(q, kc, vc, tables, out=o))
     nbytes = 2 * (P + sum(s)) * H * D * 2
-    return {"batch": B, "prefix": P, "sum_suffix": sum(s), "heads": H, "head_dim": D, "us": t * 1e6,
-            "GB/s": nbytes / t / 1e9, "frac_hbm": nbytes / t / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": nbytes,
-            "tokens/s/layer": B / t}
+    res = {"batch": B, "prefix": P, "sum_suffix": sum(s), "heads": H, "head_dim": D, "us": t * 1e6,
+           "GB/s": nbytes / t / 1e9, "frac_hbm": nbytes / t / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": nbytes,
+           "tokens/s/layer": B / t}
+    del kc, vc
+    # config 4's chunks (16 x U[64,1024] new tokens over 2048-token parents, bf16) at 40 x 64: every head runs as one
+    # half of a head pair on the 128-wide prefill kernel
+    c4 = synth.config4()
+    p4 = synth.make_prefill_case("C4-64", 3, torch.bfloat16, c4.q_lens, 2048, 40, 64, 1 << 18)
+    kc4, vc4 = synth.pool_to_device(p4.k_rows, p4.v_rows, p4.used_slots, p4.pool_slots, dev)
+    ctx = [p4.used_slots[torch.cat([a, b])].tolist() for a, b in zip(p4.parent_lists, p4.new_lists)]
+    tab = kernels.PrefillTables.build(p4.q_lens, ctx, dev)
+    q4 = p4.q.to(dev)
+    o4 = torch.empty_like(q4)
+    tp = _time_gpu(torch, lambda: kernels.prefill_attention(q4, kc4, vc4, tab, out=o4), iters=10, inner=5)
+    flops = 4 * 40 * 64 * sum(n * 2048 + n * (n + 1) // 2 for n in p4.q_lens)
+    res["prefill_c4_chunks_40x64"] = {"tokens": int(sum(p4.q_lens)), "ms": tp * 1e3, "flops": flops,
+                                      "TFLOP/s": flops / tp / 1e12}
+    return res
 
 
 def sampler_cost(torch, dev):

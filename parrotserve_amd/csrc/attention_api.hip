@@ -652,7 +652,8 @@ extern "C" size_t ph_prefill_workspace_bytes(int64_t num_tokens, int64_t num_hea
                                              int64_t max_kv_len) {
   if (num_tokens <= 0 || num_heads <= 0 || head_dim <= 0) return 0;
   const DecodePlan p = plan_decode(num_tokens, num_heads, 0, 0, max_kv_len, 0);
-  if (prefix_mfma_supported(PH_F16, (int)head_dim)) return 256 + (size_t)round_up((num_tokens + 2) * 4, 256);
+  if (prefix_mfma_supported(PH_F16, (int)head_dim) || pair_heads(head_dim, num_heads))
+    return 256 + (size_t)round_up((num_tokens + 2) * 4, 256);
   return (size_t)round_up(num_tokens * 8, 256) + (size_t)round_up(num_tokens * 4, 256) +
          plan_bytes(p, num_tokens, num_heads, head_dim);
 }
@@ -673,7 +674,8 @@ extern "C" int ph_prefill_attention(void* out, const void* q, const void* k_cach
     return PH_ERR_WORKSPACE;
   if (((uintptr_t)workspace & 255u) != 0) return PH_ERR_ALIGN;
   hipStream_t st = (hipStream_t)stream;
-  if (prefix_mfma_supported(dtype, D)) {
+  const bool paired = pair_heads(D, H) && prefix_mfma_supported(dtype, 128);  // 64-wide heads as halves of head pairs
+  if (prefix_mfma_supported(dtype, D) || paired) {
     if (num_chunks > num_tokens) return PH_ERR_ARG;  // every chunk holds at least one query (tile_cu fits the workspace)
     PrefillArgs pa{};
     pa.q = (const uint16_t*)q;
@@ -690,7 +692,8 @@ extern "C" int ph_prefill_attention(void* out, const void* q, const void* k_cach
     pa.num_chunks = (int)num_chunks;
     pa.H = H;
     pa.scale_log2e = scale * kLog2e;
-    return launch_prefill_mfma(pa, dtype, D, num_tokens, st);
+    pa.pair = paired ? 1 : 0;
+    return launch_prefill_mfma(pa, dtype, paired ? 128 : D, num_tokens, st);
   }
   int64_t* offsets = (int64_t*)workspace;
   int32_t* lens = (int32_t*)((char*)workspace + round_up(num_tokens * 8, 256));

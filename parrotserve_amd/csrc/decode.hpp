@@ -107,6 +107,7 @@ struct PrefillArgs {
   int num_chunks;
   int H;
   float scale_log2e;
+  int pair;                  // 1: heads are 64 wide and run as halves of 128-wide head pairs (q, out, caches [.., H, 64])
 };
 
 int launch_partial(const PartialArgs& a, int dtype, int D, hipStream_t st);

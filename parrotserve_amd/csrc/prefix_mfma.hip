@@ -93,6 +93,7 @@ struct TileWork {
   int slots_len;          // entries of the list (reads beyond [s0, s1) are clamped to it)
   int s0, s1;             // token range of this workgroup
   int causal_off;         // CAUSAL: query i sees token t iff t <= causal_off + i
+  int pair_half = -1;     // 0 / 1: the query is 64 wide and fills that half of the 128-wide row, the other half is zero
 };
 
 // Runs the tile on all four waves.  On return wave w holds, for the 32 dims [32w, 32w+32) of every
@@ -586,10 +587,14 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
     const int q = 32 * qb + ql;
     const bool ok = q < wk.nq;
     const uint16_t* qp = wk.qrow0 + (int64_t)(ok ? q : 0) * wk.q_stride + 64 * h;
+    // a 64-wide head as one half of a head pair: the other half of the query is zero, which cancels the
+    // neighbouring head's keys in the score (the row pointer already points at this half's 64 values)
+    const bool mine = wk.pair_half < 0 || h == wk.pair_half;
+    if (wk.pair_half >= 0) qp = wk.qrow0 + (int64_t)(ok ? q : 0) * wk.q_stride;
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
       u32x4 v = ld16(qp + 8 * s);
-      if (!ok) v = u32x4{0, 0, 0, 0};
+      if (!ok || !mine) v = u32x4{0, 0, 0, 0};
       qop[s] = v;
     }
   }
@@ -959,8 +964,10 @@ template <typename E, int TQ, int SUB>
 __global__ __launch_bounds__(512) void prefill_mfma8_kernel(PrefillArgs a) {
   constexpr int QB = 8 / TQ, NDB = 4 / TQ, QT = 32 * QB;
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  const int head = blockIdx.x;
-  if (head >= a.H) return;
+  if ((int)blockIdx.x >= a.H) return;
+  // 64-wide heads: workgroup x is head x = half (x & 1) of pair x >> 1, whose K/V rows are one 128-wide row
+  const int head = a.pair ? blockIdx.x >> 1 : blockIdx.x;
+  const int half = a.pair ? (int)(blockIdx.x & 1) : -1;
   if ((int)blockIdx.y >= a.tile_cu[a.num_chunks]) return;
   // later tiles of a chunk see more keys: hand them out first so the launch does not end on the longest ones
   const int ti = a.tile_cu[a.num_chunks] - 1 - blockIdx.y;
@@ -974,7 +981,8 @@ __global__ __launch_bounds__(512) void prefill_mfma8_kernel(PrefillArgs a) {
   const int q0 = (ti - a.tile_cu[lo]) * QT;
   const int nq = min(QT, n - q0);
   TileWork wk;
-  wk.qrow0 = a.q + (int64_t)(cq0 + q0) * a.q_stride + head * kPD;
+  wk.qrow0 = a.q + (int64_t)(cq0 + q0) * a.q_stride + (a.pair ? (int)blockIdx.x * 64 : head * kPD);
+  wk.pair_half = half;
   wk.q_stride = a.q_stride;
   wk.nq = nq;
   wk.slots = a.ctx_slots + kv0;
@@ -991,7 +999,11 @@ __global__ __launch_bounds__(512) void prefill_mfma8_kernel(PrefillArgs a) {
     const float inv = l > 0.f ? 1.f / l : 0.f;
 #pragma unroll
     for (int nd = 0; nd < NDB; ++nd) {
-      uint16_t* op = a.out + (int64_t)(cq0 + q0 + q) * a.out_stride + head * kPD + 32 * (NDB * g + nd) + 4 * h;
+      const int db = NDB * g + nd;  // 32-dim block of the 128-wide row
+      if (a.pair && (db >> 1) != half) continue;  // the other half holds the neighbouring head's values: dropped
+      // paired: head 2 * pair + half, dims 32 * (db & 1) ..; else head, dims 32 * db ..
+      uint16_t* op = a.out + (int64_t)(cq0 + q0 + q) * a.out_stride +
+                     (a.pair ? (int)blockIdx.x * 64 + 32 * (db & 1) : head * kPD + 32 * db) + 4 * h;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         u32x2 v = {pack2<E>(of[nd][4 * j] * inv, of[nd][4 * j + 1] * inv),

@@ -137,7 +137,7 @@ def test_prefill_heads_not_multiple_of_eight_and_tail_tiles(dev):
         torch.testing.assert_close(out.float(), ref.float(), **TOL[torch.bfloat16])
 
 
-@pytest.mark.parametrize("D,H", [(64, 6), (256, 2), (80, 5), (96, 3), (112, 2)])
+@pytest.mark.parametrize("D,H", [(64, 6), (64, 5), (256, 2), (80, 5), (96, 3), (112, 2)])
 def test_prefill_other_head_sizes(dev, D, H):
     """Head sizes the matrix-core kernel does not cover run every query row through the per-request kernel
     over its visible slots; same results."""
@@ -148,10 +148,13 @@ def test_prefill_other_head_sizes(dev, D, H):
     torch.testing.assert_close(out.float(), ref.float(), **TOL[torch.float16])
 
 
+@pytest.mark.parametrize("D", [128, 64])
 @pytest.mark.parametrize("seed", range(8))
-def test_randomized_prefill_shapes(dev, seed):
+def test_randomized_prefill_shapes(dev, seed, D):
     """Seeded random chunk sets: 1-6 chunks of 1-400 new tokens over parents of 0-700 tokens, odd head counts,
-    both element types (covers every query-tile size and partial tiles on both axes)."""
+    both element types (covers every query-tile size and partial tiles on both axes).  64-wide heads run as
+    halves of head pairs on the same matrix-core kernel when the head count is even, through the per-request
+    kernel when it is odd."""
     from parrotserve_amd import synth
 
     g = torch.Generator().manual_seed(2000 + seed)
@@ -160,6 +163,6 @@ def test_randomized_prefill_shapes(dev, seed):
     chunks = ri(1, 6)
     hi = [30, 120, 400][seed % 3]
     q_lens = [ri(1, hi) for _ in range(chunks)]
-    case = synth.make_prefill_case("rnd", 2000 + seed, dtype, q_lens, ri(0, 700), ri(1, 6), 128, 1 << 13)
+    case = synth.make_prefill_case("rnd", 2000 + seed, dtype, q_lens, ri(0, 700), ri(1, 6), D, 1 << 13)
     out, ref = run_prefill_case(case, dev)
     torch.testing.assert_close(out.float(), ref.float(), **TOL[dtype])
