@@ -103,9 +103,8 @@ static size_t plan_bytes(const DecodePlan& p, int64_t B, int64_t H, int64_t D) {
   size_t n = round_up((int64_t)(rows * D * sizeof(float)), 256) + round_up((int64_t)(rows * 2 * sizeof(float)), 256);
   if (p.dev_lanes > 0)
     n += round_up(p.items * 16, 256) + round_up((int64_t)p.dev_lanes * 32, 256) + round_up((B + 1) * 4, 256);
-  if (p.paired)  // the widened query rows, and the head-pair partials of the prefix parts
-    n += round_up(B * H * 128 * 2, 256) + round_up((int64_t)p.n_splits * B * H * 128 * 4, 256) +
-         round_up((int64_t)p.n_splits * B * H * 2 * 4, 256);
+  if (p.paired)  // the head-pair partials of the prefix parts
+    n += round_up((int64_t)p.n_splits * B * H * 128 * 4, 256) + round_up((int64_t)p.n_splits * B * H * 2 * 4, 256);
   return n;
 }
 
@@ -113,8 +112,7 @@ struct Carve {
   float* opart;
   float* ml;
   int32_t *items, *lane_rec, *req_item_cu;  // the device-built plan (dev_lanes > 0)
-  uint16_t* q_pairs;                        // paired prefix phase: [2B][H/2][128] queries,
-  float *opart_pairs, *ml_pairs;            // [n_splits][2B][H/2] partial rows of 128 floats / (m, l)
+  float *opart_pairs, *ml_pairs;            // paired prefix phase: [n_splits][2B][H/2] partial rows of 128 floats / (m, l)
 };
 static Carve carve(void* ws, const DecodePlan& p, int64_t B, int64_t H, int64_t D) {
   const size_t rows = p.rows(B, H);
@@ -133,8 +131,6 @@ static Carve carve(void* ws, const DecodePlan& p, int64_t B, int64_t H, int64_t 
     at += round_up((B + 1) * 4, 256);
   }
   if (p.paired) {
-    c.q_pairs = (uint16_t*)at;
-    at += round_up(B * H * 128 * 2, 256);
     c.opart_pairs = (float*)at;
     at += round_up((int64_t)p.n_splits * B * H * 128 * 4, 256);
     c.ml_pairs = (float*)at;
@@ -143,28 +139,11 @@ static Carve carve(void* ws, const DecodePlan& p, int64_t B, int64_t H, int64_t 
 }
 
 // D == 64 with an even head count: two adjacent heads of a token row are one 128-wide row of the matrix-core
-// kernel.  Request b, head 2p + s becomes row 2b + s, pseudo-head p, whose query is the head's 64 values in
-// half s and zeros in the other half: the zeros cancel the neighbour's keys in the score, and half s of the
+// kernel.  Request b, head 2p + s becomes row 2b + s, pseudo-head p, whose query (as the kernel loads it) is the
+// head's 64 values in half s and zeros in the other half: the zeros cancel the neighbour's keys in the score, and half s of the
 // 128-wide output is exactly the head's output (the other half, the neighbour's values under this head's
 // weights, is ignored).  Twice the matrix work, the same K/V traffic -- read once per group, not once per request.
 static bool pair_heads(int64_t D, int64_t H) { return D == 64 && H % 2 == 0; }
-
-__global__ __launch_bounds__(256) void widen_queries_kernel(const uint16_t* __restrict__ q, int64_t q_stride,
-                                                            uint16_t* __restrict__ q2, int B, int H) {
-  // one 16-byte chunk per thread: 16 chunks per (row, pseudo-head), chunks 8s .. 8s+7 carry the head's values
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  const int64_t total = (int64_t)2 * B * (H / 2) * 16;
-  if (i >= total) return;
-  const int c = (int)(i & 15);
-  const int64_t rp = i >> 4;
-  const int p = (int)(rp % (H / 2));
-  const int64_t row = rp / (H / 2);
-  const int s = (int)(row & 1);
-  const int64_t b = row >> 1;
-  u32x4 v = {0u, 0u, 0u, 0u};
-  if ((c >> 3) == s) v = ld16(q + b * q_stride + (int64_t)(2 * p + s) * 64 + (c & 7) * 8);
-  st16(q2 + i * 8, v);
-}
 
 static int check_common(const void* out, const void* q, const void* kc, const void* vc, int64_t B, int64_t H,
                         int64_t D, int dtype, int64_t q_stride, int64_t out_stride, int64_t row_stride) {
@@ -182,23 +161,21 @@ static int check_common(const void* out, const void* q, const void* kc, const vo
 
 // Prefix phase: matrix-core kernel for head size 128; other head sizes run the
 // per-request gather kernel once per group over the shared slot list.
+// the prefix phase's arguments as the 128-wide kernel sees them when 64-wide heads run as head pairs
+static PrefixArgs pair_args(const PrefixArgs& pa, const Carve& ws) {
+  PrefixArgs w = pa;
+  w.B = 2 * pa.B;
+  w.H = pa.H / 2;
+  w.req_shift = 1;
+  w.opart = ws.opart_pairs;
+  w.ml = ws.ml_pairs;
+  return w;
+}
+
 static int run_prefix(PrefixArgs& pa, int dtype, int D, int num_groups, const int32_t* group_req_cu_host,
                       int max_group_reqs, hipStream_t st, const Carve* pairs = nullptr) {
-  if (pairs && pairs->q_pairs) {
-    const int64_t chunks = (int64_t)2 * pa.B * (pa.H / 2) * 16;
-    hipLaunchKernelGGL(widen_queries_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, st, pa.q, pa.q_stride,
-                       pairs->q_pairs, pa.B, pa.H);
-    if (launch_status() != PH_OK) return PH_ERR_LAUNCH;
-    PrefixArgs w = pa;
-    w.q = pairs->q_pairs;
-    w.q_stride = (int64_t)(pa.H / 2) * 128;
-    w.B = 2 * pa.B;
-    w.H = pa.H / 2;
-    w.req_shift = 1;
-    w.opart = pairs->opart_pairs;
-    w.ml = pairs->ml_pairs;
-    return launch_prefix_mfma(w, dtype, 128, num_groups, 2 * max_group_reqs, st);
-  }
+  if (pairs && pairs->opart_pairs)
+    return launch_prefix_mfma(pair_args(pa, *pairs), dtype, 128, num_groups, 2 * max_group_reqs, st);
   if (prefix_mfma_supported(dtype, D)) return launch_prefix_mfma(pa, dtype, D, num_groups, max_group_reqs, st);
   int rc = launch_clear_ml(pa.ml, (int64_t)pa.n_splits * pa.B * pa.H, st);
   if (rc != PH_OK) return rc;
@@ -364,11 +341,12 @@ extern "C" int ph_decode_attention(void* out, const void* q, const void* k_cache
     pa.B = B;
     pa.H = H;
     pa.scale_log2e = sl2;
-    fuse = planned && decode_fused_supported(dtype, D, max_group_reqs);
+    fuse = planned && (paired ? decode_fused_supported(dtype, 128, 2 * max_group_reqs)
+                              : decode_fused_supported(dtype, D, max_group_reqs));
     if (fuse) {
-      fused_pa = pa;
+      fused_pa = paired ? pair_args(pa, ws) : pa;
       fused_groups = (int)num_groups;
-      fused_max_reqs = max_group_reqs;
+      fused_max_reqs = paired ? 2 * max_group_reqs : max_group_reqs;
     } else {
       rc = run_prefix(pa, dtype, D, (int)num_groups, group_req_cu_host, max_group_reqs, st, paired ? &ws : nullptr);
       if (rc != PH_OK) return rc;

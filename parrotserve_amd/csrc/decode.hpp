@@ -82,7 +82,8 @@ struct PrefixArgs {
   const int32_t* slots;        // all groups' prefix slots
   const int32_t* prefix_cu;    // [G+1] device
   const int32_t* group_req_cu; // [G+1] device
-  int req_shift;               // request indices of group_req_cu are shifted left by this (1: every request is two rows)
+  int req_shift;               // 1: 64-wide heads on head pairs -- B counts rows (two per request: row 2b + s is
+                               // request b, half s), H head pairs, q is the real [B][2 H][64] tensor
   int fixed_prefix_len;        // used when prefix_cu is null: one group, all requests, slots[0 .. len)
   int split_tokens;            // tokens per split (multiple of the tile)
   int n_splits;                // parts [0, n_splits)

@@ -93,7 +93,10 @@ struct TileWork {
   int slots_len;          // entries of the list (reads beyond [s0, s1) are clamped to it)
   int s0, s1;             // token range of this workgroup
   int causal_off;         // CAUSAL: query i sees token t iff t <= causal_off + i
-  int pair_half = -1;     // 0 / 1: the query is 64 wide and fills that half of the 128-wide row, the other half is zero
+  // 64-wide heads as halves of 128-wide head pairs (the query's other half is zero):
+  //   0 / 1: every row of the tile is that half, qrow0 points at the half's 64 values;
+  //   2: rows alternate, row q = request q >> 1 (rows of q_stride from qrow0, the pair's first value), half q & 1
+  int pair_half = -1;
 };
 
 // Runs the tile on all four waves.  On return wave w holds, for the 32 dims [32w, 32w+32) of every
@@ -589,8 +592,14 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
     const uint16_t* qp = wk.qrow0 + (int64_t)(ok ? q : 0) * wk.q_stride + 64 * h;
     // a 64-wide head as one half of a head pair: the other half of the query is zero, which cancels the
     // neighbouring head's keys in the score (the row pointer already points at this half's 64 values)
-    const bool mine = wk.pair_half < 0 || h == wk.pair_half;
-    if (wk.pair_half >= 0) qp = wk.qrow0 + (int64_t)(ok ? q : 0) * wk.q_stride;
+    int half = wk.pair_half;
+    if (wk.pair_half == 2) {  // rows alternate between the two heads of the pair: row q = request q >> 1, half q & 1
+      half = q & 1;
+      qp = wk.qrow0 + (int64_t)(ok ? q >> 1 : 0) * wk.q_stride + 64 * half;
+    } else if (wk.pair_half >= 0) {
+      qp = wk.qrow0 + (int64_t)(ok ? q : 0) * wk.q_stride;
+    }
+    const bool mine = wk.pair_half < 0 || h == half;
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
       u32x4 v = ld16(qp + 8 * s);
@@ -875,7 +884,9 @@ __device__ __forceinline__ void prefix_unit8(const PrefixArgs& a, int split, int
     return;
   }
   TileWork wk;
-  wk.qrow0 = a.q + (int64_t)qbase * a.q_stride + head * kPD;
+  // req_shift == 1: B and H count rows (two per request) and head pairs; q is the real [B][2 H][64] tensor
+  wk.qrow0 = a.q + (int64_t)(qbase >> a.req_shift) * a.q_stride + head * kPD;
+  wk.pair_half = a.req_shift ? 2 : -1;
   wk.q_stride = a.q_stride;
   wk.nq = nq;
   wk.slots = a.slots + poff;
@@ -921,10 +932,11 @@ __global__ __launch_bounds__(512) void prefix_mfma8_kernel(PrefixArgs a, int mti
 // more), then the prefix main loop on tiles that landed long ago, then the fold.  Against two launches this
 // removes one launch, hides the prefix prologue behind the suffix stream and keeps the memory system busy
 // from the first microseconds.  The merge stays a separate launch: it needs every part.
-template <typename E, int TQ>
+// DS = head size of the suffix phase: 128, or 64 when the prefix phase runs on head pairs (pa.req_shift == 1).
+template <typename E, int TQ, int DS = kPD>
 __global__ __launch_bounds__(512) void decode_fused_kernel(PrefixArgs pa, int mtiles, int n_units, ItemArgs ia) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  constexpr int HPW = kWave / (kPD / 8);
+  constexpr int HPW = HeadLanes<DS>::HPW;
   const int hgroups = (ia.H + HPW - 1) / HPW;
   const int slots = ia.num_lanes * hgroups;
   const int wave = __builtin_amdgcn_readfirstlane(blockIdx.x * 8 + (threadIdx.x >> 6));
@@ -936,10 +948,10 @@ __global__ __launch_bounds__(512) void decode_fused_kernel(PrefixArgs pa, int mt
     rec1 = ia.lane_rec[2 * piece0 + 1];
   }
   auto suffix = [&]() {
-    if (piece0 >= 0) run_piece_rec<E, kPD, 4, 2>(ia, wave - piece0 * hgroups, rec0, rec1);
+    if (piece0 >= 0) run_piece_rec<E, DS, 4, 2>(ia, wave - piece0 * hgroups, rec0, rec1);
     for (int s = wave + gridDim.x * 8; s < slots; s += gridDim.x * 8) {
       const int piece = s / hgroups;
-      run_piece<E, kPD, 4, 2>(ia, piece, s - piece * hgroups);
+      run_piece<E, DS, 4, 2>(ia, piece, s - piece * hgroups);
     }
   };
   if ((int)blockIdx.x < n_units) {
@@ -1039,7 +1051,7 @@ static void launch_prefix8(const PrefixArgs& a, int num_groups, int max_group_re
 template <typename E>
 static int launch_prefix_t(const PrefixArgs& a, int num_groups, int max_group_reqs, hipStream_t st) {
   const KernelEvents ev = take_kernel_events(0);
-  if (max_group_reqs <= 32) {  // four waves, one 32-query block
+  if (max_group_reqs <= 32 && a.req_shift == 0) {  // four waves, one 32-query block
     dim3 grid(a.n_splits, a.H, num_groups), block(256);
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefix_mfma_kernel<E, 1>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, tile_lds_bytes<1>());
@@ -1076,33 +1088,34 @@ static int launch_prefill_t(const PrefillArgs& a, int64_t num_tokens, hipStream_
   return launch_prefill_tq<E, 4, 1>(a, num_tokens, st);
 }
 
-template <typename E, int TQ>
+template <typename E, int TQ, int DS>
 static int launch_fused_tq(const PrefixArgs& a, const ItemArgs& ia, int num_groups, int max_group_reqs, int cus,
                            hipStream_t st) {
   constexpr int QT = 32 * (8 / TQ);
+  constexpr int HPW = HeadLanes<DS>::HPW;
   const int mtiles = (max_group_reqs + QT - 1) / QT;
   const int n_units = a.n_splits * a.H * num_groups * mtiles;
-  const int hgroups = (ia.H + 3) / 4;
+  const int hgroups = (ia.H + HPW - 1) / HPW;
   const int wave_slots = ia.num_lanes * hgroups;
   int grid = (wave_slots + 7) / 8;
   const int unit_grid = n_units < cus ? n_units : cus;
   if (grid < unit_grid) grid = unit_grid;
   if (grid <= 0) return PH_OK;
-  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&decode_fused_kernel<E, TQ>),
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&decode_fused_kernel<E, TQ, DS>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, kTile8Lds);
   const KernelEvents ev = take_kernel_events(1);
-  PH_LAUNCH_TIMED((decode_fused_kernel<E, TQ>), dim3(grid), dim3(512), kTile8Lds, st, ev, a, mtiles,
+  PH_LAUNCH_TIMED((decode_fused_kernel<E, TQ, DS>), dim3(grid), dim3(512), kTile8Lds, st, ev, a, mtiles,
                         n_units, ia);
   return launch_status();
 }
 
 // query tile by the largest group: 64, 128 or 256 requests share each K/V tile of the prefix
-template <typename E>
+template <typename E, int DS>
 static int launch_fused_t(const PrefixArgs& a, const ItemArgs& ia, int num_groups, int max_group_reqs, int cus,
                           hipStream_t st) {
-  if (max_group_reqs <= 64) return launch_fused_tq<E, 4>(a, ia, num_groups, max_group_reqs, cus, st);
-  if (max_group_reqs <= 128) return launch_fused_tq<E, 2>(a, ia, num_groups, max_group_reqs, cus, st);
-  return launch_fused_tq<E, 1>(a, ia, num_groups, max_group_reqs, cus, st);
+  if (max_group_reqs <= 64) return launch_fused_tq<E, 4, DS>(a, ia, num_groups, max_group_reqs, cus, st);
+  if (max_group_reqs <= 128) return launch_fused_tq<E, 2, DS>(a, ia, num_groups, max_group_reqs, cus, st);
+  return launch_fused_tq<E, 1, DS>(a, ia, num_groups, max_group_reqs, cus, st);
 }
 
 // One launch for the prefix and suffix phases: head size 128, groups of more than 32 requests (the
@@ -1113,8 +1126,12 @@ bool decode_fused_supported(int dtype, int D, int max_group_reqs) {
 
 int launch_decode_fused(const PrefixArgs& a, const ItemArgs& ia, int dtype, int num_groups, int max_group_reqs, int cus,
                         hipStream_t st) {
-  return dtype == PH_F16 ? launch_fused_t<F16>(a, ia, num_groups, max_group_reqs, cus, st)
-                         : launch_fused_t<BF16>(a, ia, num_groups, max_group_reqs, cus, st);
+  if (a.req_shift) {  // 64-wide heads: the prefix phase on head pairs, the suffix phase at its own width
+    return dtype == PH_F16 ? launch_fused_t<F16, 64>(a, ia, num_groups, max_group_reqs, cus, st)
+                           : launch_fused_t<BF16, 64>(a, ia, num_groups, max_group_reqs, cus, st);
+  }
+  return dtype == PH_F16 ? launch_fused_t<F16, kPD>(a, ia, num_groups, max_group_reqs, cus, st)
+                         : launch_fused_t<BF16, kPD>(a, ia, num_groups, max_group_reqs, cus, st);
 }
 
 bool prefix_mfma_supported(int dtype, int D) { return D == kPD && (dtype == PH_F16 || dtype == PH_BF16); }
