@@ -92,9 +92,10 @@ class IterationTables:
 
 def build_iteration_tables(jobs: Sequence[Any], grouping: str = "lca") -> IterationTables:
     """``grouping="lca"``: one prefix shared by every job of the iteration, the
-    reference's rule.  ``grouping="parent"``: Generate jobs forked from the same
-    parent context form a group whose prefix is that parent's whole context, so
-    several prompt groups can share the iteration."""
+    reference's rule.  ``grouping="parent"``: Generate jobs that descend from a common
+    context form a group whose prefix is that context's whole chain -- the deepest
+    such context per job, so several prompt groups can share the iteration and a
+    batch the reference's rule covers gets the same prefix from it."""
     assert grouping in ("lca", "parent")
     P = get_shared_context_len(jobs) if grouping == "lca" else 0
     slots0 = jobs[0].context.get_context_slot_ids() if P > 0 else []
@@ -119,11 +120,10 @@ def build_iteration_tables(jobs: Sequence[Any], grouping: str = "lca") -> Iterat
                 gen_full.append(slots)
                 t.slot_mapping.append(slots[-1])
             else:
-                # the parent's list is taken once per group below, not copied into every job's list
-                own = list(job.context.token_kv_block_ids)
-                gen_own.append(own)
+                # an ancestor's list is taken once per group below, not copied into every job's list
+                gen_own.append(job.context)
                 gen_parent.append(job.context.parent_context)
-                t.slot_mapping.append(own[-1])
+                t.slot_mapping.append(job.context.token_kv_block_ids[-1])
         else:
             raise TypeError(f"unknown job type {type(job)}")
     if grouping == "lca":
@@ -133,21 +133,49 @@ def build_iteration_tables(jobs: Sequence[Any], grouping: str = "lca") -> Iterat
         if P > 0 and gen_full:
             t.groups.append((t.flash_block_table, list(range(len(gen_full)))))
     else:
-        by_parent: Dict[int, int] = {}
-        for i, (own, parent) in enumerate(zip(gen_own, gen_parent)):
-            t.paged_block_tables.append(own)
-            t.paged_context_lens.append(len(own))
-            if parent is None:
-                continue
-            g = by_parent.get(id(parent))
-            if g is None:
-                prefix = parent.get_context_slot_ids()
-                if not prefix:
-                    continue
-                by_parent[id(parent)] = len(t.groups)
-                t.groups.append((prefix, [i]))
+        # A job's group is the deepest ancestor context that at least two Generate jobs of the iteration descend
+        # from (its fork parent when siblings decode together; a grandparent when every job sits under a
+        # context of its own, as in tests/engine/builtin/test_shared_prefix.py:57-115 of the reference); the
+        # group's prefix is that ancestor's whole context, a job's own list everything below it.
+        below: Dict[int, int] = {}
+        for parent in gen_parent:
+            c = parent
+            while c is not None:
+                below[id(c)] = below.get(id(c), 0) + 1
+                c = c.parent_context
+        by_anchor: Dict[int, int] = {}
+        for i, (ctx, parent) in enumerate(zip(gen_own, gen_parent)):
+            own = [ctx.token_kv_block_ids]
+            anchor = parent
+            while anchor is not None and below[id(anchor)] < 2:
+                own.append(anchor.token_kv_block_ids)
+                anchor = anchor.parent_context
+            g = None
+            if anchor is not None:
+                g = by_anchor.get(id(anchor))
+                if g is None:
+                    prefix = anchor.get_context_slot_ids()
+                    if prefix:
+                        g = by_anchor[id(anchor)] = len(t.groups)
+                        t.groups.append((prefix, []))
+                    else:
+                        by_anchor[id(anchor)] = g = -1
+                if g < 0:
+                    g = None
+            if g is None:  # nothing shared: the whole context is the job's own list
+                slots = ctx.get_context_slot_ids()
             else:
                 t.groups[g][1].append(i)
+                slots = [s for part in reversed(own) for s in part]
+            t.paged_block_tables.append(slots)
+            t.paged_context_lens.append(len(slots))
+        # a group that ended up with a single member (its siblings found a deeper anchor) shares nothing
+        for prefix, members in t.groups:
+            if len(members) == 1:
+                i = members[0]
+                t.paged_block_tables[i] = prefix + t.paged_block_tables[i]
+                t.paged_context_lens[i] = len(t.paged_block_tables[i])
+        t.groups = [gm for gm in t.groups if len(gm[1]) > 1]
     return t
 
 

@@ -92,3 +92,64 @@ def test_shared_prompt_generation_loop_matches_flat_oracle(dev, attn_func, fused
                 assert produced[s] == int(top2.indices[0])
     assert clear >= B * output_len // 2  # the margin filter must not hollow out the token check
     cfg.attn_func.table_cache.clear()
+
+
+@pytest.mark.parametrize("attn_func", ["xformers_fill_shared_prompts_generate", "hip_shared_prefix"])
+def test_two_level_shared_prompts_match_flat_oracle(dev, attn_func):
+    """The reference's two-level scenario (tests/engine/builtin/test_shared_prefix.py:57-115), small: a context, a child
+    of it, B Fills of different lengths forked from the child, and every Generate job in a fresh context under its own
+    Fill's context -- so no two jobs share a fork parent, and what they share is the grandparent chain.  Hidden
+    states and tokens against the flat-sequence oracle; the grouped plug-in must find the same shared prefix as the
+    reference's rule (the chain of the two upper contexts)."""
+    from parrotserve_amd.attn_func import BuiltinConfig, build_iteration_tables
+    from parrotserve_amd.primitive_job import Fill, Generate
+    from parrotserve_amd.runner import BuiltinRunner, LlamaConfig, SamplingConfig
+
+    V, N, H, L, Fdim = 211, 256, 2, 2, 384
+    B, len1, len2, output_len = 5, 20, 10, 6
+    mc = LlamaConfig(vocab_size=V, hidden_size=N, intermediate_size=Fdim, num_hidden_layers=L, num_attention_heads=H,
+                     rms_norm_eps=1e-6, max_position_embeddings=256)
+    cfg = BuiltinConfig(num_kv_cache_blocks=2048, attn_func=attn_func, dtype=torch.float16, device=dev)
+    cfg.attn_func.table_cache.clear()
+    runner = BuiltinRunner(mc, cfg, dummy_weights=False)
+    w = _set_weights(runner.model, 9)
+    seen = []
+    runner.model.sampler.register_forward_pre_hook(lambda mod, args: seen.append(args[0].detach().float().cpu()))
+
+    g = torch.Generator().manual_seed(13)
+    top = torch.randint(0, V, (len1,), generator=g).tolist()
+    mid = torch.randint(0, V, (len2,), generator=g).tolist()
+    diverged = [torch.randint(0, V, (3 * (b + 1),), generator=g).tolist() for b in range(B)]
+    sc = SamplingConfig(top_p=1e-6, max_gen_length=output_len)
+    runner.run_iter([Fill(0, 0, 0, -1, token_ids=top)])
+    runner.run_iter([Fill(0, 0, 1, 0, token_ids=mid)])
+    runner.run_iter([Fill(0, 0, b + 2, 1, token_ids=diverged[b]) for b in range(B)])
+    gens = [Generate(0, 0, b + 2 + B, b + 2, sampling_config=sc) for b in range(B)]
+    for it in range(output_len - 1):
+        runner.run_iter(gens)
+        if it == 0:  # both rules see the same 30 shared tokens; the grouped rule puts every job into that one group
+            lca = build_iteration_tables(gens, "lca")
+            par = build_iteration_tables(gens, "parent")
+            assert lca.flash_context_len == len1 + len2
+            assert len(par.groups) == 1 and par.groups[0][0] == lca.flash_block_table
+            assert sorted(par.groups[0][1]) == list(range(B)) and par.paged_block_tables == lca.paged_block_tables
+    assert all(j.finish_event.is_set() and j.gen_length == output_len for j in gens)
+
+    rows = [s for s in seen if s.shape[0] > 0]
+    assert len(rows) == output_len and all(r.shape == (B, N) for r in rows)
+    clear = 0
+    for b, job in enumerate(gens):
+        produced = list(job.output_queue)
+        assert produced == job.context.token_ids and len(produced) == output_len
+        seq = top + mid + diverged[b] + produced
+        hid = ref_llama_hidden(w, seq[:-1], H, 1e-6, cache_dtype=torch.float16)
+        first = len1 + len2 + len(diverged[b]) - 1
+        for s in range(output_len):
+            torch.testing.assert_close(rows[s][b], hid[first + s], atol=3e-2, rtol=3e-2)
+            logits = hid[first + s] @ w["lm_head"].t()
+            top2 = logits.topk(2)
+            if top2.values[0] - top2.values[1] > 0.25:
+                clear += 1
+                assert produced[s] == int(top2.indices[0])
+    assert clear >= B * output_len // 2
+    cfg.attn_func.table_cache.clear()

@@ -316,3 +316,42 @@ def test_forked_fill_tables_grouping_rules():
     # it has to pay: two 12-token chunks read 2 x 78 own pairs for the 80 parent rows they save
     assert forked_fill_tables([fork(pa, 0, 12, 20), fork(pa, 0, 12, 21)], 32, 16) is None
     assert forked_fill_tables([fork(None, 0, 5, 7), fork(None, 0, 5, 8)], 0, 16) is None  # no parent
+
+
+def test_grouping_by_the_deepest_shared_ancestor():
+    """Jobs under contexts of their own share the grandparent chain (the reference's two-level scenario); nested
+    forks group at the lower level; a job nothing is shared with keeps its whole context as its own list."""
+    pool = RecyclePool(pool_size=10000)
+
+    def ctx(cid, parent, n):
+        c = BlockContext(cid, parent, pool, 1)
+        c.allocate(n)
+        return c
+
+    def gen(c):
+        j = Generate(0, c.context_id, c.context_id, -1)
+        j.context = c
+        return j
+
+    top = ctx(0, None, 20)
+    mid = ctx(1, top, 10)
+    fills = [ctx(2 + i, mid, 3 + i) for i in range(4)]
+    jobs = [gen(ctx(10 + i, fills[i], 1)) for i in range(4)]
+    t = build_iteration_tables(jobs, "parent")
+    lca = build_iteration_tables(jobs, "lca")
+    assert lca.flash_context_len == 30
+    assert t.groups == [(lca.flash_block_table, [0, 1, 2, 3])]
+    assert t.paged_block_tables == lca.paged_block_tables
+    assert t.paged_block_tables[2] == fills[2].token_kv_slot_ids + jobs[2].context.token_kv_slot_ids
+    # nested forks: two jobs under fills[0], one under fills[1] -> the pair groups at fills[0] (33 tokens); the
+    # third job would anchor at mid, alone there (its cousins found a deeper anchor), so it shares nothing
+    a, b = gen(ctx(20, fills[0], 2)), gen(ctx(21, fills[0], 1))
+    c = gen(ctx(22, fills[1], 1))
+    t = build_iteration_tables([a, c, b], "parent")
+    assert [len(p) for p, _ in t.groups] == [33] and [m for _, m in t.groups] == [[0, 2]]
+    assert t.paged_context_lens == [2, 30 + 4 + 1, 1]
+    assert t.paged_block_tables[1] == c.context.get_context_slot_ids()
+    # unrelated roots: nothing shared, no group, whole contexts
+    x, y = gen(ctx(30, ctx(31, None, 7), 2)), gen(ctx(32, ctx(33, None, 5), 1))
+    t = build_iteration_tables([x, y], "parent")
+    assert t.groups == [] and t.paged_context_lens == [9, 6]
