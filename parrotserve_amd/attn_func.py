@@ -101,8 +101,8 @@ def build_iteration_tables(jobs: Sequence[Any], grouping: str = "lca") -> Iterat
     slots0 = jobs[0].context.get_context_slot_ids() if P > 0 else []
     t = IterationTables(P, slots0[:P], [], [], [], [], [], [], [], [], [], 0)
     gen_full: List[List[int]] = []    # "lca": every Generate job's whole context
-    gen_own: List[List[int]] = []     # "parent": only what lies beyond the fork parent (the job's own tokens)
-    gen_parent: List[Any] = []
+    gen_own: List[Any] = []           # "parent": every Generate job's context ...
+    gen_parent: List[Any] = []        # ... and its fork parent
     for job in jobs:
         if isinstance(job, Fill):
             slots = job.context.get_context_slot_ids()
