@@ -153,3 +153,45 @@ def test_two_level_shared_prompts_match_flat_oracle(dev, attn_func):
                 assert produced[s] == int(top2.indices[0])
     assert clear >= B * output_len // 2
     cfg.attn_func.table_cache.clear()
+
+
+@pytest.mark.parametrize("attn_func", ["xformers_with_buffer", "hip_shared_prefix"])
+def test_staggered_fills_and_generates_match_flat_oracle(dev, attn_func):
+    """The reference's mixed scenario (parrot/testing/model_runner_test_template.py:148-190): three unrelated
+    requests arrive one iteration apart, so iterations hold a Fill next to running Generate jobs and the batch
+    changes from one iteration to the next (the cached slot tables must be rebuilt each time it does)."""
+    from parrotserve_amd.attn_func import BuiltinConfig
+    from parrotserve_amd.primitive_job import Fill, Generate
+    from parrotserve_amd.runner import BuiltinRunner, LlamaConfig, SamplingConfig
+
+    V, N, H, L, Fdim = 211, 256, 2, 2, 384
+    mc = LlamaConfig(vocab_size=V, hidden_size=N, intermediate_size=Fdim, num_hidden_layers=L, num_attention_heads=H,
+                     rms_norm_eps=1e-6, max_position_embeddings=256)
+    cfg = BuiltinConfig(num_kv_cache_blocks=2048, attn_func=attn_func, dtype=torch.float16, device=dev)
+    cfg.attn_func.table_cache.clear()
+    runner = BuiltinRunner(mc, cfg, dummy_weights=False)
+    w = _set_weights(runner.model, 5)
+    g = torch.Generator().manual_seed(17)
+    prompts = [torch.randint(0, V, (n,), generator=g).tolist() for n in (9, 33, 17)]
+    sc = SamplingConfig(top_p=1e-6, max_gen_length=8)
+    fills = [Fill(0, i, i, -1, token_ids=prompts[i]) for i in range(3)]
+    gens = [Generate(0, i, i, -1, sampling_config=sc) for i in range(3)]
+    runner.run_iter([fills[0]])
+    runner.run_iter([gens[0], fills[1]])
+    runner.run_iter([gens[0], gens[1], fills[2]])
+    for _ in range(4):
+        runner.run_iter([gens[0], gens[1], gens[2]])
+    for i, job in enumerate(gens):
+        produced = list(job.output_queue)
+        assert len(produced) == [7, 6, 5][i] and job.context.token_ids == prompts[i] + produced
+        seq = prompts[i] + produced
+        hid = ref_llama_hidden(w, seq[:-1], H, 1e-6, cache_dtype=torch.float16)
+        clear = 0
+        for s, tok in enumerate(produced):
+            logits = hid[len(prompts[i]) - 1 + s] @ w["lm_head"].t()
+            top2 = logits.topk(2)
+            if top2.values[0] - top2.values[1] > 0.25:
+                clear += 1
+                assert tok == int(top2.indices[0]), (i, s)
+        assert clear >= len(produced) // 2
+    cfg.attn_func.table_cache.clear()
