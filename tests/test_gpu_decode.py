@@ -147,6 +147,37 @@ def test_other_head_sizes_and_odd_head_counts(dev, D, H):
     _check(case, dev)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("D", [64, 80, 96, 112, 128, 256])
+def test_vllm_test_distribution_over_head_sizes(dev, D, dtype):
+    """The vendored vLLM kernel test's inputs (3rdparty/vllm/tests/kernels/test_attention.py:159-246): q, k, v uniform
+    in [-1e-3, 1e-3], 7 sequences of random length, every head size its kernels take.  Outputs are of the order of
+    1e-5, so the comparison is relative with a floor two orders below them instead of that test's atol of 1e-3."""
+    from parrotserve_amd import kernels
+
+    g = torch.Generator().manual_seed(D)
+    B, H = 7, 12
+    lens = torch.randint(1, 300, (B,), generator=g).tolist()
+    total = sum(lens)
+    uni = lambda *shape: ((torch.rand(*shape, generator=g) * 2 - 1) * 1e-3).to(dtype)  # noqa: E731
+    q, k, v = uni(B, H, D), uni(total + 5, H, D), uni(total + 5, H, D)
+    perm = torch.randperm(total + 5, generator=g)
+    lists, pos = [], 0
+    for n in lens:
+        lists.append(perm[pos:pos + n])
+        pos += n
+    ref = ref_decode_attention(q, k, v, lists)
+    width = max(lens)
+    table = torch.zeros((B, width), dtype=torch.int32)
+    for i, x in enumerate(lists):
+        table[i, : len(x)] = x.to(torch.int32)
+    hm = torch.arange(H, dtype=torch.int32, device=dev)
+    out = kernels.vllm_paged_attention(q.to(dev), k.to(dev), v.to(dev), hm, torch.tensor(lens, dtype=torch.int32, device=dev),
+                                       table.to(dev)).cpu()
+    rel = 1e-2 if dtype == torch.float16 else 2e-2
+    torch.testing.assert_close(out.float(), ref.float(), atol=2e-7 if dtype == torch.float16 else 1e-6, rtol=rel)
+
+
 def test_config3_ragged_decode_scaled(dev):
     """Config 3's distribution (ctx log-uniform[128,8192], 32x128) on 32 of the 256 requests."""
     from parrotserve_amd import synth
