@@ -500,7 +500,7 @@ struct NoMid {
   __device__ __forceinline__ void operator()() const {}
 };
 
-template <typename E, bool CAUSAL, int TQ, typename Mid = NoMid, int SUB = 1>
+template <typename E, bool CAUSAL, int TQ, typename Mid = NoMid, int SUB = 1, bool HALF = false>
 __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* __restrict__ kc,
                                            const uint16_t* __restrict__ vc, int64_t row_stride, int head,
                                            float scale_log2e, char* smem, float16_t (&ofold)[4 / TQ], float& mfin,
@@ -531,6 +531,10 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
   constexpr bool PREFETCH = !CAUSAL && A == 1 && STEP * TQ == 128;
   constexpr int kPfSteps = 2;
   constexpr float kSlack = 8.f;
+  // HALF: a 64-wide head as half wk.pair_half (0 / 1) of a head pair -- only that half's two 32-dim blocks of the
+  // output are wanted, so only they are multiplied (accumulators 0 and 1 stand for blocks 2 half, 2 half + 1)
+  static_assert(!HALF || TQ == 1, "the half-output form has no fold across token groups");
+  constexpr int NDBV = HALF ? 2 : 4;
   float16_t oacc[4];
   float m = -INFINITY, lsum = 0.f, mtrue = -INFINITY;
   const int lane = threadIdx.x & 63;
@@ -630,8 +634,9 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
         asm("" : "+v"(kaddr[hi][s]));  // keep the sum in one register (otherwise it is re-added at every read)
       }
 #pragma unroll
-      for (int db = 0; db < 4; ++db) {
-        vaddr[hi][db] = gl_a + hi * 65536 + kVtOff + trow * 256 + (sl & 1) * 8 + (((4 * db + tcol) ^ tswz) * 16);
+      for (int db = 0; db < NDBV; ++db) {
+        const int dbr = HALF ? 2 * wk.pair_half + db : db;  // 32-dim block of the 128-wide row
+        vaddr[hi][db] = gl_a + hi * 65536 + kVtOff + trow * 256 + (sl & 1) * 8 + (((4 * dbr + tcol) ^ tswz) * 16);
         asm("" : "+v"(vaddr[hi][db]));
       }
     }
@@ -695,7 +700,7 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
       const int off = stage * SBYTES + sb * kStage;
       const int shi = off >> 16, slo = off & 65535;
 #pragma unroll
-      for (int db = 0; db < 4; ++db)
+      for (int db = 0; db < NDBV; ++db)
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
           const u32x2 lo = lds_tr16_a(vaddr[shi][db] + slo + (16 * u) * 256);
@@ -742,7 +747,7 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
       // results being read by the vector ALU and the rewritten registers feeding the next C operand
       asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 #pragma unroll
-      for (int db = 0; db < 4; ++db)
+      for (int db = 0; db < NDBV; ++db)
 #pragma unroll
         for (int r = 0; r < 16; ++r) asm volatile("v_mul_f32 %0, %0, %1" : "+v"(oacc[db][r]) : "v"(alpha));
       asm volatile("s_nop 7" ::: "memory");
@@ -762,7 +767,7 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
           ps = Elem<E>::dot2(pop[u][e], Elem<E>::kOnes, ps);
         }
 #pragma unroll
-      for (int db = 0; db < 4; ++db)
+      for (int db = 0; db < NDBV; ++db)
 #pragma unroll
         for (int u = 0; u < 2; ++u) oacc[db] = Mfma32<E>::run(va[sb][db][u], pop[u], oacc[db]);
     }
@@ -972,7 +977,8 @@ __global__ __launch_bounds__(512) void decode_fused_kernel(PrefixArgs pa, int mt
 }
 
 // Prefill with parent context, eight waves: workgroup = (head, tile of 32 * (8 / TQ) queries of one chunk)
-template <typename E, int TQ, int SUB>
+// HALF (64-wide heads, 256-query tiles): only this head's half of the pair's output is computed
+template <typename E, int TQ, int SUB, bool HALF = false>
 __global__ __launch_bounds__(512) void prefill_mfma8_kernel(PrefillArgs a) {
   constexpr int QB = 8 / TQ, NDB = 4 / TQ, QT = 32 * QB;
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -1004,14 +1010,15 @@ __global__ __launch_bounds__(512) void prefill_mfma8_kernel(PrefillArgs a) {
   wk.s1 = min(kvn, wk.causal_off + nq);  // the last live query sees tokens up to causal_off + nq - 1
   float16_t of[NDB];
   float m, l;
-  attn_tile8<E, true, TQ, NoMid, SUB>(wk, a.kc, a.vc, a.row_stride, head, a.scale_log2e, smem, of, m, l);
+  attn_tile8<E, true, TQ, NoMid, SUB, HALF>(wk, a.kc, a.vc, a.row_stride, head, a.scale_log2e, smem, of, m, l);
   const int lane = threadIdx.x & 63, w8 = threadIdx.x >> 6, g = w8 / QB, qb = w8 % QB, h = lane >> 5, ql = lane & 31;
   const int q = 32 * qb + ql;
   if (q < nq) {
     const float inv = l > 0.f ? 1.f / l : 0.f;
 #pragma unroll
     for (int nd = 0; nd < NDB; ++nd) {
-      const int db = NDB * g + nd;  // 32-dim block of the 128-wide row
+      if (HALF && nd >= 2) continue;                      // accumulators 0, 1 hold this half's two blocks
+      const int db = HALF ? 2 * half + nd : NDB * g + nd;  // 32-dim block of the 128-wide row
       if (a.pair && (db >> 1) != half) continue;  // the other half holds the neighbouring head's values: dropped
       // paired: head 2 * pair + half, dims 32 * (db & 1) ..; else head, dims 32 * db ..
       uint16_t* op = a.out + (int64_t)(cq0 + q0 + q) * a.out_stride +
@@ -1066,15 +1073,16 @@ static int launch_prefix_t(const PrefixArgs& a, int num_groups, int max_group_re
   return launch_status();
 }
 
-template <typename E, int TQ, int SUB>
+template <typename E, int TQ, int SUB, bool HALF = false>
 static int launch_prefill_tq(const PrefillArgs& a, int64_t num_tokens, hipStream_t st) {
   constexpr int QT = 32 * (8 / TQ);  // queries per workgroup tile
   hipLaunchKernelGGL(prefill_tiles_kernel, dim3(1), dim3(64), 0, st, a.q_cu, a.num_chunks, a.tile_cu, QT);
-  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_mfma8_kernel<E, TQ, SUB>),
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_mfma8_kernel<E, TQ, SUB, HALF>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, kTile8Lds);
   const int hx = (a.H + 7) / 8 * 8;  // keeps head == linear id mod 8 for every tile row
   const int64_t max_tiles = num_tokens / QT + a.num_chunks;  // >= sum of ceil(n_c / QT)
-  hipLaunchKernelGGL((prefill_mfma8_kernel<E, TQ, SUB>), dim3(hx, (unsigned)max_tiles), dim3(512), kTile8Lds, st, a);
+  hipLaunchKernelGGL((prefill_mfma8_kernel<E, TQ, SUB, HALF>), dim3(hx, (unsigned)max_tiles), dim3(512), kTile8Lds, st,
+                     a);
   return launch_status();
 }
 
@@ -1083,6 +1091,7 @@ static int launch_prefill_tq(const PrefillArgs& a, int64_t num_tokens, hipStream
 template <typename E>
 static int launch_prefill_t(const PrefillArgs& a, int64_t num_tokens, hipStream_t st) {
   const int64_t avg = num_tokens / (a.num_chunks > 0 ? a.num_chunks : 1);
+  if (avg >= 192 && a.pair) return launch_prefill_tq<E, 1, 2, true>(a, num_tokens, st);
   if (avg >= 192) return launch_prefill_tq<E, 1, 2>(a, num_tokens, st);  // 64-token steps (measured 4 % faster)
   if (avg >= 96) return launch_prefill_tq<E, 2, 1>(a, num_tokens, st);
   return launch_prefill_tq<E, 4, 1>(a, num_tokens, st);
