@@ -334,8 +334,7 @@ def prefix_length_sweep(torch, dev):
             kernels.decode_attention(q, kc, vc, tabs, out=o)
         sets = [ev.create(6) for _ in range(30)]
         for s6 in sets:
-            lib.ph_arm_kernel_events(s6)
-            kernels.decode_attention(q, kc, vc, tabs, out=o)
+            kernels.decode_attention(q, kc, vc, tabs, out=o, events6=s6)
         torch.cuda.synchronize()
         t = sorted(ev.elapsed_ms(s6[2], s6[3]) for s6 in sets)[15] * 1e3
         for s6 in sets:
@@ -593,9 +592,9 @@ def main():
         qs.append(case.q.to(dev) if l == 0 else torch.randn((B, H, D), generator=dgen, device=dev, dtype=torch.float16))
     out = torch.empty((B, H, D), dtype=torch.float16, device=dev)
 
-    def step(i):
+    def step(i, events6=None):
         l = i % NL
-        kernels.decode_attention(qs[l], kc, vc, tables[l], out=out)
+        kernels.decode_attention(qs[l], kc, vc, tables[l], out=out, events6=events6)
 
     def timed(fn, steps, warmup):
         for i in range(warmup):
@@ -628,8 +627,7 @@ def main():
     n_ev = min(args.steps, 200)
     sets = [ev.create(6) for _ in range(n_ev)]
     for i in range(n_ev):
-        lib.ph_arm_kernel_events(sets[i])
-        step(i)
+        step(i, sets[i])
     torch.cuda.synchronize()
     ph = [[ev.elapsed_ms(s[2 * k], s[2 * k + 1]) for s in sets] for k in range(3)]
     for s in sets:
@@ -695,10 +693,8 @@ def main():
             kernels.decode_attention(qs[i % NL], kc, vc, ptabs[i % NL], out=out)
         sets = [ev.create(6) for _ in range(64)]
         for i, s6 in enumerate(sets):
-            lib.ph_arm_kernel_events(s6)
-            kernels.decode_attention(qs[i % NL], kc, vc, ptabs[i % NL], out=out)
+            kernels.decode_attention(qs[i % NL], kc, vc, ptabs[i % NL], out=out, events6=s6)
         torch.cuda.synchronize()
-        lib.ph_arm_kernel_events(None)
         tp = [ev.elapsed_ms(s6[0], s6[1]) for s6 in sets]
         for s6 in sets:
             ev.destroy(s6)

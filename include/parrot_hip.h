@@ -178,7 +178,10 @@ int ph_rotary_embedding(void* state, const void* cos, const void* sin,
  *   suffix_slots_count: number of int32 entries readable behind suffix_slots
  *                 (the kernel prefetches slot ids before it knows a list's
  *                 length and clamps those reads to this bound);
- *   suffix_lens:  int32 [B] (DEVICE); max_suffix_len: host upper bound.
+ *   suffix_lens:  int32 [B] (DEVICE); max_suffix_len: host upper bound -- the
+ *                 kernels read a length as min(max(len, 0), max_suffix_len),
+ *                 so a bad entry cannot walk into another request's slots
+ *                 (for a padded table pass at most its width).
  * chunk_tokens: suffix split size of the plain (request, chunk) grid form
  *   (multiple of 16); 0 = leave the decomposition to the library.
  * plan (HOST struct of DEVICE pointers, may be NULL): a caller that knows the
@@ -378,11 +381,14 @@ int ph_suffix_tables_append(int32_t* table, int64_t table_stride, int32_t* lens,
  * hold num_lanes + num_reqs entries of 4 ints, lane_rec num_lanes entries of
  * 8, req_item_cu num_reqs + 1.  The stream is cut into
  * min(num_lanes, ceil(total / 4)) pieces; records of the remaining lanes are
- * empty.  num_reqs <= 8192; the lengths must sum to less than 2^31.  The
- * reference has no counterpart (its kernels take fixed-size blocks per
+ * empty.  num_reqs <= 8192; the lengths must sum to less than 2^31; a length
+ * is read as min(max(len, 0), max_suffix_len), the same clamp the attention
+ * kernels apply (pass the max_suffix_len of the ph_decode_attention call).
+ * The reference has no counterpart (its kernels take fixed-size blocks per
  * request, attention_post_kernels.cu:74-110). */
-int ph_suffix_plan_build(const int32_t* suffix_lens, int64_t num_reqs, int64_t num_lanes,
-                         int32_t* items, int32_t* lane_rec, int32_t* req_item_cu, void* stream);
+int ph_suffix_plan_build(const int32_t* suffix_lens, int64_t num_reqs, int64_t max_suffix_len,
+                         int64_t num_lanes, int32_t* items, int32_t* lane_rec, int32_t* req_item_cu,
+                         void* stream);
 
 /* ------------------------------------------------------------------------ */
 /* Token sampler: temperature, top-p filter and one draw per row, in one launch.
@@ -413,15 +419,29 @@ int ph_sample_top_p(const void* logits, int64_t row_stride, const float* tempera
 /* ------------------------------------------------------------------------ */
 /* Instrumentation (no counterpart in the reference, which times whole
  * iterations from Python, parrot/engine/builtin/builtin_runner.py:158-175).
- * Arms the NEXT ph_decode_attention call of the process: its prefix, suffix
- * and merge kernels are launched with (start, stop) event pairs that carry
- * each dispatch's own begin and end timestamps: events[0,1] prefix kernel,
- * events[2,3] suffix kernel, events[4,5] merge kernel (hipEvent_t handles
- * created and owned by the caller; read them with hipEventElapsedTime after
- * synchronising).  A pair whose kernel the call does not launch is left
- * untouched.  One call consumes the arming; pass NULL to disarm.  Not for
- * concurrent callers. */
-int ph_arm_kernel_events(void* const* events6);
+ * ph_decode_attention with one more argument: events6, six hipEvent_t handles
+ * created and owned by the caller.  The call's prefix, suffix and merge
+ * kernels are launched with (start, stop) event pairs that carry each
+ * dispatch's own begin and end timestamps: events6[0,1] prefix kernel,
+ * events6[2,3] suffix kernel (or the kernel that runs both phases),
+ * events6[4,5] merge kernel; read them with hipEventElapsedTime after
+ * synchronising.  A pair whose kernel the call does not launch is left
+ * untouched.  events6 == NULL is exactly ph_decode_attention.  The events
+ * travel with the call: the library keeps no state between calls. */
+int ph_decode_attention_timed(void* out, const void* q, const void* k_cache, const void* v_cache,
+                              int64_t num_reqs, int64_t num_heads, int64_t head_dim, int dtype,
+                              int64_t q_stride, int64_t out_stride, int64_t cache_stride_n,
+                              float scale,
+                              int64_t num_groups, const int32_t* prefix_slots, const int32_t* prefix_cu,
+                              const int32_t* group_req_cu, const int32_t* group_req_cu_host,
+                              int64_t max_prefix_len,
+                              const int32_t* suffix_slots, const int64_t* suffix_offsets,
+                              int64_t suffix_table_stride, int64_t suffix_slots_count,
+                              const int32_t* suffix_lens,
+                              int64_t max_suffix_len, int64_t chunk_tokens,
+                              const ph_suffix_plan* plan,
+                              void* workspace, size_t workspace_bytes, void* stream,
+                              void* const* events6);
 
 #ifdef __cplusplus
 }

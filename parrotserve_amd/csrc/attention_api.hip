@@ -72,7 +72,7 @@ static DecodePlan plan_decode(int64_t B, int64_t H, int64_t groups, int64_t max_
   }
   if (groups > 0 && max_prefix > 0) {
     // One workgroup per CU at a time (the kernel uses most of the register file), so pick the
-    // split count whose workgroup total wastes the least of a whole number of 256-wide rounds.
+    // split count whose workgroup total wastes the least of a whole number of rounds over the device's CUs.
     // Cost model: rounds x (tokens per split + a fixed prologue/epilogue worth ~96 tokens).
     // the kernel takes 64-, 128- or 256-query tiles by the largest group; the mean group size stands in here
     p.paired = paired;
@@ -83,9 +83,10 @@ static DecodePlan plan_decode(int64_t B, int64_t H, int64_t groups, int64_t max_
     const int64_t base = groups * rows_h * (mtiles > 0 ? mtiles : 1);
     const int64_t max_splits = cdiv(max_prefix, 4 * kPrefixTile);
     int64_t splits = 1, best = -1;
+    const int64_t cus = device_cus();
     for (int64_t s = 1; s <= 64 && s <= (max_splits > 0 ? max_splits : 1); ++s) {
       const int64_t tok = round_up(cdiv(max_prefix, s), 2 * kPrefixTile);
-      const int64_t cost = cdiv(base * s, 256) * (tok + 96);
+      const int64_t cost = cdiv(base * s, cus) * (tok + 96);
       if (best < 0 || cost < best) {
         best = cost;
         splits = s;
@@ -173,10 +174,11 @@ static PrefixArgs pair_args(const PrefixArgs& pa, const Carve& ws) {
 }
 
 static int run_prefix(PrefixArgs& pa, int dtype, int D, int num_groups, const int32_t* group_req_cu_host,
-                      int max_group_reqs, hipStream_t st, const Carve* pairs = nullptr) {
+                      int max_group_reqs, hipStream_t st, const Carve* pairs = nullptr,
+                      const KernelEvents& ev = KernelEvents()) {
   if (pairs && pairs->opart_pairs)
-    return launch_prefix_mfma(pair_args(pa, *pairs), dtype, 128, num_groups, 2 * max_group_reqs, st);
-  if (prefix_mfma_supported(dtype, D)) return launch_prefix_mfma(pa, dtype, D, num_groups, max_group_reqs, st);
+    return launch_prefix_mfma(pair_args(pa, *pairs), dtype, 128, num_groups, 2 * max_group_reqs, st, ev);
+  if (prefix_mfma_supported(dtype, D)) return launch_prefix_mfma(pa, dtype, D, num_groups, max_group_reqs, st, ev);
   int rc = launch_clear_ml(pa.ml, (int64_t)pa.n_splits * pa.B * pa.H, st);
   if (rc != PH_OK) return rc;
   for (int g = 0; g < num_groups; ++g) {
@@ -238,26 +240,7 @@ extern "C" const char* ph_status_string(int status) {
   }
 }
 
-extern "C" int ph_abi_version(void) { return 1; }
-
-static hipEvent_t g_kernel_events[6];
-static bool g_events_armed = false;
-
-extern "C" int ph_arm_kernel_events(void* const* events6) {
-  g_events_armed = events6 != nullptr;
-  if (events6)
-    for (int i = 0; i < 6; ++i) g_kernel_events[i] = (hipEvent_t)events6[i];
-  return PH_OK;
-}
-
-ph::KernelEvents ph::take_kernel_events(int which) {
-  KernelEvents e;
-  if (g_events_armed && which >= 0 && which < 3) {
-    e.start = g_kernel_events[2 * which];
-    e.stop = g_kernel_events[2 * which + 1];
-  }
-  return e;
-}
+extern "C" int ph_abi_version(void) { return 2; }
 
 extern "C" size_t ph_decode_workspace_bytes(int64_t num_reqs, int64_t num_heads, int64_t head_dim,
                                             int64_t num_groups, int64_t max_prefix_len, int64_t max_suffix_len,
@@ -269,21 +252,28 @@ extern "C" size_t ph_decode_workspace_bytes(int64_t num_reqs, int64_t num_heads,
   return plan_bytes(p, num_reqs, num_heads, head_dim);
 }
 
-extern "C" int ph_decode_attention(void* out, const void* q, const void* k_cache, const void* v_cache,
-                                   int64_t num_reqs, int64_t num_heads, int64_t head_dim, int dtype,
-                                   int64_t q_stride, int64_t out_stride, int64_t cache_stride_n, float scale,
-                                   int64_t num_groups, const int32_t* prefix_slots, const int32_t* prefix_cu,
-                                   const int32_t* group_req_cu, const int32_t* group_req_cu_host,
-                                   int64_t max_prefix_len, const int32_t* suffix_slots,
-                                   const int64_t* suffix_offsets, int64_t suffix_table_stride,
-                                   int64_t suffix_slots_count, const int32_t* suffix_lens, int64_t max_suffix_len,
-                                   int64_t chunk_tokens, const ph_suffix_plan* plan, void* workspace,
-                                   size_t workspace_bytes, void* stream) {
+// events6: null, or (start, stop) event pairs for the prefix, suffix and merge kernels of this call
+static int decode_attention_impl(void* out, const void* q, const void* k_cache, const void* v_cache,
+                                 int64_t num_reqs, int64_t num_heads, int64_t head_dim, int dtype,
+                                 int64_t q_stride, int64_t out_stride, int64_t cache_stride_n, float scale,
+                                 int64_t num_groups, const int32_t* prefix_slots, const int32_t* prefix_cu,
+                                 const int32_t* group_req_cu, const int32_t* group_req_cu_host,
+                                 int64_t max_prefix_len, const int32_t* suffix_slots,
+                                 const int64_t* suffix_offsets, int64_t suffix_table_stride,
+                                 int64_t suffix_slots_count, const int32_t* suffix_lens, int64_t max_suffix_len,
+                                 int64_t chunk_tokens, const ph_suffix_plan* plan, void* workspace,
+                                 size_t workspace_bytes, void* stream, void* const* events6) {
   const int B = (int)num_reqs, H = (int)num_heads, D = (int)head_dim;
+  KernelEvents ev_prefix, ev_suffix, ev_merge;
+  if (events6) {
+    ev_prefix = KernelEvents{(hipEvent_t)events6[0], (hipEvent_t)events6[1]};
+    ev_suffix = KernelEvents{(hipEvent_t)events6[2], (hipEvent_t)events6[3]};
+    ev_merge = KernelEvents{(hipEvent_t)events6[4], (hipEvent_t)events6[5]};
+  }
   int rc = check_common(out, q, k_cache, v_cache, num_reqs, num_heads, head_dim, dtype, q_stride, out_stride,
                         cache_stride_n);
   if (rc != PH_OK || num_reqs == 0) return rc;
-  if (num_groups < 0 || max_prefix_len < 0 || max_suffix_len < 0) return PH_ERR_ARG;
+  if (num_groups < 0 || max_prefix_len < 0 || max_suffix_len < 0 || max_suffix_len > INT32_MAX) return PH_ERR_ARG;
   const bool has_prefix = num_groups > 0 && max_prefix_len > 0;
   const bool has_suffix = max_suffix_len > 0;
   if (has_prefix && (!prefix_slots || !prefix_cu || !group_req_cu || !group_req_cu_host)) return PH_ERR_ARG;
@@ -302,7 +292,7 @@ extern "C" int ph_decode_attention(void* out, const void* q, const void* k_cache
   hipStream_t st = (hipStream_t)stream;
   ph_suffix_plan own_plan{};
   if (!planned && p.dev_lanes > 0) {  // no plan from the caller: one is built on the device first
-    rc = launch_suffix_plan(suffix_lens, B, p.dev_lanes, ws.items, ws.lane_rec, ws.req_item_cu, st);
+    rc = launch_suffix_plan(suffix_lens, B, (int)max_suffix_len, p.dev_lanes, ws.items, ws.lane_rec, ws.req_item_cu, st);
     if (rc != PH_OK) return rc;
     own_plan = ph_suffix_plan{ws.items, p.items, ws.lane_rec, p.dev_lanes, ws.req_item_cu};
     plan = &own_plan;
@@ -348,7 +338,8 @@ extern "C" int ph_decode_attention(void* out, const void* q, const void* k_cache
       fused_groups = (int)num_groups;
       fused_max_reqs = paired ? 2 * max_group_reqs : max_group_reqs;
     } else {
-      rc = run_prefix(pa, dtype, D, (int)num_groups, group_req_cu_host, max_group_reqs, st, paired ? &ws : nullptr);
+      rc = run_prefix(pa, dtype, D, (int)num_groups, group_req_cu_host, max_group_reqs, st, paired ? &ws : nullptr,
+                      ev_prefix);
       if (rc != PH_OK) return rc;
     }
   }
@@ -370,8 +361,8 @@ extern "C" int ph_decode_attention(void* out, const void* q, const void* k_cache
     ia.ml = ws.ml + item_base * 2;
     ia.H = H;
     ia.scale_log2e = sl2;
-    rc = fuse ? launch_decode_fused(fused_pa, ia, dtype, fused_groups, fused_max_reqs, device_cus(), st)
-              : launch_items(ia, dtype, D, st);
+    rc = fuse ? launch_decode_fused(fused_pa, ia, dtype, fused_groups, fused_max_reqs, device_cus(), st, ev_suffix)
+              : launch_items(ia, dtype, D, st, ev_suffix);
     if (rc != PH_OK) return rc;
   } else if (has_suffix) {
     PartialArgs sa{};
@@ -385,6 +376,7 @@ extern "C" int ph_decode_attention(void* out, const void* q, const void* k_cache
     sa.offsets = suffix_offsets;
     sa.table_stride = suffix_table_stride;
     sa.lens = suffix_lens;
+    sa.max_len = (int)max_suffix_len;
     sa.shared_cu = nullptr;
     sa.shared_len = -1;
     sa.chunk = p.chunk;
@@ -397,7 +389,7 @@ extern "C" int ph_decode_attention(void* out, const void* q, const void* k_cache
     sa.req_begin = 0;
     sa.num_reqs = B;
     sa.scale_log2e = sl2;
-    rc = launch_partial(sa, dtype, D, st);
+    rc = launch_partial(sa, dtype, D, st, ev_suffix);
     if (rc != PH_OK) return rc;
   }
   MergeArgs ma{};
@@ -414,12 +406,46 @@ extern "C" int ph_decode_attention(void* out, const void* q, const void* k_cache
   }
   ma.baseB = p.n_splits;
   ma.lens = has_suffix ? suffix_lens : nullptr;
+  ma.max_len = (int)max_suffix_len;
   ma.chunk = p.chunk;
   ma.req_item_cu = planned ? plan->req_item_cu : nullptr;
   ma.item_base = item_base;
-  rc = launch_merge(ma, dtype, D, st);
-  g_events_armed = false;  // one call consumes the arming
-  return rc;
+  return launch_merge(ma, dtype, D, st, ev_merge);
+}
+
+extern "C" int ph_decode_attention(void* out, const void* q, const void* k_cache, const void* v_cache,
+                                   int64_t num_reqs, int64_t num_heads, int64_t head_dim, int dtype,
+                                   int64_t q_stride, int64_t out_stride, int64_t cache_stride_n, float scale,
+                                   int64_t num_groups, const int32_t* prefix_slots, const int32_t* prefix_cu,
+                                   const int32_t* group_req_cu, const int32_t* group_req_cu_host,
+                                   int64_t max_prefix_len, const int32_t* suffix_slots,
+                                   const int64_t* suffix_offsets, int64_t suffix_table_stride,
+                                   int64_t suffix_slots_count, const int32_t* suffix_lens, int64_t max_suffix_len,
+                                   int64_t chunk_tokens, const ph_suffix_plan* plan, void* workspace,
+                                   size_t workspace_bytes, void* stream) {
+  return decode_attention_impl(out, q, k_cache, v_cache, num_reqs, num_heads, head_dim, dtype, q_stride, out_stride,
+                               cache_stride_n, scale, num_groups, prefix_slots, prefix_cu, group_req_cu,
+                               group_req_cu_host, max_prefix_len, suffix_slots, suffix_offsets, suffix_table_stride,
+                               suffix_slots_count, suffix_lens, max_suffix_len, chunk_tokens, plan, workspace,
+                               workspace_bytes, stream, nullptr);
+}
+
+extern "C" int ph_decode_attention_timed(void* out, const void* q, const void* k_cache, const void* v_cache,
+                                         int64_t num_reqs, int64_t num_heads, int64_t head_dim, int dtype,
+                                         int64_t q_stride, int64_t out_stride, int64_t cache_stride_n, float scale,
+                                         int64_t num_groups, const int32_t* prefix_slots, const int32_t* prefix_cu,
+                                         const int32_t* group_req_cu, const int32_t* group_req_cu_host,
+                                         int64_t max_prefix_len, const int32_t* suffix_slots,
+                                         const int64_t* suffix_offsets, int64_t suffix_table_stride,
+                                         int64_t suffix_slots_count, const int32_t* suffix_lens,
+                                         int64_t max_suffix_len, int64_t chunk_tokens, const ph_suffix_plan* plan,
+                                         void* workspace, size_t workspace_bytes, void* stream,
+                                         void* const* events6) {
+  return decode_attention_impl(out, q, k_cache, v_cache, num_reqs, num_heads, head_dim, dtype, q_stride, out_stride,
+                               cache_stride_n, scale, num_groups, prefix_slots, prefix_cu, group_req_cu,
+                               group_req_cu_host, max_prefix_len, suffix_slots, suffix_offsets, suffix_table_stride,
+                               suffix_slots_count, suffix_lens, max_suffix_len, chunk_tokens, plan, workspace,
+                               workspace_bytes, stream, events6);
 }
 
 // Prefix phase over one shared slot list, merged with an optional partial already in out / prev_m / prev_l; the
@@ -519,7 +545,7 @@ static int suffix_phase(void* out, const float* prev_m, const float* prev_l, flo
   int rc = check_common(out, q, k_cache, v_cache, num_reqs, num_heads, head_dim, dtype, q_stride, out_stride,
                         cache_stride_n);
   if (rc != PH_OK || num_reqs == 0) return rc;
-  if (max_suffix_len < 0) return PH_ERR_ARG;
+  if (max_suffix_len < 0 || max_suffix_len > INT32_MAX) return PH_ERR_ARG;
   const bool has_suffix = max_suffix_len > 0;
   if (has_suffix && (!suffix_slots || !suffix_lens || suffix_slots_count <= 0)) return PH_ERR_ARG;
   const DecodePlan p = plan_decode(num_reqs, num_heads, 0, 0, max_suffix_len, chunk_tokens, 0, head_dim);
@@ -529,7 +555,7 @@ static int suffix_phase(void* out, const float* prev_m, const float* prev_l, flo
   const Carve ws = carve(workspace, p, B, H, D);
   hipStream_t st = (hipStream_t)stream;
   if (has_suffix && p.dev_lanes > 0) {  // balanced form on a plan built on the device
-    rc = launch_suffix_plan(suffix_lens, B, p.dev_lanes, ws.items, ws.lane_rec, ws.req_item_cu, st);
+    rc = launch_suffix_plan(suffix_lens, B, (int)max_suffix_len, p.dev_lanes, ws.items, ws.lane_rec, ws.req_item_cu, st);
     if (rc != PH_OK) return rc;
     ItemArgs ia{};
     ia.q = (const uint16_t*)q;
@@ -561,6 +587,7 @@ static int suffix_phase(void* out, const float* prev_m, const float* prev_l, flo
     sa.offsets = suffix_offsets;
     sa.table_stride = suffix_table_stride;
     sa.lens = suffix_lens;
+    sa.max_len = (int)max_suffix_len;
     sa.shared_cu = nullptr;
     sa.shared_len = -1;
     sa.chunk = p.chunk;
@@ -586,6 +613,7 @@ static int suffix_phase(void* out, const float* prev_m, const float* prev_l, flo
   ma.nA = 0;
   ma.baseB = 0;
   ma.lens = has_suffix ? suffix_lens : nullptr;
+  ma.max_len = (int)max_suffix_len;
   ma.chunk = p.chunk;
   ma.req_item_cu = has_suffix && p.dev_lanes > 0 ? ws.req_item_cu : nullptr;
   ma.item_base = 0;
@@ -647,7 +675,7 @@ extern "C" int ph_prefill_attention(void* out, const void* q, const void* k_cach
   int rc = check_common(out, q, k_cache, v_cache, num_tokens, num_heads, head_dim, dtype, q_stride, out_stride,
                         cache_stride_n);
   if (rc != PH_OK || num_tokens == 0) return rc;
-  if (num_chunks <= 0 || max_kv_len <= 0 || !q_cu || !kv_cu || !ctx_slots || ctx_slots_count <= 0) return PH_ERR_ARG;
+  if (num_chunks <= 0 || max_kv_len <= 0 || max_kv_len > INT32_MAX || !q_cu || !kv_cu || !ctx_slots || ctx_slots_count <= 0) return PH_ERR_ARG;
   if (ph_prefill_workspace_bytes(num_tokens, num_heads, head_dim, max_kv_len) > workspace_bytes || !workspace)
     return PH_ERR_WORKSPACE;
   if (((uintptr_t)workspace & 255u) != 0) return PH_ERR_ALIGN;
@@ -691,6 +719,7 @@ extern "C" int ph_prefill_attention(void* out, const void* q, const void* k_cach
   sa.slots_total = ctx_slots_count;
   sa.offsets = offsets;
   sa.lens = lens;
+  sa.max_len = (int)max_kv_len;
   sa.shared_len = -1;
   sa.chunk = p.chunk;
   sa.n_chunks = p.n_chunks;
@@ -713,6 +742,7 @@ extern "C" int ph_prefill_attention(void* out, const void* q, const void* k_cach
   ma.nA = 0;
   ma.baseB = 0;
   ma.lens = lens;
+  ma.max_len = (int)max_kv_len;
   ma.chunk = p.chunk;
   return launch_merge(ma, dtype, D, st);
 }

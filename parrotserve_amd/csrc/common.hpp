@@ -137,13 +137,13 @@ __device__ __forceinline__ void rotate8(u32x4& x, u32x4& y, const u32x4 c, const
   }
 }
 
-// Optional timing of one kernel's own dispatch: the three main kernels of the decode path (0 prefix,
-// 1 suffix, 2 merge) are launched through hipExtLaunchKernelGGL, which stamps a start and a stop event
-// with the dispatch's begin and end timestamps.  Null events (the normal case) make it a plain launch.
+// Optional timing of one kernel's own dispatch: the three main kernels of the decode path (prefix, suffix,
+// merge) can be launched through hipExtLaunchKernelGGL, which stamps a start and a stop event with the
+// dispatch's begin and end timestamps.  The events come in per call (ph_decode_attention_timed); null events
+// (the normal case) make it a plain launch.
 struct KernelEvents {
   hipEvent_t start = nullptr, stop = nullptr;
 };
-KernelEvents take_kernel_events(int which);  // attention_api.hip; nulls unless the call was armed
 
 // Launch with the optional event pair; without events this is the ordinary launch call (the one that
 // stream capture and every tool expects), the extended call is only used when a caller asked for timing.

@@ -55,7 +55,8 @@ __global__ __launch_bounds__(256) void decode_partial_kernel(PartialArgs a) {
   if (last < 0) return;  // an empty shared list, or an offset at the very end of the table
   const int32_t* slots = a.slots + off;
   const int myslot = slots[min((int64_t)(t0 + lane), last)];
-  if (len < 0) len = a.lens[b];
+  // a length beyond the host's bound (or the table's end) would walk into other requests' slots
+  if (len < 0) len = (int)min((int64_t)min(max(a.lens[b], 0), a.max_len), last + 1);
 
   const int head = hg * HPW + lane / LPH;
   const bool head_ok = head < a.H;
@@ -128,7 +129,7 @@ __global__ __launch_bounds__(256) void merge_kernel(MergeArgs a) {
     it0 = a.req_item_cu[b];
     nB = a.req_item_cu[b + 1] - it0;
   } else {
-    nB = a.lens ? (a.lens[b] + a.chunk - 1) / a.chunk : 0;
+    nB = a.lens ? (min(max(a.lens[b], 0), a.max_len) + a.chunk - 1) / a.chunk : 0;
   }
   const int total = a.nA + nB;
 #pragma unroll 2
@@ -205,37 +206,34 @@ __global__ __launch_bounds__(256) void clear_ml_kernel(float* ml, int64_t n2) {
 }
 
 template <typename E, int D>
-static int launch_partial_t(const PartialArgs& a, hipStream_t st) {
+static int launch_partial_t(const PartialArgs& a, hipStream_t st, const KernelEvents& ev) {
   constexpr int HPW = HeadLanes<D>::HPW;
   const int64_t hgroups = (a.H + HPW - 1) / HPW;
   const int64_t waves = (int64_t)a.num_reqs * a.n_chunks * hgroups;
   if (waves == 0) return PH_OK;
   dim3 grid((unsigned)((waves + 3) / 4)), block(256);
-  const KernelEvents ev = take_kernel_events(1);
   PH_LAUNCH_TIMED((decode_partial_kernel<E, D, 4, 2>), grid, block, 0, st, ev, a);
   return launch_status();
 }
 
 template <typename E, int D>
-static int launch_items_t(const ItemArgs& a, hipStream_t st) {
+static int launch_items_t(const ItemArgs& a, hipStream_t st, const KernelEvents& ev) {
   constexpr int HPW = HeadLanes<D>::HPW;
   const int64_t hgroups = (a.H + HPW - 1) / HPW;
   const int64_t waves = (int64_t)a.num_lanes * hgroups;
   if (waves == 0) return PH_OK;
   dim3 grid((unsigned)((waves + 3) / 4)), block(256);
-  const KernelEvents ev = take_kernel_events(1);
   PH_LAUNCH_TIMED((decode_items_kernel<E, D, 4, 2>), grid, block, 0, st, ev, a);
   return launch_status();
 }
 
 template <typename E, int D>
-static int launch_merge_t(const MergeArgs& a, hipStream_t st) {
+static int launch_merge_t(const MergeArgs& a, hipStream_t st, const KernelEvents& ev) {
   constexpr int HPW = HeadLanes<D>::HPW;
   const int64_t hgroups = (a.H + HPW - 1) / HPW;
   const int64_t groups = (int64_t)a.B * hgroups;
   if (groups == 0) return PH_OK;
   dim3 grid((unsigned)groups), block(256);
-  const KernelEvents ev = take_kernel_events(2);
   PH_LAUNCH_TIMED((merge_kernel<E, D>), grid, block, 0, st, ev, a);
   return launch_status();
 }
@@ -260,14 +258,14 @@ static int launch_merge_t(const MergeArgs& a, hipStream_t st) {
     return PH_ERR_HEAD_DIM;                                             \
   } while (0)
 
-int launch_partial(const PartialArgs& a, int dtype, int D, hipStream_t st) {
-  PH_DISPATCH(launch_partial_t, dtype, D, a, st);
+int launch_partial(const PartialArgs& a, int dtype, int D, hipStream_t st, const KernelEvents& ev) {
+  PH_DISPATCH(launch_partial_t, dtype, D, a, st, ev);
 }
-int launch_items(const ItemArgs& a, int dtype, int D, hipStream_t st) {
-  PH_DISPATCH(launch_items_t, dtype, D, a, st);
+int launch_items(const ItemArgs& a, int dtype, int D, hipStream_t st, const KernelEvents& ev) {
+  PH_DISPATCH(launch_items_t, dtype, D, a, st, ev);
 }
-int launch_merge(const MergeArgs& a, int dtype, int D, hipStream_t st) {
-  PH_DISPATCH(launch_merge_t, dtype, D, a, st);
+int launch_merge(const MergeArgs& a, int dtype, int D, hipStream_t st, const KernelEvents& ev) {
+  PH_DISPATCH(launch_merge_t, dtype, D, a, st, ev);
 }
 int launch_clear_ml(float* ml, int64_t entries, hipStream_t st) {
   if (entries == 0) return PH_OK;

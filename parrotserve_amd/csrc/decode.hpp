@@ -19,6 +19,7 @@ struct PartialArgs {
   const int64_t* offsets;   // per-request start inside `slots`, or null
   int64_t table_stride;     // start = b * table_stride when offsets is null
   const int32_t* lens;      // per-request list length
+  int max_len;              // host bound of any list's length: a length read from `lens` is clamped to [0, max_len]
   const int32_t* shared_cu; // if set: every request uses slots[cu[0] .. cu[1])
   int shared_len;           // if >= 0 (and shared_cu null): every request uses slots[0 .. shared_len)
   int chunk;                // tokens per part
@@ -64,6 +65,7 @@ struct MergeArgs {
   int nA;                   // parts [0, nA) are candidates for every request
   int baseB;                // parts [baseB, baseB + ceil(lens[b]/chunk)) likewise
   const int32_t* lens;      // may be null (no B range)
+  int max_len;              // lengths read from `lens` are clamped to [0, max_len]
   int chunk;
   const int32_t* req_item_cu; // balanced form: request b owns items [cu[b], cu[b+1]) ...
   int64_t item_base;          // ... whose partial rows start at item_base (rows of H)
@@ -111,22 +113,24 @@ struct PrefillArgs {
   int pair;                  // 1: heads are 64 wide and run as halves of 128-wide head pairs (q, out, caches [.., H, 64])
 };
 
-int launch_partial(const PartialArgs& a, int dtype, int D, hipStream_t st);
+int launch_partial(const PartialArgs& a, int dtype, int D, hipStream_t st, const KernelEvents& ev = KernelEvents());
 // MFMA prefill: grid (head, query tile); num_tokens = total query rows (bounds the tile count).
 int launch_prefill_mfma(const PrefillArgs& a, int dtype, int D, int64_t num_tokens, hipStream_t st);
-int launch_items(const ItemArgs& a, int dtype, int D, hipStream_t st);
-int launch_merge(const MergeArgs& a, int dtype, int D, hipStream_t st);
+int launch_items(const ItemArgs& a, int dtype, int D, hipStream_t st, const KernelEvents& ev = KernelEvents());
+int launch_merge(const MergeArgs& a, int dtype, int D, hipStream_t st, const KernelEvents& ev = KernelEvents());
 int launch_clear_ml(float* ml, int64_t entries, hipStream_t st);
 // balanced suffix plan written on the device from the length vector (tables.hip); arrays as in ph_suffix_plan
 constexpr int kPlanMaxReqs = 8192;
-int launch_suffix_plan(const int32_t* lens, int B, int lanes, int32_t* items, int32_t* lane_rec, int32_t* req_item_cu,
-                       hipStream_t st);
+// lengths are clamped to [0, max_len]
+int launch_suffix_plan(const int32_t* lens, int B, int max_len, int lanes, int32_t* items, int32_t* lane_rec,
+                       int32_t* req_item_cu, hipStream_t st);
 // MFMA shared-prefix kernel: grid (split, head, group x m-tile).
-int launch_prefix_mfma(const PrefixArgs& a, int dtype, int D, int num_groups, int max_group_reqs, hipStream_t st);
+int launch_prefix_mfma(const PrefixArgs& a, int dtype, int D, int num_groups, int max_group_reqs, hipStream_t st,
+                       const KernelEvents& ev = KernelEvents());
 bool prefix_mfma_supported(int dtype, int D);
 // Prefix + suffix phases in one launch (see decode_fused_kernel); cus = compute units of the device.
 bool decode_fused_supported(int dtype, int D, int max_group_reqs);
 int launch_decode_fused(const PrefixArgs& a, const ItemArgs& ia, int dtype, int num_groups, int max_group_reqs, int cus,
-                        hipStream_t st);
+                        hipStream_t st, const KernelEvents& ev = KernelEvents());
 
 }  // namespace ph

@@ -1056,8 +1056,8 @@ static void launch_prefix8(const PrefixArgs& a, int num_groups, int max_group_re
 }
 
 template <typename E>
-static int launch_prefix_t(const PrefixArgs& a, int num_groups, int max_group_reqs, hipStream_t st) {
-  const KernelEvents ev = take_kernel_events(0);
+static int launch_prefix_t(const PrefixArgs& a, int num_groups, int max_group_reqs, hipStream_t st,
+                           const KernelEvents& ev) {
   if (max_group_reqs <= 32 && a.req_shift == 0) {  // four waves, one 32-query block
     dim3 grid(a.n_splits, a.H, num_groups), block(256);
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefix_mfma_kernel<E, 1>),
@@ -1099,7 +1099,7 @@ static int launch_prefill_t(const PrefillArgs& a, int64_t num_tokens, hipStream_
 
 template <typename E, int TQ, int DS>
 static int launch_fused_tq(const PrefixArgs& a, const ItemArgs& ia, int num_groups, int max_group_reqs, int cus,
-                           hipStream_t st) {
+                           hipStream_t st, const KernelEvents& ev) {
   constexpr int QT = 32 * (8 / TQ);
   constexpr int HPW = HeadLanes<DS>::HPW;
   const int mtiles = (max_group_reqs + QT - 1) / QT;
@@ -1112,7 +1112,6 @@ static int launch_fused_tq(const PrefixArgs& a, const ItemArgs& ia, int num_grou
   if (grid <= 0) return PH_OK;
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&decode_fused_kernel<E, TQ, DS>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, kTile8Lds);
-  const KernelEvents ev = take_kernel_events(1);
   PH_LAUNCH_TIMED((decode_fused_kernel<E, TQ, DS>), dim3(grid), dim3(512), kTile8Lds, st, ev, a, mtiles,
                         n_units, ia);
   return launch_status();
@@ -1121,10 +1120,10 @@ static int launch_fused_tq(const PrefixArgs& a, const ItemArgs& ia, int num_grou
 // query tile by the largest group: 64, 128 or 256 requests share each K/V tile of the prefix
 template <typename E, int DS>
 static int launch_fused_t(const PrefixArgs& a, const ItemArgs& ia, int num_groups, int max_group_reqs, int cus,
-                          hipStream_t st) {
-  if (max_group_reqs <= 64) return launch_fused_tq<E, 4, DS>(a, ia, num_groups, max_group_reqs, cus, st);
-  if (max_group_reqs <= 128) return launch_fused_tq<E, 2, DS>(a, ia, num_groups, max_group_reqs, cus, st);
-  return launch_fused_tq<E, 1, DS>(a, ia, num_groups, max_group_reqs, cus, st);
+                          hipStream_t st, const KernelEvents& ev) {
+  if (max_group_reqs <= 64) return launch_fused_tq<E, 4, DS>(a, ia, num_groups, max_group_reqs, cus, st, ev);
+  if (max_group_reqs <= 128) return launch_fused_tq<E, 2, DS>(a, ia, num_groups, max_group_reqs, cus, st, ev);
+  return launch_fused_tq<E, 1, DS>(a, ia, num_groups, max_group_reqs, cus, st, ev);
 }
 
 // One launch for the prefix and suffix phases: head size 128, groups of more than 32 requests (the
@@ -1134,22 +1133,23 @@ bool decode_fused_supported(int dtype, int D, int max_group_reqs) {
 }
 
 int launch_decode_fused(const PrefixArgs& a, const ItemArgs& ia, int dtype, int num_groups, int max_group_reqs, int cus,
-                        hipStream_t st) {
+                        hipStream_t st, const KernelEvents& ev) {
   if (a.req_shift) {  // 64-wide heads: the prefix phase on head pairs, the suffix phase at its own width
-    return dtype == PH_F16 ? launch_fused_t<F16, 64>(a, ia, num_groups, max_group_reqs, cus, st)
-                           : launch_fused_t<BF16, 64>(a, ia, num_groups, max_group_reqs, cus, st);
+    return dtype == PH_F16 ? launch_fused_t<F16, 64>(a, ia, num_groups, max_group_reqs, cus, st, ev)
+                           : launch_fused_t<BF16, 64>(a, ia, num_groups, max_group_reqs, cus, st, ev);
   }
-  return dtype == PH_F16 ? launch_fused_t<F16, kPD>(a, ia, num_groups, max_group_reqs, cus, st)
-                         : launch_fused_t<BF16, kPD>(a, ia, num_groups, max_group_reqs, cus, st);
+  return dtype == PH_F16 ? launch_fused_t<F16, kPD>(a, ia, num_groups, max_group_reqs, cus, st, ev)
+                         : launch_fused_t<BF16, kPD>(a, ia, num_groups, max_group_reqs, cus, st, ev);
 }
 
 bool prefix_mfma_supported(int dtype, int D) { return D == kPD && (dtype == PH_F16 || dtype == PH_BF16); }
 
-int launch_prefix_mfma(const PrefixArgs& a, int dtype, int D, int num_groups, int max_group_reqs, hipStream_t st) {
+int launch_prefix_mfma(const PrefixArgs& a, int dtype, int D, int num_groups, int max_group_reqs, hipStream_t st,
+                       const KernelEvents& ev) {
   if (D != kPD) return PH_ERR_HEAD_DIM;
   if (num_groups <= 0 || max_group_reqs <= 0 || a.n_splits <= 0) return PH_OK;
-  return dtype == PH_F16 ? launch_prefix_t<F16>(a, num_groups, max_group_reqs, st)
-                         : launch_prefix_t<BF16>(a, num_groups, max_group_reqs, st);
+  return dtype == PH_F16 ? launch_prefix_t<F16>(a, num_groups, max_group_reqs, st, ev)
+                         : launch_prefix_t<BF16>(a, num_groups, max_group_reqs, st, ev);
 }
 
 int launch_prefill_mfma(const PrefillArgs& a, int dtype, int D, int64_t num_tokens, hipStream_t st) {

@@ -79,13 +79,15 @@ __device__ __forceinline__ void block_scan(F v, int n, int* out, int* part) {
   __syncthreads();
 }
 
-__global__ __launch_bounds__(kPlanThreads) void suffix_plan_kernel(const int32_t* __restrict__ lens, int B, int lanes_cap,
+__global__ __launch_bounds__(kPlanThreads) void suffix_plan_kernel(const int32_t* __restrict__ lens, int B, int max_len,
+                                                                   int lanes_cap,
                                                                    int4* __restrict__ items,
                                                                    int4* __restrict__ lane_rec,
                                                                    int32_t* __restrict__ req_item_cu) {
   __shared__ PlanScratch sh;
   const int t = threadIdx.x;
-  block_scan([&](int i) { return max(lens[i], 0); }, B, sh.cu, sh.part);
+  // a length beyond the host's bound would walk into the next request's row of the slot table
+  block_scan([&](int i) { return min(max(lens[i], 0), max_len); }, B, sh.cu, sh.part);
   const int64_t total = sh.cu[B];
   const int lanes = (int)max((int64_t)1, min((int64_t)lanes_cap, min((total + kMinPiece - 1) / kMinPiece, total)));
   auto cut = [&](int l) { return (int)((int64_t)l * total / lanes); };
@@ -146,22 +148,24 @@ __global__ __launch_bounds__(kPlanThreads) void suffix_plan_kernel(const int32_t
   }
 }
 
-int launch_suffix_plan(const int32_t* lens, int B, int lanes, int32_t* items, int32_t* lane_rec, int32_t* req_item_cu,
-                       hipStream_t st) {
-  hipLaunchKernelGGL(suffix_plan_kernel, dim3(1), dim3(kPlanThreads), 0, st, lens, B, lanes,
+int launch_suffix_plan(const int32_t* lens, int B, int max_len, int lanes, int32_t* items, int32_t* lane_rec,
+                       int32_t* req_item_cu, hipStream_t st) {
+  hipLaunchKernelGGL(suffix_plan_kernel, dim3(1), dim3(kPlanThreads), 0, st, lens, B, max_len, lanes,
                      reinterpret_cast<int4*>(items), reinterpret_cast<int4*>(lane_rec), req_item_cu);
   return launch_status();
 }
 
 }  // namespace ph
 
-extern "C" int ph_suffix_plan_build(const int32_t* suffix_lens, int64_t num_reqs, int64_t num_lanes, int32_t* items,
-                                    int32_t* lane_rec, int32_t* req_item_cu, void* stream) {
+extern "C" int ph_suffix_plan_build(const int32_t* suffix_lens, int64_t num_reqs, int64_t max_suffix_len,
+                                    int64_t num_lanes, int32_t* items, int32_t* lane_rec, int32_t* req_item_cu,
+                                    void* stream) {
   if (num_reqs < 0 || num_lanes <= 0 || num_reqs > ph::kPlanMaxReqs || num_lanes > (1 << 20)) return PH_ERR_ARG;
+  if (max_suffix_len < 0 || max_suffix_len > INT32_MAX) return PH_ERR_ARG;
   if (num_reqs == 0) return PH_OK;
   if (!suffix_lens || !items || !lane_rec || !req_item_cu) return PH_ERR_ARG;
-  return ph::launch_suffix_plan(suffix_lens, (int)num_reqs, (int)num_lanes, items, lane_rec, req_item_cu,
-                                (hipStream_t)stream);
+  return ph::launch_suffix_plan(suffix_lens, (int)num_reqs, (int)max_suffix_len, (int)num_lanes, items, lane_rec,
+                                req_item_cu, (hipStream_t)stream);
 }
 
 extern "C" int ph_suffix_tables_append(int32_t* table, int64_t table_stride, int32_t* lens, const int32_t* rows,

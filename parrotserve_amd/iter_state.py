@@ -1,8 +1,9 @@
 """Per-iteration carrier (parrot/engine/builtin/iter_state.py:15-60): built once per
 iteration, shared by every layer's attention call.
 
-    | ---- fill tokens ----- | ---- generation tokens ---- |
-    |    F1   |   F2  |  F3  | G1 | G2 | G3 | G4 | G5 | G6 |
+Token rows of an iteration are packed job after job: first every Fill job's new tokens
+(``num_fill_tokens[j]`` rows for Fill job j, in job order), then one row per Generate job.
+The attention plug-in attaches its index tables to this object in ``init_iteration_state``.
 """
 from __future__ import annotations
 

@@ -92,15 +92,32 @@ def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
 
 
 _workspaces: Dict[Tuple[int, int], torch.Tensor] = {}
+_captured_keys: set = set()               # (device, stream) whose current buffer a captured graph points at
+_pinned_workspaces: List[torch.Tensor] = []  # outgrown buffers that recorded graphs still use
 
 
 def _workspace(nbytes: int, device: torch.device) -> torch.Tensor:
-    """Grow-only scratch buffer per (device, stream); reuse is ordered by the stream."""
+    """Grow-only scratch buffer per (device, stream); reuse is ordered by the stream.
+
+    A buffer handed out while the stream is being captured into a graph is recorded by address in that graph, so
+    it is pinned for the life of the process: growing never frees it (an eager call that needs more gets a new
+    buffer, the recorded graph keeps the old one), and a request made under capture that does not fit the
+    stream's buffer is refused instead of allocating inside the capture."""
     key = (device.index or 0, _stream())
     buf = _workspaces.get(key)
+    capturing = torch.cuda.is_current_stream_capturing()
     if buf is None or buf.numel() < nbytes:
+        if capturing and buf is not None:
+            raise RuntimeError(
+                f"decode workspace of {buf.numel()} bytes is too small for {nbytes} bytes and the stream is being "
+                "captured: run the step once eagerly at its largest shape before capturing it")
+        if buf is not None and key in _captured_keys:
+            _pinned_workspaces.append(buf)  # a recorded graph still points at it
+            _captured_keys.discard(key)
         buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
         _workspaces[key] = buf
+    if capturing:
+        _captured_keys.add(key)
     return buf
 
 
@@ -442,7 +459,8 @@ class DecodeTables:
             self.plan_req_item_cu = buf[o_cu:]
             self.plan = _lib.SuffixPlan(self.plan_items.data_ptr(), cap, self.plan_lane_item_cu.data_ptr(),
                                         num_lanes, self.plan_req_item_cu.data_ptr())
-        suffix_plan_build(self.suffix_lens, num_lanes, self.plan_items, self.plan_lane_item_cu, self.plan_req_item_cu)
+        suffix_plan_build(self.suffix_lens, num_lanes, self.plan_items, self.plan_lane_item_cu, self.plan_req_item_cu,
+                          max_len=self.max_suffix_len)
 
     @staticmethod
     def build(prefix_lists: Sequence[Sequence[int]], group_req_cu: Sequence[int],
@@ -528,15 +546,16 @@ def suffix_tables_append(table: torch.Tensor, lens: torch.Tensor, rows: Optional
 
 
 def suffix_plan_build(lens: torch.Tensor, num_lanes: int, items: torch.Tensor, lane_rec: torch.Tensor,
-                      req_item_cu: torch.Tensor) -> None:
+                      req_item_cu: torch.Tensor, max_len: int = 2 ** 31 - 1) -> None:
     """The balanced suffix plan written on the device from the device length vector (``ph_suffix_plan_build``):
-    ``items [num_lanes + B, 4]``, ``lane_rec [num_lanes, 8]``, ``req_item_cu [B + 1]``, all int32."""
+    ``items [num_lanes + B, 4]``, ``lane_rec [num_lanes, 8]``, ``req_item_cu [B + 1]``, all int32.  Lengths are
+    read clamped to ``[0, max_len]`` (the width of the slot table), as the attention kernels read them."""
     _require_gpu(lens, items, lane_rec, req_item_cu)
     B = lens.numel()
     assert lens.dtype == items.dtype == lane_rec.dtype == req_item_cu.dtype == torch.int32
     assert items.numel() >= (num_lanes + B) * 4 and lane_rec.numel() >= num_lanes * 8 and req_item_cu.numel() >= B + 1
-    check(_lib.load().ph_suffix_plan_build(_ptr(lens), B, num_lanes, _ptr(items), _ptr(lane_rec), _ptr(req_item_cu),
-                                           _stream()), "suffix_plan_build")
+    check(_lib.load().ph_suffix_plan_build(_ptr(lens), B, int(max_len), num_lanes, _ptr(items), _ptr(lane_rec),
+                                           _ptr(req_item_cu), _stream()), "suffix_plan_build")
 
 
 PLAN_MAX_REQS = 8192  # batch size up to which the library plans on the device
@@ -597,9 +616,12 @@ def plan_suffix_items(lens: Sequence[int], num_lanes: int):
 
 
 def decode_attention(query: torch.Tensor, key_cache: torch.Tensor, value_cache: torch.Tensor, tables: DecodeTables,
-                     scale: Optional[float] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     scale: Optional[float] = None, out: Optional[torch.Tensor] = None,
+                     events6=None) -> torch.Tensor:
     """Shared-prefix (or plain ragged) decode attention: prefix phase on the
-    matrix cores, per-request suffix phase, log-sum-exp merge."""
+    matrix cores, per-request suffix phase, log-sum-exp merge.  ``events6``: optional array of six
+    ``hipEvent_t`` handles that receive the begin / end timestamps of the call's prefix, suffix and merge
+    kernels (``ph_decode_attention_timed``)."""
     _require_gpu(query, key_cache, value_cache)
     assert query.dim() == 3 and key_cache.dim() == 3 and value_cache.shape == key_cache.shape
     B, H, D = query.shape
@@ -618,7 +640,7 @@ def decode_attention(query: torch.Tensor, key_cache: torch.Tensor, value_cache: 
     nbytes = lib.ph_decode_workspace_bytes(B, H, D, tables.num_groups, tables.max_prefix_len, tables.max_suffix_len,
                                            tables.chunk_tokens, 0 if plan is None else plan.num_items)
     ws = _workspace(nbytes, query.device)
-    rc = lib.ph_decode_attention(
+    args = (
         _ptr(out), _ptr(query), _ptr(key_cache), _ptr(value_cache), B, H, D, _dtype_code(query),
         query.stride(0), out.stride(0), key_cache.stride(0), float(scale),
         tables.num_groups, _ptr(tables.prefix_slots), _ptr(tables.prefix_cu), _ptr(tables.group_req_cu),
@@ -627,6 +649,7 @@ def decode_attention(query: torch.Tensor, key_cache: torch.Tensor, value_cache: 
         tables.suffix_slots_count(), _ptr(tables.suffix_lens),
         tables.max_suffix_len, tables.chunk_tokens, None if plan is None else ctypes.byref(plan),
         _ptr(ws), ws.numel(), _stream())
+    rc = lib.ph_decode_attention(*args) if events6 is None else lib.ph_decode_attention_timed(*args, events6)
     check(rc, "decode_attention")
     return out
 
@@ -646,10 +669,30 @@ def _single_group_cu(P: int, B: int, device) -> Tuple[torch.Tensor, torch.Tensor
     return hit
 
 
+_identity_head_maps: Dict[Tuple[int, int, int], bool] = {}
+
+
+def _check_head_mapping(head_mapping: torch.Tensor, num_heads: int) -> None:
+    """``head_mapping[h]`` names the KV head of query head h (3rdparty/vllm/csrc/attention/attention_kernels.cu:
+    ``kv_head_idx = head_mapping[head_idx]``).  The reference's models always pass ``arange(num_heads)``
+    (models/llama.py:95-97); the kernels here read KV head h for query head h, so anything else is refused rather
+    than silently ignored.  The contents are checked once per tensor (address and version): one small copy to the
+    host the first time a mapping is seen."""
+    assert head_mapping.shape[0] == num_heads, "head_mapping must have one entry per head"
+    key = (head_mapping.data_ptr(), head_mapping._version, num_heads)
+    if key in _identity_head_maps:
+        return
+    if not torch.equal(head_mapping.detach().cpu().to(torch.int64), torch.arange(num_heads)):
+        raise ValueError("head_mapping must be arange(num_heads): grouped / multi-query KV heads are not supported")
+    if len(_identity_head_maps) > 64:
+        _identity_head_maps.clear()
+    _identity_head_maps[key] = True
+
+
 def _check_paged_args(query, key_cache, value_cache, head_mapping, context_lens, block_tables):
     if key_cache.dim() != 3 or value_cache.dim() != 3:
         raise ValueError("key_cache / value_cache must be token-granular [slots, H, D] (block_size 1)")
-    assert head_mapping.shape[0] == query.shape[1], "head_mapping must have one entry per head (MQA/GQA unsupported)"
+    _check_head_mapping(head_mapping, query.shape[1])
     assert block_tables.dim() == 2 and block_tables.dtype == torch.int32
     assert context_lens.dtype == torch.int32 and context_lens.shape[0] == query.shape[0]
     assert block_tables.shape[0] == query.shape[0]
@@ -690,10 +733,43 @@ def flash_paged_attention(query, key_cache, value_cache, head_mapping, flash_con
 
 def paged_flash_attention(query, key_cache, value_cache, head_mapping, flash_context_len, flash_block_table,
                           paged_context_lens, paged_block_tables):
-    """Same result with the phases in the other order in the reference
-    (shared_flash_decoding.py:332-376); here both names run the same launches."""
-    return flash_paged_attention(query, key_cache, value_cache, head_mapping, flash_context_len, flash_block_table,
-                                 paged_context_lens, paged_block_tables)
+    """The phases in the other order, as in the reference (shared_flash_decoding.py:332-376): the suffix phase
+    first, exporting its row maxima and denominators (``single_query_cached_kv_prev_attention``), then the prefix
+    phase merged on top of it in place (the Triton kernel with ``load_mid_results``) -- two calls of the library,
+    ``ph_suffix_prev_attention`` and ``ph_prefix_post_attention``.  Same result as ``flash_paged_attention``."""
+    _check_paged_args(query, key_cache, value_cache, head_mapping, paged_context_lens, paged_block_tables)
+    _require_gpu(query, key_cache, value_cache, paged_context_lens, paged_block_tables)
+    B, H, D = query.shape
+    assert key_cache.shape[1:] == (H, D) and value_cache.shape == key_cache.shape
+    assert query.dtype == key_cache.dtype == value_cache.dtype
+    assert query.stride(2) == 1 and query.stride(1) == D
+    assert key_cache.stride(2) == 1 and key_cache.stride(1) == D and key_cache.stride() == value_cache.stride()
+    out = torch.empty((B, H, D), dtype=query.dtype, device=query.device)
+    if B == 0:
+        return out
+    P = int(flash_context_len)
+    table = paged_block_tables if paged_block_tables.stride(1) == 1 else paged_block_tables.contiguous()
+    lens = paged_context_lens.contiguous()
+    width = table.shape[1]
+    lib = _lib.load()
+    scale = D ** -0.5
+    m = torch.empty((B, H), dtype=torch.float32, device=query.device)
+    l = torch.empty((B, H), dtype=torch.float32, device=query.device)
+    nbytes = max(lib.ph_decode_workspace_bytes(B, H, D, 0, 0, width, 0, 0),
+                 lib.ph_decode_workspace_bytes(B, H, D, 1 if P > 0 else 0, P, 0, 0, 0))
+    ws = _workspace(nbytes, query.device)
+    code, st = _dtype_code(query), _stream()
+    check(lib.ph_suffix_prev_attention(
+        _ptr(out), _ptr(m), _ptr(l), _ptr(query), _ptr(key_cache), _ptr(value_cache), B, H, D, code,
+        query.stride(0), out.stride(0), key_cache.stride(0), float(scale), _ptr(table), None, table.stride(0),
+        (B - 1) * table.stride(0) + width, _ptr(lens), width, 0, _ptr(ws), ws.numel(), st), "paged_flash_attention")
+    if P > 0:
+        assert flash_block_table.dtype == torch.int32 and flash_block_table.numel() >= P
+        check(lib.ph_prefix_post_attention(
+            _ptr(out), _ptr(m), _ptr(l), _ptr(query), _ptr(key_cache), _ptr(value_cache), B, H, D, code,
+            query.stride(0), out.stride(0), key_cache.stride(0), float(scale), _ptr(flash_block_table.contiguous()), P,
+            _ptr(ws), ws.numel(), st), "paged_flash_attention")
+    return out
 
 
 # --------------------------------------------------------------------------- #

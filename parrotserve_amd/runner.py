@@ -79,8 +79,9 @@ class EngineContextManager:
 class Sampler(nn.Module):
     """Temperature, top-p, one draw per row over ``hidden @ lm_head.T`` (models/sampler.py:19-66).  Everything
     after the logits GEMM is one kernel (``ph_sample_top_p``): the reference's two sorts become a threshold search
-    and its ``torch.multinomial`` an inverse-CDF draw from ``torch.rand`` numbers, so the tokens follow torch's
-    generator (same seed, same tokens) with the reference's distribution."""
+    and its ``torch.multinomial`` an inverse-CDF draw from ``torch.rand`` numbers: the tokens are deterministic
+    in torch's generator (same seed, same tokens from run to run) and follow the reference's distribution, but for a
+    given seed they are NOT the ids the reference's ``torch.multinomial`` call would draw."""
 
     def __init__(self, config: LlamaConfig, embd_weight: torch.Tensor):
         super().__init__()

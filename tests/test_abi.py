@@ -29,7 +29,7 @@ def test_status_strings_and_version():
     from parrotserve_amd import _lib
 
     lib = _lib.load()
-    assert lib.ph_abi_version() >= 1
+    assert lib.ph_abi_version() >= 2
     assert _lib.status_string(0) == "ok"
     assert "head size" in _lib.status_string(_lib.PH_ERR_HEAD_DIM)
     with pytest.raises(RuntimeError):
@@ -87,10 +87,11 @@ def test_argument_validation_needs_no_gpu():
     gv = lambda n, bs: lib.ph_gather_blocked_v(None, None, None, None, 0, n, 2, 128, bs, 2, 4096, 2048, 16, 1, 256, 128,
                                                1, None)
     assert gv(4, 16) == _lib.PH_ERR_ARG and gv(0, 16) == _lib.PH_OK and gv(4, 0) == _lib.PH_ERR_ARG
-    assert lib.ph_suffix_plan_build(None, 4, 256, None, None, None, None) == _lib.PH_ERR_ARG      # null pointers
-    assert lib.ph_suffix_plan_build(None, 0, 256, None, None, None, None) == _lib.PH_OK           # no requests
-    assert lib.ph_suffix_plan_build(None, 8193, 256, None, None, None, None) == _lib.PH_ERR_ARG   # beyond the device planner
-    assert lib.ph_suffix_plan_build(None, 4, 0, None, None, None, None) == _lib.PH_ERR_ARG
+    assert lib.ph_suffix_plan_build(None, 4, 512, 256, None, None, None, None) == _lib.PH_ERR_ARG      # null pointers
+    assert lib.ph_suffix_plan_build(None, 0, 512, 256, None, None, None, None) == _lib.PH_OK           # no requests
+    assert lib.ph_suffix_plan_build(None, 8193, 512, 256, None, None, None, None) == _lib.PH_ERR_ARG   # beyond the device planner
+    assert lib.ph_suffix_plan_build(None, 4, 512, 0, None, None, None, None) == _lib.PH_ERR_ARG
+    assert lib.ph_suffix_plan_build(None, 4, -1, 256, None, None, None, None) == _lib.PH_ERR_ARG       # negative bound
     assert lib.ph_sample_top_p(None, 32000, None, None, None, None, 4, 32000, 0, None) == _lib.PH_ERR_ARG  # null pointers
     assert lib.ph_sample_top_p(None, 32000, None, None, None, None, 0, 32000, 2, None) == _lib.PH_OK       # no rows
     assert lib.ph_sample_top_p(None, 32000, None, None, None, None, 4, 32000, 7, None) == _lib.PH_ERR_DTYPE

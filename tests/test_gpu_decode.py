@@ -251,6 +251,51 @@ def test_reference_named_entry_points(dev):
     torch.testing.assert_close(out1.float(), ref.float(), **TOL[torch.float16])
 
 
+def test_head_mapping_must_be_identity(dev):
+    """A mapping other than arange(H) (grouped KV heads) is refused, not silently ignored."""
+    from parrotserve_amd import kernels
+
+    B, H, D = 2, 4, 128
+    q = torch.zeros(B, H, D, dtype=torch.float16, device=dev)
+    kc = torch.zeros(8, H, D, dtype=torch.float16, device=dev)
+    table = torch.zeros(B, 4, dtype=torch.int32, device=dev)
+    lens = torch.full((B,), 2, dtype=torch.int32, device=dev)
+    gqa = torch.tensor([0, 0, 1, 1], dtype=torch.int32, device=dev)
+    for fn in (lambda hm: kernels.vllm_paged_attention(q, kc, kc, hm, lens, table),
+               lambda hm: kernels.flash_paged_attention(q, kc, kc, hm, 0, table[0, :0], lens, table),
+               lambda hm: kernels.paged_flash_attention(q, kc, kc, hm, 0, table[0, :0], lens, table)):
+        with pytest.raises(ValueError, match="head_mapping"):
+            fn(gqa)
+        fn(torch.arange(H, dtype=torch.int32, device=dev))
+
+
+@pytest.mark.parametrize("balanced", [True, False])
+def test_lengths_beyond_the_table_are_clamped(dev, balanced):
+    """A context length larger than the table's width must not walk into the next request's row (or past the
+    table): the kernels read it clamped to the width, so the result is that of the full row."""
+    from parrotserve_amd import kernels
+
+    g = torch.Generator().manual_seed(31)
+    B, H, D, W = 6, 4, 128, 24
+    k = torch.randn(B * W, H, D, generator=g).half()
+    v = torch.randn(B * W, H, D, generator=g).half()
+    q = torch.randn(B, H, D, generator=g).half()
+    rows = torch.randperm(B * W, generator=g).view(B, W)
+    good = torch.tensor([W, 5, W, 1, 17, W], dtype=torch.int32)
+    bad = good.clone()
+    bad[0], bad[2], bad[5] = W + 9, 100000, 2 ** 31 - 1
+    ref = ref_decode_attention(q, k, v, [rows[b, : int(good[b])] for b in range(B)])
+    table = rows.to(torch.int32).to(dev)
+    hm = torch.arange(H, dtype=torch.int32, device=dev)
+    if balanced:
+        out = kernels.vllm_paged_attention(q.to(dev), k.to(dev), v.to(dev), hm, bad.to(dev), table)
+    else:
+        t = kernels.DecodeTables(num_reqs=B, suffix_slots=table, suffix_table_stride=W, suffix_lens=bad.to(dev),
+                                 max_suffix_len=W, chunk_tokens=16)
+        out = kernels.decode_attention(q.to(dev), k.to(dev), v.to(dev), t)
+    torch.testing.assert_close(out.cpu().float(), ref.float(), **TOL[torch.float16])
+
+
 @pytest.mark.parametrize("B,grouped", [(8192, True), (8193, False), (9000, True)])
 def test_batches_around_the_device_planner_limit(dev, B, grouped):
     """The suffix plan is written on the device for up to 8192 requests and on the host beyond; thousands of

@@ -138,6 +138,38 @@ def test_move_from_blocked_equals_token_move_at_scale(dev):
         assert torch.equal(got.view(torch.int16), want.view(torch.int16))
 
 
+@pytest.mark.parametrize("idx_dtype", [torch.int64, torch.int32])
+def test_config3_token_move_full_size(dev, idx_dtype):
+    """Config 3's move at its own size: 65,536 random source rows to 65,536 other rows of one 4M-slot pool
+    (32 x 128 fp16, 8 KB rows), bit-exact against the oracle on the touched rows, and every other row of the pool
+    unchanged.  The oracle runs on the compacted rows (source rows first, then the destinations' old contents)
+    with the indices renumbered to match; the pool itself only exists on the device (34 GB)."""
+    from parrotserve_amd import kernels, synth
+
+    pool, H, D = 1 << 22, 32, 128
+    src, dst = synth.config3_move(index_dtype=idx_dtype)
+    n = src.numel()
+    assert n == 65536 and src.dtype == idx_dtype and torch.unique(dst).numel() == n
+    assert not torch.isin(dst.long(), src.long()).any()
+    gen = torch.Generator(device=dev).manual_seed(5)
+    kc = torch.randn((pool, H, D), generator=gen, device=dev, dtype=torch.float16)
+    before = kc.clone()
+    sd, dd = src.to(dev), dst.to(dev)
+    compact = torch.cat([before[sd.long()], before[dd.long()]]).cpu()  # [2n, H, D]
+    ref_move_tokens(compact, compact, torch.arange(n), n + torch.arange(n))
+    kernels.discontinuous_move_tokens(kc, kc, sd, dd)
+    torch.cuda.synchronize()
+    assert torch.equal(_bits(kc[dd.long()].cpu()), _bits(compact[n:]))
+    # everything but the destination rows is what it was (compared as bits, in slices of 256K rows)
+    before[dd.long()] = kc[dd.long()]
+    a, b = kc.view(torch.int16), before.view(torch.int16)
+    step = 1 << 18
+    for r in range(0, pool, step):
+        assert torch.equal(a[r:r + step], b[r:r + step]), f"rows {r}..{r + step} changed"
+    del kc, before, a, b
+    torch.cuda.empty_cache()
+
+
 def test_move_tokens_reference_selftest_shape(dev):
     """tokens_moving.py:316-362: H 96 x D 128 fp16, random src rows to every second dest row (scaled-down count)."""
     from parrotserve_amd import kernels
