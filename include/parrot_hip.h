@@ -38,7 +38,8 @@ enum {
   PH_ERR_ALIGN = 3,     /* pointer or stride not aligned as the kernel needs */
   PH_ERR_ARG = 4,       /* inconsistent sizes, null pointer, negative count */
   PH_ERR_WORKSPACE = 5, /* workspace too small */
-  PH_ERR_LAUNCH = 6     /* hipLaunchKernel reported an error */
+  PH_ERR_LAUNCH = 6,    /* hipLaunchKernel reported an error */
+  PH_ERR_SCRATCH = 7    /* the shape needs more scratch than the library's own fixed array holds */
 };
 
 const char* ph_status_string(int status);
@@ -240,6 +241,35 @@ int ph_decode_attention(void* out, const void* q, const void* k_cache, const voi
                         int64_t max_suffix_len, int64_t chunk_tokens,
                         const ph_suffix_plan* plan,
                         void* workspace, size_t workspace_bytes, void* stream);
+
+/* ph_decode_attention without a workspace argument, for callers that cannot
+ * allocate device memory (code under HIP graph capture, serving loops with a
+ * fixed memory plan, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference, whose launcher lets torch allocate its temporaries
+ * (shared_flash_decoding.py:298-313).  Same arguments, same kernels, same
+ * results; the partials live in an array of ph_decode_static_scratch_bytes()
+ * (32 MiB) that the library holds on every device it runs on until the process
+ * ends.  The call allocates and frees nothing.  A shape whose
+ * ph_decode_workspace_bytes() exceeds the array returns PH_ERR_SCRATCH before
+ * anything is launched (config 2, batch 64 x 32 x 128 with a 4096-token prefix,
+ * needs 13.9 MB; config 5, 128 x 40 x 128 in four groups, 15 MB).  All calls on
+ * one device share the array: calls that overlap on one device (two streams,
+ * two threads) race on it -- serialise them, or use ph_decode_attention with a
+ * workspace per stream. */
+size_t ph_decode_static_scratch_bytes(void);
+
+int ph_decode_attention_static(void* out, const void* q, const void* k_cache, const void* v_cache,
+                               int64_t num_reqs, int64_t num_heads, int64_t head_dim, int dtype,
+                               int64_t q_stride, int64_t out_stride, int64_t cache_stride_n,
+                               float scale,
+                               int64_t num_groups, const int32_t* prefix_slots, const int32_t* prefix_cu,
+                               const int32_t* group_req_cu, const int32_t* group_req_cu_host,
+                               int64_t max_prefix_len,
+                               const int32_t* suffix_slots, const int64_t* suffix_offsets,
+                               int64_t suffix_table_stride, int64_t suffix_slots_count,
+                               const int32_t* suffix_lens,
+                               int64_t max_suffix_len, int64_t chunk_tokens,
+                               const ph_suffix_plan* plan, void* stream);
 
 /* The two halves of the shared-prefix op, exposed separately because the
  * reference's extension does (csrc/attention.cpp:19-47):

@@ -16,7 +16,7 @@ LIB_PATH = os.path.join(PKG_DIR, "libparrot_hip.so")
 
 PH_F16, PH_BF16, PH_F32 = 0, 1, 2
 PH_IDX_I32, PH_IDX_I64 = 0, 1
-PH_OK, PH_ERR_DTYPE, PH_ERR_HEAD_DIM, PH_ERR_ALIGN, PH_ERR_ARG, PH_ERR_WORKSPACE, PH_ERR_LAUNCH = range(7)
+PH_OK, PH_ERR_DTYPE, PH_ERR_HEAD_DIM, PH_ERR_ALIGN, PH_ERR_ARG, PH_ERR_WORKSPACE, PH_ERR_LAUNCH, PH_ERR_SCRATCH = range(8)
 
 P, I, L, F, Z = c_void_p, c_int, c_int64, c_float, c_size_t
 
@@ -41,6 +41,8 @@ SIGNATURES: Dict[str, Tuple[object, List[object]]] = {
     "ph_silu_mul": (I, [P, P, P, L, L, L, L, L, I, P]),
     "ph_rope_append": (I, [P, P, P, P, P, P, P, P, I, L, L, L, L, L, L, L, L, L, I, P]),
     "ph_suffix_tables_append": (I, [P, L, P, P, P, L, P]),
+    "ph_decode_static_scratch_bytes": (Z, []),
+    "ph_decode_attention_static": (I, [P, P, P, P, L, L, L, I, L, L, L, F, L, P, P, P, P, L, P, P, L, L, P, L, L, P, P]),
     "ph_decode_attention_timed": (I, [P, P, P, P, L, L, L, I, L, L, L, F, L, P, P, P, P, L, P, P, L, L, P, L, L, P, P, Z, P, P]),
     "ph_suffix_plan_build": (I, [P, L, L, L, P, P, P, P]),
     "ph_sample_top_p": (I, [P, L, P, P, P, P, L, L, I, P]),

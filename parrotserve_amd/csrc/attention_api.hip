@@ -3,7 +3,34 @@
 // enqueued on the caller's stream.
 #include "decode.hpp"
 
+#include <mutex>
+
 namespace ph {
+
+// Scratch of ph_decode_attention_static: the partials workspace of a decode call, held by the library for
+// callers that cannot allocate.  Every device the library runs on holds its own copy until the process ends.
+constexpr size_t kStaticScratchBytes = (size_t)32 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+// Device address of `scratch` on the current device.  The array's name is a host-side stand-in for the symbol,
+// not an address a kernel can use: the address is asked for once per device and kept.
+static int static_scratch_ptr(void** out) {
+  static std::mutex mu;
+  static void* ptrs[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return PH_ERR_ARG;
+  std::lock_guard<std::mutex> lock(mu);
+  if (!ptrs[dev]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) {
+      (void)hipGetLastError();
+      return PH_ERR_LAUNCH;
+    }
+    ptrs[dev] = p;
+  }
+  *out = ptrs[dev];
+  return PH_OK;
+}
 
 struct DecodePlan {
   int chunk;         // suffix tokens per part (grid form)
@@ -236,6 +263,7 @@ extern "C" const char* ph_status_string(int status) {
     case PH_ERR_ARG: return "invalid argument";
     case PH_ERR_WORKSPACE: return "workspace too small";
     case PH_ERR_LAUNCH: return "kernel launch failed";
+    case PH_ERR_SCRATCH: return "shape needs more scratch than the library's static array holds (use the workspace form)";
     default: return "unknown status";
   }
 }
@@ -428,6 +456,34 @@ extern "C" int ph_decode_attention(void* out, const void* q, const void* k_cache
                                group_req_cu_host, max_prefix_len, suffix_slots, suffix_offsets, suffix_table_stride,
                                suffix_slots_count, suffix_lens, max_suffix_len, chunk_tokens, plan, workspace,
                                workspace_bytes, stream, nullptr);
+}
+
+extern "C" size_t ph_decode_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+extern "C" int ph_decode_attention_static(void* out, const void* q, const void* k_cache, const void* v_cache,
+                                          int64_t num_reqs, int64_t num_heads, int64_t head_dim, int dtype,
+                                          int64_t q_stride, int64_t out_stride, int64_t cache_stride_n, float scale,
+                                          int64_t num_groups, const int32_t* prefix_slots, const int32_t* prefix_cu,
+                                          const int32_t* group_req_cu, const int32_t* group_req_cu_host,
+                                          int64_t max_prefix_len, const int32_t* suffix_slots,
+                                          const int64_t* suffix_offsets, int64_t suffix_table_stride,
+                                          int64_t suffix_slots_count, const int32_t* suffix_lens,
+                                          int64_t max_suffix_len, int64_t chunk_tokens, const ph_suffix_plan* plan,
+                                          void* stream) {
+  // the same sizing as ph_decode_workspace_bytes; a shape whose partials do not fit the array is refused
+  if (num_reqs > 0 && num_heads > 0 && head_dim > 0) {
+    const size_t need = ph_decode_workspace_bytes(num_reqs, num_heads, head_dim, num_groups, max_prefix_len,
+                                                  max_suffix_len, chunk_tokens, plan ? plan->num_items : 0);
+    if (need > kStaticScratchBytes) return PH_ERR_SCRATCH;
+  }
+  void* ws = nullptr;
+  const int rc = static_scratch_ptr(&ws);
+  if (rc != PH_OK) return rc;
+  return decode_attention_impl(out, q, k_cache, v_cache, num_reqs, num_heads, head_dim, dtype, q_stride, out_stride,
+                               cache_stride_n, scale, num_groups, prefix_slots, prefix_cu, group_req_cu,
+                               group_req_cu_host, max_prefix_len, suffix_slots, suffix_offsets, suffix_table_stride,
+                               suffix_slots_count, suffix_lens, max_suffix_len, chunk_tokens, plan, ws,
+                               kStaticScratchBytes, stream, nullptr);
 }
 
 extern "C" int ph_decode_attention_timed(void* out, const void* q, const void* k_cache, const void* v_cache,

@@ -37,6 +37,7 @@ __all__ = [
     "DecodeTables",
     "PrefillTables",
     "decode_attention",
+    "decode_attention_static",
     "prefill_attention",
     "kv_append",
 ]
@@ -651,6 +652,34 @@ def decode_attention(query: torch.Tensor, key_cache: torch.Tensor, value_cache: 
         _ptr(ws), ws.numel(), _stream())
     rc = lib.ph_decode_attention(*args) if events6 is None else lib.ph_decode_attention_timed(*args, events6)
     check(rc, "decode_attention")
+    return out
+
+
+def decode_attention_static(query: torch.Tensor, key_cache: torch.Tensor, value_cache: torch.Tensor,
+                            tables: DecodeTables, out: torch.Tensor, scale: Optional[float] = None) -> torch.Tensor:
+    """``decode_attention`` on the library's own fixed scratch array (``ph_decode_attention_static``): nothing is
+    allocated, here or in the library, so ``out`` must be given.  Shapes whose partials exceed the array raise
+    ``RuntimeError``; calls that overlap on one device share the array and must be serialised by the caller."""
+    _require_gpu(query, key_cache, value_cache, out)
+    B, H, D = query.shape
+    assert B == tables.num_reqs and out.shape == query.shape and out.dtype == query.dtype
+    assert key_cache.shape[1:] == (H, D) and value_cache.shape == key_cache.shape
+    assert query.dtype == key_cache.dtype == value_cache.dtype
+    assert query.stride(2) == 1 and query.stride(1) == D and out.stride(2) == 1 and out.stride(1) == D
+    assert key_cache.stride(2) == 1 and key_cache.stride(1) == D and key_cache.stride() == value_cache.stride()
+    if B == 0:
+        return out
+    scale = D ** -0.5 if scale is None else scale
+    plan = tables.plan
+    rc = _lib.load().ph_decode_attention_static(
+        _ptr(out), _ptr(query), _ptr(key_cache), _ptr(value_cache), B, H, D, _dtype_code(query),
+        query.stride(0), out.stride(0), key_cache.stride(0), float(scale),
+        tables.num_groups, _ptr(tables.prefix_slots), _ptr(tables.prefix_cu), _ptr(tables.group_req_cu),
+        _ptr(tables.group_req_cu_host), tables.max_prefix_len,
+        _ptr(tables.suffix_slots), _ptr(tables.suffix_offsets), tables.suffix_table_stride,
+        tables.suffix_slots_count(), _ptr(tables.suffix_lens),
+        tables.max_suffix_len, tables.chunk_tokens, None if plan is None else ctypes.byref(plan), _stream())
+    check(rc, "decode_attention_static")
     return out
 
 

@@ -102,6 +102,18 @@ def test_argument_validation_needs_no_gpu():
     assert lib.ph_suffix_tables_append(None, 64, None, None, None, 3, None) == _lib.PH_ERR_ARG
 
 
+def test_static_scratch_entry_point_refuses_oversize_without_a_gpu():
+    """The size check of ph_decode_attention_static comes before anything touches the device."""
+    from parrotserve_amd import _lib
+
+    lib = _lib.load()
+    assert lib.ph_decode_static_scratch_bytes() == 32 << 20
+    assert lib.ph_decode_workspace_bytes(64, 32, 128, 1, 4096, 512, 0, 320) < lib.ph_decode_static_scratch_bytes()
+    rc = lib.ph_decode_attention_static(1, 1, 1, 1, 4096, 32, 128, 0, 4096, 4096, 4096, 1.0, 0, None, None, None, None,
+                                        0, 1, None, 8192, 4096 * 8192, 1, 8192, 32, None, None)
+    assert rc == _lib.PH_ERR_SCRATCH and "scratch" in _lib.status_string(rc)
+
+
 def test_cpu_tensors_are_refused_loudly():
     import torch
 
