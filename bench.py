@@ -241,6 +241,47 @@ def extras(torch, dev):
     return out
 
 
+TIMELINE_MARKS = ["kernel entry", "prefix slot window in LDS", "prefix ring requested, suffix stream starts",
+                  "suffix stream done", "prefix step 0 (tile landed, workgroup barrier passed)", "prefix step 1",
+                  "prefix step 2", "prefix step 3", "prefix main loop done", "token groups folded",
+                  None, "kernel exit"]
+
+
+def fused_timeline(torch, lib, step, launches=8):
+    """Per-wave timestamps at the marks of the fused prefix + suffix kernel (profiling variant of the library), in
+    microseconds from the first wave's entry; the median over the launches of every wave's time, then its spread
+    over the 2048 waves.  The marks cost a store each: the instrumented kernel runs about 2 us longer."""
+    import numpy as np
+
+    for i in range(16):
+        step(i)
+    torch.cuda.synchronize()
+    runs = []
+    for i in range(launches):
+        lib.ph_timeline_clear()
+        torch.cuda.synchronize()
+        step(i)
+        torch.cuda.synchronize()
+        buf = np.zeros(4096 * 12, dtype=np.uint64)
+        assert lib.ph_timeline_read(buf.ctypes.data_as(ctypes.c_void_p), buf.nbytes) == 0
+        t = buf.reshape(4096, 12).astype(np.float64)
+        t = t[t[:, 0] > 0]
+        runs.append(np.where(t > 0, (t - t[:, 0].min()) / 100.0, np.nan))
+    rel = np.nanmedian(np.stack(runs), axis=0)
+    out = {"waves": int(rel.shape[0]), "unit": "us from the first wave's entry", "marks": {}}
+    for i, name in enumerate(TIMELINE_MARKS):
+        c = rel[:, i]
+        c = c[~np.isnan(c)]
+        if name is None or c.size == 0:
+            continue
+        out["marks"][name] = {k: round(float(v), 2) for k, v in
+                              zip(("min", "p10", "p50", "p90", "max"), np.percentile(c, [0, 10, 50, 90, 100]))}
+    wg = rel.reshape(-1, 8, 12)
+    out["suffix_done_spread_inside_workgroup_p50"] = round(float(np.nanmedian(wg[:, :, 3].max(1) - wg[:, :, 3].min(1))), 2)
+    out["exit_by_xcd_p50"] = [round(float(np.nanmedian(wg[x::8, :, 11].max(1))), 2) for x in range(8)]
+    return out
+
+
 def head_size_64_step(torch, dev):
     """Config 2's batch with 64-wide heads (32 x 64, the OPT-1.3B shape): the prefix phase runs on head pairs through
     the 128-wide matrix-core kernel, the suffix phase and the merge at the native width.  Warm (one KV set)."""
@@ -516,6 +557,9 @@ def main():
                          "of a whole engine iteration)")
     ap.add_argument("--sampler-only", action="store_true",
                     help="only time the token sampler (kernel and the reference's library-call sequence) and exit")
+    ap.add_argument("--timeline", action="store_true",
+                    help="only record where the waves of the fused decode kernel spend their time (needs the "
+                         "profiling variant of the library, built beside the product one) and exit")
     ap.add_argument("--prefill-only", action="store_true",
                     help="only run config 4's prefill kernel a few times (for profiler counter passes) and exit")
     args = ap.parse_args()
@@ -528,6 +572,10 @@ def main():
 
     from parrotserve_amd import _lib, kernels, synth
 
+    if args.timeline:  # before the first load(): this run binds the profiling variant of the library
+        from parrotserve_amd import build as _build
+
+        _lib.LIB_PATH = _build.TIMELINE_LIB_PATH
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     lib = _lib.load()
@@ -605,6 +653,10 @@ def main():
             fn(i)
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / steps
+
+    if args.timeline:
+        print(json.dumps({"fused_kernel_timeline": fused_timeline(torch, lib, step)}))
+        return
 
     t_step = timed(step, args.steps, args.warmup)
     t_warm = timed(lambda i: kernels.decode_attention(qs[0], kc, vc, tables[0], out=out), args.steps, args.warmup)

@@ -77,6 +77,11 @@ def load() -> ctypes.CDLL:
         fn = getattr(lib, name)  # AttributeError if the symbol is not exported
         fn.restype = res
         fn.argtypes = args
+    if hasattr(lib, "ph_timeline_read"):  # profiling variant of the library (build.TIMELINE_LIB_PATH)
+        lib.ph_timeline_read.restype = c_int
+        lib.ph_timeline_read.argtypes = [c_void_p, c_size_t]
+        lib.ph_timeline_clear.restype = c_int
+        lib.ph_timeline_clear.argtypes = []
     _lib = lib
     return lib
 

@@ -14,6 +14,8 @@ from concurrent.futures import ThreadPoolExecutor
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libparrot_hip.so")
+# profiling variant: the same sources with the fused decode kernel's timeline marks switched on (csrc/timeline.hpp)
+TIMELINE_LIB_PATH = os.path.join(PKG_DIR, "libparrot_hip_timeline.so")
 SOURCES = ["move_tokens.hip", "gather_blocked.hip", "norm_rope.hip", "fused.hip", "sampler.hip", "tables.hip", "decode.hip", "prefix_mfma.hip", "attention_api.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -31,9 +33,10 @@ FLAGS = [
 EXTRA_FLAGS = {"prefix_mfma.hip": ["-fno-honor-nans"]}
 
 
-def _compile(src: str, obj_dir: str) -> str:
-    obj = os.path.join(obj_dir, src.replace(".hip", ".o"))
-    cmd = [HIPCC, *FLAGS, *EXTRA_FLAGS.get(src, []), "-c", os.path.join(CSRC, src), "-o", obj]
+def _compile(src: str, obj_dir: str, timeline: bool = False) -> str:
+    obj = os.path.join(obj_dir, src.replace(".hip", ".timeline.o" if timeline else ".o"))
+    extra = ["-include", os.path.join(CSRC, "timeline.hpp")] if timeline else []
+    cmd = [HIPCC, *FLAGS, *EXTRA_FLAGS.get(src, []), *extra, "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{r.stdout}\n{r.stderr}")
@@ -51,6 +54,15 @@ def build(verbose: bool = True) -> str:
         raise RuntimeError(f"link failed:\n{r.stdout}\n{r.stderr}")
     if verbose:
         print(f"built {LIB_PATH}")
+    # the profiling variant shares every object but the one that holds the marks
+    tl_obj = _compile("prefix_mfma.hip", obj_dir, timeline=True)
+    tl_objs = [tl_obj if o.endswith("prefix_mfma.o") else o for o in objs]
+    r = subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", TIMELINE_LIB_PATH, *tl_objs],
+                       capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"link failed:\n{r.stdout}\n{r.stderr}")
+    if verbose:
+        print(f"built {TIMELINE_LIB_PATH}")
     return LIB_PATH
 
 

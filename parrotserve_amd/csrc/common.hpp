@@ -172,6 +172,12 @@ struct HeadLanes {
   static __device__ __forceinline__ int chunk(int lane) { return active(lane) ? lane % LPH : 0; }
 };
 
+// Timeline marks of the decode kernels: nothing unless a profiling build defines PH_TL(i) (it then records a
+// timestamp per wave at mark i).
+#ifndef PH_TL
+#define PH_TL(i)
+#endif
+
 inline int launch_status() { return hipGetLastError() == hipSuccess ? PH_OK : PH_ERR_LAUNCH; }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

@@ -20,49 +20,85 @@ __device__ __forceinline__ float block_sum_256(float v, float* red) {
   return red[0] + red[1] + red[2] + red[3];
 }
 
-// One workgroup per row; ITERS 16-byte chunks per thread are kept in registers.
-template <typename E, int ITERS, bool ROUND_FIRST>
+// One workgroup per ROWS consecutive rows; ITERS 16-byte chunks per thread and row are kept in registers.  The
+// rows' loads and the weights' are all requested before the first reduction, so a workgroup has ROWS rows in
+// flight and pays the load -> reduce -> store chain once per round.  Measured at 8192 x 5120 fp16: three rows per
+// workgroup 29.6 us (71 % of HBM peak) against 31.4 us with one, 32 us with four; with one row per workgroup the
+// weights are better read behind the reduction (31.4 against 35 us), with three ahead of it (29.6 against 31.4).
+template <typename E, int ITERS, bool ROUND_FIRST, int ROWS>
 __global__ __launch_bounds__(kNormThreads) void rms_norm_vec(uint16_t* __restrict__ out,
                                                              const uint16_t* __restrict__ x,
                                                              const uint16_t* __restrict__ w, float eps,
-                                                             int n, int64_t x_stride, int64_t out_stride) {
-  __shared__ float red[4];
-  const int64_t row = blockIdx.x;
-  const uint16_t* xr = x + row * x_stride;
-  uint16_t* orow = out + row * out_stride;
+                                                             int n, int64_t rows, int64_t x_stride,
+                                                             int64_t out_stride) {
+  __shared__ float red[ROWS][4];
+  const int64_t row0 = (int64_t)blockIdx.x * ROWS;
   const int chunks = n >> 3;
-  u32x4 v[ITERS];
-  float ss = 0.f;
+  u32x4 v[ROWS][ITERS], wv[ITERS];
+  float ss[ROWS];
 #pragma unroll
-  for (int i = 0; i < ITERS; ++i) {
-    const int c = threadIdx.x + i * kNormThreads;
-    if (c < chunks) {
-      v[i] = ld16_nt(xr + c * 8);
+  for (int r = 0; r < ROWS; ++r) {
+    const uint16_t* xr = x + (row0 + r < rows ? row0 + r : rows - 1) * x_stride;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const float a = Elem<E>::lo(v[i][j]), b = Elem<E>::hi(v[i][j]);
-        ss += a * a + b * b;
-      }
+    for (int i = 0; i < ITERS; ++i) {
+      const int c = threadIdx.x + i * kNormThreads;
+      if (c < chunks) v[r][i] = ld16_nt(xr + c * 8);
     }
   }
-  ss = block_sum_256(ss, red);
-  const float rstd = rsqrtf(ss / (float)n + eps);
+  if (ROWS > 1) {
 #pragma unroll
-  for (int i = 0; i < ITERS; ++i) {
-    const int c = threadIdx.x + i * kNormThreads;
-    if (c < chunks) {
-      const u32x4 wv = ld16(w + c * 8);
-      u32x4 o;
+    for (int i = 0; i < ITERS; ++i) {
+      const int c = threadIdx.x + i * kNormThreads;
+      if (c < chunks) wv[i] = ld16(w + c * 8);
+    }
+  }
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        float a = Elem<E>::lo(v[i][j]) * rstd, b = Elem<E>::hi(v[i][j]) * rstd;
-        if (ROUND_FIRST) {
-          a = rnd<E>(a);
-          b = rnd<E>(b);
+  for (int r = 0; r < ROWS; ++r) {
+    ss[r] = 0.f;
+#pragma unroll
+    for (int i = 0; i < ITERS; ++i) {
+      const int c = threadIdx.x + i * kNormThreads;
+      if (c < chunks) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float a = Elem<E>::lo(v[r][i][j]), b = Elem<E>::hi(v[r][i][j]);
+          ss[r] += a * a + b * b;
         }
-        o[j] = pack2<E>(a * Elem<E>::lo(wv[j]), b * Elem<E>::hi(wv[j]));
       }
-      st16(orow + c * 8, o);
+    }
+    ss[r] = group_sum<64>(ss[r]);
+    if ((threadIdx.x & 63) == 0) red[r][threadIdx.x >> 6] = ss[r];
+  }
+  __syncthreads();
+  if (ROWS == 1) {
+#pragma unroll
+    for (int i = 0; i < ITERS; ++i) {
+      const int c = threadIdx.x + i * kNormThreads;
+      if (c < chunks) wv[i] = ld16(w + c * 8);
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < ROWS; ++r) {
+    if (row0 + r >= rows) break;
+    const float tot = red[r][0] + red[r][1] + red[r][2] + red[r][3];
+    const float rstd = rsqrtf(tot / (float)n + eps);
+    uint16_t* orow = out + (row0 + r) * out_stride;
+#pragma unroll
+    for (int i = 0; i < ITERS; ++i) {
+      const int c = threadIdx.x + i * kNormThreads;
+      if (c < chunks) {
+        u32x4 o;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          float a = Elem<E>::lo(v[r][i][j]) * rstd, b = Elem<E>::hi(v[r][i][j]) * rstd;
+          if (ROUND_FIRST) {
+            a = rnd<E>(a);
+            b = rnd<E>(b);
+          }
+          o[j] = pack2<E>(a * Elem<E>::lo(wv[i][j]), b * Elem<E>::hi(wv[i][j]));
+        }
+        st16(orow + c * 8, o);
+      }
     }
   }
 }
@@ -102,7 +138,16 @@ static int launch_rms(void* out, const void* x, const void* w, float eps, int64_
   dim3 grid((unsigned)rows), block(kNormThreads);
   if (vec) {
     const int iters = (int)((n / 8 + kNormThreads - 1) / kNormThreads);
-#define PH_RMS(I) hipLaunchKernelGGL((rms_norm_vec<E, I, RF>), grid, block, 0, st, o, xi, wi, eps, (int)n, xs, os)
+    // three rows per workgroup once there are rows enough to fill the device that way
+    const bool multi = rows >= 2048 && iters <= 4;
+    const dim3 vgrid((unsigned)(multi ? (rows + 2) / 3 : rows));
+#define PH_RMS(I)                                                                                                \
+  do {                                                                                                           \
+    if (multi)                                                                                                   \
+      hipLaunchKernelGGL((rms_norm_vec<E, I, RF, 3>), vgrid, block, 0, st, o, xi, wi, eps, (int)n, rows, xs, os); \
+    else                                                                                                         \
+      hipLaunchKernelGGL((rms_norm_vec<E, I, RF, 1>), vgrid, block, 0, st, o, xi, wi, eps, (int)n, rows, xs, os); \
+  } while (0)
     if (iters <= 1) PH_RMS(1);
     else if (iters <= 2) PH_RMS(2);
     else if (iters <= 3) PH_RMS(3);

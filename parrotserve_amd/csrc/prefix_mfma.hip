@@ -583,6 +583,7 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
   const int iters = (ntile + TQ - 1) / TQ;                 // same for all eight waves
   const int my_iters = ntile > g ? (ntile - g + TQ - 1) / TQ : 0;  // tiles of this token group
   __syncthreads();                                         // window visible
+  PH_TL(1);
   // the whole ring is filled up front: tiles 0 .. A (the main loop issues tile it + A at step it >= 1)
 #pragma unroll
   for (int j = 0; j < NST; ++j)
@@ -614,7 +615,9 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
   // last token any query of this wave's block may see (none if the block has no live query)
   const int wave_last = 32 * qb >= wk.nq ? -1 : CAUSAL ? min(s1 - 1, wk.causal_off + 32 * qb + 31) : s1 - 1;
 
+  PH_TL(2);
   mid();
+  PH_TL(3);
 
   // Operand read addresses of ring stage 0 (and of stage 4, beyond the reach of the 16-bit immediate).
   // K: row ql, chunk (8h + s) swizzled by the row; V: the transposing read's row/column of this lane.
@@ -660,6 +663,7 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
       wait_vmcnt<(A - 1) * LPT>();
     }
     __syncthreads();
+    if (it < 4) PH_TL(4 + it);
     {
       const int front = s0 + STEP * TQ * (it + A);           // first token of the step being staged
       if (front < s1 && front >= win0 + kWin) {              // workgroup-uniform: slide the slot window
@@ -775,6 +779,7 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
    }
   }
 
+  PH_TL(8);
   if constexpr (TQ == 1) {
     // one token group: nothing to fold across waves
     const float Lall = lsum + __shfl_xor(lsum, 32, kWave);
@@ -902,6 +907,7 @@ __device__ __forceinline__ void prefix_unit8(const PrefixArgs& a, int split, int
   float16_t of[NDB];
   float m, l;
   attn_tile8<E, false, TQ>(wk, a.kc, a.vc, a.row_stride, head, a.scale_log2e, smem, of, m, l, mid);
+  PH_TL(9);
   const int lane = threadIdx.x & 63, w8 = threadIdx.x >> 6, tq = w8 / QB, qh = w8 % QB, h = lane >> 5, ql = lane & 31;
   const int q = 32 * qh + ql;
   if (q < nq) {
@@ -941,6 +947,7 @@ __global__ __launch_bounds__(512) void prefix_mfma8_kernel(PrefixArgs a, int mti
 template <typename E, int TQ, int DS = kPD>
 __global__ __launch_bounds__(512) void decode_fused_kernel(PrefixArgs pa, int mtiles, int n_units, ItemArgs ia) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
+  PH_TL(0);
   constexpr int HPW = HeadLanes<DS>::HPW;
   const int hgroups = (ia.H + HPW - 1) / HPW;
   const int slots = ia.num_lanes * hgroups;
@@ -974,6 +981,7 @@ __global__ __launch_bounds__(512) void decode_fused_kernel(PrefixArgs pa, int mt
   } else {
     suffix();
   }
+  PH_TL(11);
 }
 
 // Prefill with parent context, eight waves: workgroup = (head, tile of 32 * (8 / TQ) queries of one chunk)
