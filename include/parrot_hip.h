@@ -28,7 +28,11 @@
 extern "C" {
 #endif
 
-typedef enum { PH_F16 = 0, PH_BF16 = 1, PH_F32 = 2 /* ph_sample_top_p only */ } ph_dtype;
+/* Element types.  The reference's configuration offers float16 and float32 (parrot/engine/config.py:22-25), its CUDA
+ * kernels also bfloat16.  PH_F32 is served by the per-request decode kernels (every attention entry point: a
+ * shared prefix is then read once per request, a prefill runs row by row), the merge, RMSNorm, both rotary forms,
+ * the token move, the KV append and the sampler; the matrix-core kernels and the fused per-layer ops are 16-bit. */
+typedef enum { PH_F16 = 0, PH_BF16 = 1, PH_F32 = 2 } ph_dtype;
 typedef enum { PH_IDX_I32 = 0, PH_IDX_I64 = 1 } ph_index_type;
 
 enum {
@@ -346,7 +350,7 @@ int ph_prefix_post_attention(void* out, const float* prev_m, const float* prev_l
  * The new tokens' K/V must already be in the cache (append first).
  * max_kv_len: host upper bound of any chunk's context length.
  * workspace: at least ph_prefill_workspace_bytes(...) bytes, 256-byte aligned. */
-size_t ph_prefill_workspace_bytes(int64_t num_tokens, int64_t num_heads, int64_t head_dim,
+size_t ph_prefill_workspace_bytes(int64_t num_tokens, int64_t num_heads, int64_t head_dim, int dtype,
                                   int64_t max_kv_len);
 
 int ph_prefill_attention(void* out, const void* q, const void* k_cache, const void* v_cache,

@@ -385,7 +385,8 @@ class BuiltinConfig:
 
     def __post_init__(self):
         if isinstance(self.dtype, str):
-            table = {"float16": torch.float16, "bfloat16": torch.bfloat16}
+            # float16 / float32 are the reference's choices (parrot/engine/config.py:22-25); bfloat16 its kernels' third
+            table = {"float16": torch.float16, "float32": torch.float32, "bfloat16": torch.bfloat16}
             if self.dtype not in table:
                 raise ValueError(f"Unknown dtype {self.dtype}")
             self.dtype = table[self.dtype]

@@ -175,7 +175,7 @@ static bool pair_heads(int64_t D, int64_t H) { return D == 64 && H % 2 == 0; }
 
 static int check_common(const void* out, const void* q, const void* kc, const void* vc, int64_t B, int64_t H,
                         int64_t D, int dtype, int64_t q_stride, int64_t out_stride, int64_t row_stride) {
-  if (dtype != PH_F16 && dtype != PH_BF16) return PH_ERR_DTYPE;
+  if (dtype != PH_F16 && dtype != PH_BF16 && dtype != PH_F32) return PH_ERR_DTYPE;
   if (D != 64 && D != 80 && D != 96 && D != 112 && D != 128 && D != 256) return PH_ERR_HEAD_DIM;
   if (B < 0 || H <= 0 || B > (1 << 24) || H > 4096) return PH_ERR_ARG;
   if (B == 0) return PH_OK;
@@ -710,11 +710,11 @@ extern "C" int ph_suffix_prev_attention(void* out, float* m_out, float* l_out, c
                       stream);
 }
 
-extern "C" size_t ph_prefill_workspace_bytes(int64_t num_tokens, int64_t num_heads, int64_t head_dim,
+extern "C" size_t ph_prefill_workspace_bytes(int64_t num_tokens, int64_t num_heads, int64_t head_dim, int dtype,
                                              int64_t max_kv_len) {
   if (num_tokens <= 0 || num_heads <= 0 || head_dim <= 0) return 0;
   const DecodePlan p = plan_decode(num_tokens, num_heads, 0, 0, max_kv_len, 0);
-  if (prefix_mfma_supported(PH_F16, (int)head_dim) || pair_heads(head_dim, num_heads))
+  if (prefix_mfma_supported(dtype, (int)head_dim) || (pair_heads(head_dim, num_heads) && prefix_mfma_supported(dtype, 128)))
     return 256 + (size_t)round_up((num_tokens + 2) * 4, 256);
   return (size_t)round_up(num_tokens * 8, 256) + (size_t)round_up(num_tokens * 4, 256) +
          plan_bytes(p, num_tokens, num_heads, head_dim);
@@ -732,7 +732,7 @@ extern "C" int ph_prefill_attention(void* out, const void* q, const void* k_cach
                         cache_stride_n);
   if (rc != PH_OK || num_tokens == 0) return rc;
   if (num_chunks <= 0 || max_kv_len <= 0 || max_kv_len > INT32_MAX || !q_cu || !kv_cu || !ctx_slots || ctx_slots_count <= 0) return PH_ERR_ARG;
-  if (ph_prefill_workspace_bytes(num_tokens, num_heads, head_dim, max_kv_len) > workspace_bytes || !workspace)
+  if (ph_prefill_workspace_bytes(num_tokens, num_heads, head_dim, dtype, max_kv_len) > workspace_bytes || !workspace)
     return PH_ERR_WORKSPACE;
   if (((uintptr_t)workspace & 255u) != 0) return PH_ERR_ALIGN;
   hipStream_t st = (hipStream_t)stream;

@@ -24,6 +24,16 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 struct F16 {};   // IEEE binary16
 struct BF16 {};  // bfloat16
+struct F32 {};   // IEEE binary32: the per-request decode, merge, norm, rotary and copy kernels only (no matrix cores)
+
+template <typename E>
+struct is_f32 {
+  static constexpr bool value = false;
+};
+template <>
+struct is_f32<F32> {
+  static constexpr bool value = true;
+};
 
 template <typename E>
 struct Elem;
@@ -74,6 +84,22 @@ __device__ __forceinline__ uint32_t pack2<BF16>(float a, float b) {
   return __builtin_bit_cast(uint32_t, v);
 }
 
+template <>
+struct Elem<F32> {
+  static __device__ __forceinline__ float one(float b) { return b; }
+  static __device__ __forceinline__ float bits(float f) { return f; }
+};
+
+// storage type of one element
+template <typename E>
+struct ElemStore {
+  typedef uint16_t T;
+};
+template <>
+struct ElemStore<F32> {
+  typedef float T;
+};
+
 // Round a float to the element type and back (the "t(.)" of the reference's
 // element-type arithmetic).
 template <typename E>
@@ -88,6 +114,39 @@ __device__ __forceinline__ u32x4 ld16_nt(const void* p) {
 }
 __device__ __forceinline__ void st16_nt(void* p, u32x4 v) {
   __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
+}
+
+// Eight consecutive elements at element offset `off` behind `base`, as floats / from floats rounded to the element type.
+template <typename E>
+__device__ __forceinline__ void load8f(const void* base, int64_t off, float (&f)[8]) {
+  if constexpr (is_f32<E>::value) {
+    const float4_t a = *reinterpret_cast<const float4_t*>(reinterpret_cast<const float*>(base) + off);
+    const float4_t b = *reinterpret_cast<const float4_t*>(reinterpret_cast<const float*>(base) + off + 4);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[i] = a[i];
+      f[4 + i] = b[i];
+    }
+  } else {
+    const u32x4 v = ld16(reinterpret_cast<const uint16_t*>(base) + off);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      f[2 * k] = Elem<E>::lo(v[k]);
+      f[2 * k + 1] = Elem<E>::hi(v[k]);
+    }
+  }
+}
+template <typename E>
+__device__ __forceinline__ void store8f(void* base, int64_t off, const float (&f)[8]) {
+  if constexpr (is_f32<E>::value) {
+    *reinterpret_cast<float4_t*>(reinterpret_cast<float*>(base) + off) = float4_t{f[0], f[1], f[2], f[3]};
+    *reinterpret_cast<float4_t*>(reinterpret_cast<float*>(base) + off + 4) = float4_t{f[4], f[5], f[6], f[7]};
+  } else {
+    u32x4 r;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) r[k] = pack2<E>(f[2 * k], f[2 * k + 1]);
+    st16(reinterpret_cast<uint16_t*>(base) + off, r);
+  }
 }
 
 // v + (v of the lane selected by a DPP control): one v_add_f32_dpp, no LDS round trip.

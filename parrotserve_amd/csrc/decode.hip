@@ -62,14 +62,11 @@ __global__ __launch_bounds__(256) void decode_partial_kernel(PartialArgs a) {
   const bool head_ok = head < a.H;
   const int hclamp = head_ok ? head : a.H - 1;
   const uint32_t lane_off = (uint32_t)(hclamp * D + HeadLanes<D>::chunk(lane) * 8);  // elements inside a token row
-  u32x4 qv = ld16(a.q + (int64_t)b * a.q_stride + lane_off);
-  if (!HeadLanes<D>::active(lane)) qv = u32x4{0u, 0u, 0u, 0u};
-
   if (t0 >= len) return;
   const int t1 = min(len, t0 + a.chunk);
   const int64_t pr = ((int64_t)(a.part_base + c) * a.B + b) * a.H + hclamp;
-  stream_item<E, D, TB, STAGES>(a.kc, a.vc, a.row_stride, slots, myslot, t0, t1, qv, lane_off, a.scale_log2e, head_ok,
-                                a.opart, a.ml, pr);
+  stream_request<E, D, TB, STAGES>(a.q, (int64_t)b * a.q_stride, a.kc, a.vc, a.row_stride, slots, myslot, t0, t1,
+                                   lane_off, a.scale_log2e, head_ok, a.opart, a.ml, pr);
 }
 
 // Balanced form: the host cut the batch's token stream into `num_lanes` near-equal pieces; a piece is
@@ -111,14 +108,12 @@ __global__ __launch_bounds__(256) void merge_kernel(MergeArgs a) {
   if (a.prev_m && w == 0) {  // a partial already sitting in out / prev_m / prev_l
     const float lp = a.prev_l[(int64_t)b * a.H + head];
     if (lp > 0.f) {
-      const u32x4 ov = ld16(a.out + (int64_t)b * a.out_stride + (int64_t)head * D + dl);
+      float ov[8];
+      load8f<E>(a.out, (int64_t)b * a.out_stride + (int64_t)head * D + dl, ov);
       M = a.prev_m[(int64_t)b * a.H + head];
       L = lp;
 #pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        acc[2 * k] = lp * Elem<E>::lo(ov[k]);
-        acc[2 * k + 1] = lp * Elem<E>::hi(ov[k]);
-      }
+      for (int k = 0; k < 8; ++k) acc[k] = lp * ov[k];
     }
   }
 
@@ -189,10 +184,9 @@ __global__ __launch_bounds__(256) void merge_kernel(MergeArgs a) {
   }
   if (!head_ok || !HeadLanes<D>::active(lane)) return;
   const float inv = L > 0.f ? 1.f / L : 0.f;
-  u32x4 r;
 #pragma unroll
-  for (int k = 0; k < 4; ++k) r[k] = pack2<E>(acc[2 * k] * inv, acc[2 * k + 1] * inv);
-  st16(a.out + (int64_t)b * a.out_stride + (int64_t)head * D + dl, r);
+  for (int k = 0; k < 8; ++k) acc[k] *= inv;
+  store8f<E>(a.out, (int64_t)b * a.out_stride + (int64_t)head * D + dl, acc);
   if (a.m_out && lane % LPH == 0) {
     a.m_out[(int64_t)b * a.H + head] = M;
     a.l_out[(int64_t)b * a.H + head] = L;
@@ -247,6 +241,13 @@ static int launch_merge_t(const MergeArgs& a, hipStream_t st, const KernelEvents
       if ((D) == 80) return FN<F16, 80>(__VA_ARGS__);                   \
       if ((D) == 96) return FN<F16, 96>(__VA_ARGS__);                   \
       if ((D) == 112) return FN<F16, 112>(__VA_ARGS__);                 \
+    } else if ((dtype) == PH_F32) {                                     \
+      if ((D) == 128) return FN<F32, 128>(__VA_ARGS__);                 \
+      if ((D) == 64) return FN<F32, 64>(__VA_ARGS__);                   \
+      if ((D) == 256) return FN<F32, 256>(__VA_ARGS__);                 \
+      if ((D) == 80) return FN<F32, 80>(__VA_ARGS__);                   \
+      if ((D) == 96) return FN<F32, 96>(__VA_ARGS__);                   \
+      if ((D) == 112) return FN<F32, 112>(__VA_ARGS__);                 \
     } else {                                                            \
       if ((D) == 128) return FN<BF16, 128>(__VA_ARGS__);                \
       if ((D) == 64) return FN<BF16, 64>(__VA_ARGS__);                  \

@@ -163,11 +163,11 @@ extern "C" int ph_kv_append(const void* k, const void* v, void* k_cache, void* v
                             int64_t num_heads, int64_t head_dim, int dtype, int64_t k_stride_n,
                             int64_t v_stride_n, int64_t cache_stride_n, void* stream) {
   if (num_tokens < 0 || num_heads <= 0 || head_dim <= 0) return PH_ERR_ARG;
-  if (dtype != PH_F16 && dtype != PH_BF16) return PH_ERR_DTYPE;
+  if (dtype != PH_F16 && dtype != PH_BF16 && dtype != PH_F32) return PH_ERR_DTYPE;
   if (index_type != PH_IDX_I32 && index_type != PH_IDX_I64) return PH_ERR_ARG;
   if (num_tokens == 0) return PH_OK;
   if (!k || !v || !k_cache || !v_cache || !slot_mapping) return PH_ERR_ARG;
-  const int eb = 2;
+  const int eb = dtype == PH_F32 ? 4 : 2;
   MoveArgs a{};
   a.set[0] = MoveSet{(const char*)k,  (char*)k_cache,      k_stride_n * eb, head_dim * eb, eb,
                      cache_stride_n * eb, head_dim * eb, eb};

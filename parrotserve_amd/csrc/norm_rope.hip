@@ -105,14 +105,15 @@ __global__ __launch_bounds__(kNormThreads) void rms_norm_vec(uint16_t* __restric
 
 // Any n / alignment: two passes over the row, scalar accesses.
 template <typename E, bool ROUND_FIRST>
-__global__ __launch_bounds__(kNormThreads) void rms_norm_generic(uint16_t* __restrict__ out,
-                                                                 const uint16_t* __restrict__ x,
-                                                                 const uint16_t* __restrict__ w, float eps,
-                                                                 int n, int64_t x_stride, int64_t out_stride) {
+__global__ __launch_bounds__(kNormThreads) void rms_norm_generic(typename ElemStore<E>::T* __restrict__ out,
+                                                                 const typename ElemStore<E>::T* __restrict__ x,
+                                                                 const typename ElemStore<E>::T* __restrict__ w,
+                                                                 float eps, int n, int64_t x_stride,
+                                                                 int64_t out_stride) {
   __shared__ float red[4];
   const int64_t row = blockIdx.x;
-  const uint16_t* xr = x + row * x_stride;
-  uint16_t* orow = out + row * out_stride;
+  const typename ElemStore<E>::T* xr = x + row * x_stride;
+  typename ElemStore<E>::T* orow = out + row * out_stride;
   float ss = 0.f;
   for (int i = threadIdx.x; i < n; i += kNormThreads) {
     const float a = Elem<E>::one(xr[i]);
@@ -157,6 +158,15 @@ static int launch_rms(void* out, const void* x, const void* w, float eps, int64_
   } else {
     hipLaunchKernelGGL((rms_norm_generic<E, RF>), grid, block, 0, st, o, xi, wi, eps, (int)n, xs, os);
   }
+  return launch_status();
+}
+
+// 32-bit elements: the element-wise kernel (rounding to the element type is the identity, so both rounding orders
+// of the 16-bit kernels coincide)
+static int launch_rms_f32(void* out, const void* x, const void* w, float eps, int64_t rows, int64_t n, int64_t xs,
+                          int64_t os, hipStream_t st) {
+  hipLaunchKernelGGL((rms_norm_generic<F32, false>), dim3((unsigned)rows), dim3(kNormThreads), 0, st, (float*)out,
+                     (const float*)x, (const float*)w, eps, (int)n, xs, os);
   return launch_status();
 }
 
@@ -210,20 +220,22 @@ __global__ __launch_bounds__(256) void rope_vec(const int64_t* __restrict__ posi
 }
 
 template <typename E>
-__global__ __launch_bounds__(256) void rope_generic(const int64_t* __restrict__ positions, uint16_t* q, uint16_t* k,
-                                                    const uint16_t* __restrict__ cos_base,
-                                                    const uint16_t* __restrict__ sin_base, int64_t cs_stride,
+__global__ __launch_bounds__(256) void rope_generic(const int64_t* __restrict__ positions,
+                                                    typename ElemStore<E>::T* q, typename ElemStore<E>::T* k,
+                                                    const typename ElemStore<E>::T* __restrict__ cos_base,
+                                                    const typename ElemStore<E>::T* __restrict__ sin_base,
+                                                    int64_t cs_stride,
                                                     int hq, int hk, int64_t q_stride_n, int64_t q_stride_h,
                                                     int64_t k_stride_n, int64_t k_stride_h, int half_rot) {
   const int64_t t = blockIdx.x;
   const int64_t p = positions ? positions[t] : t;
-  const uint16_t* cr = cos_base + p * cs_stride;
-  const uint16_t* sr = sin_base + p * cs_stride;
+  const typename ElemStore<E>::T* cr = cos_base + p * cs_stride;
+  const typename ElemStore<E>::T* sr = sin_base + p * cs_stride;
   const int units = (hq + hk) * half_rot;
   for (int u = threadIdx.x; u < units; u += 256) {
     const int h = u / half_rot;
     const int i = u - h * half_rot;
-    uint16_t* base = h < hq ? q + t * q_stride_n + (int64_t)h * q_stride_h
+    typename ElemStore<E>::T* base = h < hq ? q + t * q_stride_n + (int64_t)h * q_stride_h
                             : k + t * k_stride_n + (int64_t)(h - hq) * k_stride_h;
     const float x = Elem<E>::one(base[i]), y = Elem<E>::one(base[half_rot + i]);
     const float c = Elem<E>::one(cr[i]), s = Elem<E>::one(sr[i]);
@@ -249,6 +261,15 @@ static int launch_rope(const int64_t* pos, void* q, void* k, const void* cosb, c
   return launch_status();
 }
 
+// 32-bit elements: the element-wise kernel (fp32 products and sums, as the reference's CUDA kernel computes in float)
+static int launch_rope_f32(const int64_t* pos, void* q, void* k, const void* cosb, const void* sinb, int64_t cs_stride,
+                           int64_t T, int hq, int hk, int64_t qsn, int64_t qsh, int64_t ksn, int64_t ksh, int half_rot,
+                           hipStream_t st) {
+  hipLaunchKernelGGL((rope_generic<F32>), dim3((unsigned)T), dim3(256), 0, st, pos, (float*)q, (float*)k,
+                     (const float*)cosb, (const float*)sinb, cs_stride, hq, hk, qsn, qsh, ksn, ksh, half_rot);
+  return launch_status();
+}
+
 }  // namespace ph
 
 using namespace ph;
@@ -257,10 +278,11 @@ extern "C" int ph_rms_norm(void* out, const void* x, const void* weight, float e
                            int64_t x_stride, int64_t out_stride, int dtype, int round_before_weight,
                            void* stream) {
   if (rows < 0 || n <= 0 || x_stride < n || out_stride < n) return PH_ERR_ARG;
-  if (dtype != PH_F16 && dtype != PH_BF16) return PH_ERR_DTYPE;
+  if (dtype != PH_F16 && dtype != PH_BF16 && dtype != PH_F32) return PH_ERR_DTYPE;
   if (rows == 0) return PH_OK;
   if (!out || !x || !weight) return PH_ERR_ARG;
   hipStream_t st = (hipStream_t)stream;
+  if (dtype == PH_F32) return launch_rms_f32(out, x, weight, eps, rows, n, x_stride, out_stride, st);
   if (dtype == PH_F16)
     return round_before_weight ? launch_rms<F16, true>(out, x, weight, eps, rows, n, x_stride, out_stride, st)
                                : launch_rms<F16, false>(out, x, weight, eps, rows, n, x_stride, out_stride, st);
@@ -274,13 +296,16 @@ extern "C" int ph_rope_neox(const int64_t* positions, void* q, void* k, const vo
   if (num_tokens < 0 || num_q_heads <= 0 || num_k_heads < 0 || head_dim <= 0 || rot_dim <= 0 || rot_dim % 2 ||
       rot_dim > head_dim)
     return PH_ERR_ARG;
-  if (dtype != PH_F16 && dtype != PH_BF16) return PH_ERR_DTYPE;
+  if (dtype != PH_F16 && dtype != PH_BF16 && dtype != PH_F32) return PH_ERR_DTYPE;
   if (num_tokens == 0) return PH_OK;
   if (!positions || !q || !cos_sin_cache || (num_k_heads > 0 && !k)) return PH_ERR_ARG;
   const int half = (int)(rot_dim / 2);
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == PH_F32)
+    return launch_rope_f32(positions, q, k, cos_sin_cache, (const float*)cos_sin_cache + half, rot_dim, num_tokens,
+                           (int)num_q_heads, (int)num_k_heads, q_stride, head_dim, k_stride, head_dim, half, st);
   const uint16_t* cosb = (const uint16_t*)cos_sin_cache;
   const uint16_t* sinb = cosb + half;
-  hipStream_t st = (hipStream_t)stream;
   if (dtype == PH_F16)
     return launch_rope<F16>(positions, q, k, cosb, sinb, rot_dim, num_tokens, (int)num_q_heads, (int)num_k_heads,
                             q_stride, head_dim, k_stride, head_dim, half, st);
@@ -292,11 +317,14 @@ extern "C" int ph_rotary_embedding(void* state, const void* cos, const void* sin
                                    int64_t num_heads, int64_t head_dim, int64_t stride_n, int64_t stride_h,
                                    int64_t cs_stride, int dtype, void* stream) {
   if (num_tokens < 0 || num_heads <= 0 || head_dim <= 0 || head_dim % 2) return PH_ERR_ARG;
-  if (dtype != PH_F16 && dtype != PH_BF16) return PH_ERR_DTYPE;
+  if (dtype != PH_F16 && dtype != PH_BF16 && dtype != PH_F32) return PH_ERR_DTYPE;
   if (num_tokens == 0) return PH_OK;
   if (!state || !cos || !sin) return PH_ERR_ARG;
   hipStream_t st = (hipStream_t)stream;
   const int half = (int)(head_dim / 2);
+  if (dtype == PH_F32)
+    return launch_rope_f32(nullptr, state, nullptr, cos, sin, cs_stride, num_tokens, (int)num_heads, 0, stride_n,
+                           stride_h, 0, 0, half, st);
   if (dtype == PH_F16)
     return launch_rope<F16>(nullptr, state, nullptr, cos, sin, cs_stride, num_tokens, (int)num_heads, 0, stride_n,
                             stride_h, 0, 0, half, st);

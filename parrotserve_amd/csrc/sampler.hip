@@ -23,8 +23,6 @@
 
 namespace ph {
 
-struct F32 {};
-
 constexpr int kSampThreads = 1024;
 constexpr int kSampWaves = kSampThreads / kWave;
 constexpr int kSampLdsFloats = 36 * 1024;

@@ -104,6 +104,104 @@ __device__ __forceinline__ void stream_item(const uint16_t* __restrict__ kc, con
   }
 }
 
+// The same for 32-bit elements: a lane's eight elements of a token row are two 128-bit loads (the lanes of a head
+// still cover the head's row contiguously), the dot product and P.V are plain fp32 FMAs.  One stage of TB token
+// rows in flight; this element type is served for completeness of the reference's configuration (float32), the
+// tuned path is the 16-bit one above.
+template <int D, int TB>
+__device__ __forceinline__ void stream_item_f32(const float* __restrict__ kc, const float* __restrict__ vc,
+                                                int64_t row_stride, const int32_t* __restrict__ slots, int myslot,
+                                                int t0, int t1, const float (&q)[8], uint32_t lane_off,
+                                                float scale_log2e, bool head_ok, float* __restrict__ opart,
+                                                float* __restrict__ ml, int64_t pr) {
+  constexpr int LPH = HeadLanes<D>::LPH;
+  const int lane = threadIdx.x & 63;
+  float m = -INFINITY, l = 0.f;
+  float o[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) o[i] = 0.f;
+  for (int tb = t0; tb < t1; tb += kWave) {
+    if (tb > t0) myslot = slots[min(tb + lane, t1 - 1)];
+    const int nb = min(kWave, t1 - tb);
+    for (int j0 = 0; j0 < nb; j0 += TB) {
+      float4_t k0[TB], k1[TB], v0[TB], v1[TB];
+#pragma unroll
+      for (int j = 0; j < TB; ++j) {
+        const int64_t slot = __builtin_amdgcn_readlane(myslot, min(j0 + j, nb - 1));
+        const float* kr = kc + slot * row_stride + lane_off;
+        const float* vr = vc + slot * row_stride + lane_off;
+        k0[j] = __builtin_nontemporal_load(reinterpret_cast<const float4_t*>(kr));
+        k1[j] = __builtin_nontemporal_load(reinterpret_cast<const float4_t*>(kr + 4));
+        v0[j] = __builtin_nontemporal_load(reinterpret_cast<const float4_t*>(vr));
+        v1[j] = __builtin_nontemporal_load(reinterpret_cast<const float4_t*>(vr + 4));
+      }
+      float s[TB];
+      float mb = -INFINITY;
+#pragma unroll
+      for (int j = 0; j < TB; ++j) {
+        float d = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          d = __builtin_fmaf(q[i], k0[j][i], d);
+          d = __builtin_fmaf(q[4 + i], k1[j][i], d);
+        }
+        d = group_sum<LPH>(d) * scale_log2e;
+        s[j] = (j0 + j < nb) ? d : -INFINITY;
+        mb = fmaxf(mb, s[j]);
+      }
+      const float mn = fmaxf(m, mb);
+      const float alpha = __builtin_amdgcn_exp2f(m - mn);
+      l *= alpha;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) o[i] *= alpha;
+#pragma unroll
+      for (int j = 0; j < TB; ++j) {
+        const float p = __builtin_amdgcn_exp2f(s[j] - mn);
+        l += p;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          o[i] = __builtin_fmaf(p, v0[j][i], o[i]);
+          o[4 + i] = __builtin_fmaf(p, v1[j][i], o[4 + i]);
+        }
+      }
+      m = mn;
+    }
+  }
+  if (!head_ok || !HeadLanes<D>::active(lane)) return;
+  const float inv = 1.f / l;
+  float* op = opart + pr * D + (lane % LPH) * 8;
+  *reinterpret_cast<float4_t*>(op) = float4_t{o[0] * inv, o[1] * inv, o[2] * inv, o[3] * inv};
+  *reinterpret_cast<float4_t*>(op + 4) = float4_t{o[4] * inv, o[5] * inv, o[6] * inv, o[7] * inv};
+  if (lane % LPH == 0) {
+    ml[pr * 2] = m;
+    ml[pr * 2 + 1] = l;
+  }
+}
+
+// One request's list [t0, t1) through one wave, whatever the element type: loads the query and runs the streaming body.
+template <typename E, int D, int TB, int STAGES>
+__device__ __forceinline__ void stream_request(const uint16_t* q, int64_t q_off, const uint16_t* kc, const uint16_t* vc,
+                                               int64_t row_stride, const int32_t* slots, int myslot, int t0, int t1,
+                                               uint32_t lane_off, float scale_log2e, bool head_ok, float* opart,
+                                               float* ml, int64_t pr) {
+  const int lane = threadIdx.x & 63;
+  if constexpr (is_f32<E>::value) {
+    float qf[8];
+    load8f<F32>(q, q_off + lane_off, qf);
+    if (!HeadLanes<D>::active(lane)) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) qf[i] = 0.f;
+    }
+    stream_item_f32<D, TB>(reinterpret_cast<const float*>(kc), reinterpret_cast<const float*>(vc), row_stride, slots,
+                           myslot, t0, t1, qf, lane_off, scale_log2e, head_ok, opart, ml, pr);
+  } else {
+    u32x4 qv = ld16(q + q_off + lane_off);
+    if (!HeadLanes<D>::active(lane)) qv = u32x4{0u, 0u, 0u, 0u};
+    stream_item<E, D, TB, STAGES>(kc, vc, row_stride, slots, myslot, t0, t1, qv, lane_off, scale_log2e, head_ok, opart,
+                                  ml, pr);
+  }
+}
+
 // One piece of the balanced form for one head group: the piece's items (request, first token, count) are
 // streamed one after the other by this wave, one partial row per item.
 // (rec0, rec1) = the piece's lane record, already loaded by the caller
@@ -123,10 +221,8 @@ __device__ __forceinline__ void run_piece_rec(const ItemArgs& a, int hg, int4 re
     const int b = meta.x, t0 = meta.y, t1 = meta.y + meta.z;
     const int32_t* slots = a.slots + (a.offsets ? a.offsets[b] : (int64_t)b * a.table_stride);
     const int myslot = slots[min(t0 + lane, t1 - 1)];
-    u32x4 qv = ld16(a.q + (int64_t)b * a.q_stride + lane_off);
-    if (!HeadLanes<D>::active(lane)) qv = u32x4{0u, 0u, 0u, 0u};
-    stream_item<E, D, TB, STAGES>(a.kc, a.vc, a.row_stride, slots, myslot, t0, t1, qv, lane_off, a.scale_log2e,
-                                  head_ok, a.opart, a.ml, (int64_t)it * a.H + hclamp);
+    stream_request<E, D, TB, STAGES>(a.q, (int64_t)b * a.q_stride, a.kc, a.vc, a.row_stride, slots, myslot, t0, t1,
+                                     lane_off, a.scale_log2e, head_ok, a.opart, a.ml, (int64_t)it * a.H + hclamp);
   }
 }
 

@@ -51,6 +51,8 @@ def _dtype_code(t: torch.Tensor) -> int:
         return PH_F16
     if t.dtype == torch.bfloat16:
         return PH_BF16
+    if t.dtype == torch.float32:
+        return _lib.PH_F32
     # TORCH_CHECK(false, "Unsupported data type") in the reference's launcher
     raise RuntimeError(f"Unsupported data type: {t.dtype}")
 
@@ -848,7 +850,7 @@ def prefill_attention(query, key_cache, value_cache, tables: PrefillTables, scal
         return out
     scale = D ** -0.5 if scale is None else scale
     lib = _lib.load()
-    nbytes = lib.ph_prefill_workspace_bytes(T, H, D, tables.max_kv_len)
+    nbytes = lib.ph_prefill_workspace_bytes(T, H, D, _dtype_code(query), tables.max_kv_len)
     ws = _workspace(nbytes, query.device)
     rc = lib.ph_prefill_attention(
         _ptr(out), _ptr(query), _ptr(key_cache), _ptr(value_cache), T, tables.num_chunks, H, D, _dtype_code(query),

@@ -28,10 +28,23 @@ def make_cos_sin_cache(max_seq_len: int, rotary_size: int, rope_theta: float, dt
 Model_Cache: Optional[ModelCacheStorage] = None
 
 
-def init_model_cache_storage(num_layers: int, num_slots: int, num_heads: int, head_size: int, dtype, device,
-                             max_seq_len: int = 0, rope_theta: float = 10000.0) -> ModelCacheStorage:
+def init_model_cache_storage(*args, **kwargs) -> ModelCacheStorage:
+    """Two call forms.  The reference's (parrot/engine/builtin/mem.py:179-184):
+    ``init_model_cache_storage(hf_config, builtin_config)`` -- layers, heads, head size, maximum positions and rope
+    base are read from the model configuration, slot count, dtype and device from the engine configuration.  And the
+    explicit one: ``init_model_cache_storage(num_layers, num_slots, num_heads, head_size, dtype, device,
+    max_seq_len=0, rope_theta=10000.0)``."""
     global Model_Cache
-    Model_Cache = ModelCacheStorage(num_layers, num_slots, num_heads, head_size, dtype, device, max_seq_len, rope_theta)
+    if args and hasattr(args[0], "num_hidden_layers"):
+        hf_config, builtin_config = args[0], (args[1] if len(args) > 1 else kwargs["builtin_config"])
+        heads = hf_config.num_attention_heads
+        Model_Cache = ModelCacheStorage(
+            hf_config.num_hidden_layers, builtin_config.num_kv_cache_blocks, heads, hf_config.hidden_size // heads,
+            builtin_config.dtype, builtin_config.device,
+            max_seq_len=getattr(hf_config, "max_position_embeddings", 0) or 0,
+            rope_theta=float(getattr(hf_config, "rope_theta", 10000.0) or 10000.0))
+    else:
+        Model_Cache = ModelCacheStorage(*args, **kwargs)
     return Model_Cache
 
 

@@ -47,7 +47,9 @@ def test_workspace_queries_are_host_only():
     assert n > 0 and n % 256 == 0
     assert lib.ph_decode_workspace_bytes(0, 32, 128, 1, 4096, 512, 32, 0) == 0
     assert lib.ph_decode_workspace_bytes(64, 32, 128, 1, 4096, 512, 0, 448) < n  # balanced form: fewer partial rows
-    assert lib.ph_prefill_workspace_bytes(1000, 40, 128, 3000) > 0
+    assert lib.ph_prefill_workspace_bytes(1000, 40, 128, 1, 3000) > 0
+    # 32-bit elements take the row-by-row path: partials for every token
+    assert lib.ph_prefill_workspace_bytes(1000, 40, 128, 2, 3000) > lib.ph_prefill_workspace_bytes(1000, 40, 128, 1, 3000)
 
 
 def test_argument_validation_needs_no_gpu():

@@ -355,3 +355,23 @@ def test_grouping_by_the_deepest_shared_ancestor():
     x, y = gen(ctx(30, ctx(31, None, 7), 2)), gen(ctx(32, ctx(33, None, 5), 1))
     t = build_iteration_tables([x, y], "parent")
     assert t.groups == [] and t.paged_context_lens == [9, 6]
+
+
+def test_model_cache_storage_takes_the_reference_call_form():
+    """init_model_cache_storage(hf_config, builtin_config), as parrot/engine/builtin/mem.py:179-184 is called."""
+    import types
+
+    import torch
+
+    from parrotserve_amd import mem
+    from parrotserve_amd.attn_func import BuiltinConfig
+
+    hf = types.SimpleNamespace(num_hidden_layers=2, num_attention_heads=4, hidden_size=64, max_position_embeddings=32,
+                               rope_theta=10000.0)
+    cfg = BuiltinConfig(num_kv_cache_blocks=10, attn_func="hip_shared_prefix", dtype="float32", device="cpu")
+    store = mem.init_model_cache_storage(hf, cfg)
+    assert store.k_cache.shape == (2, 10, 4, 16) and store.v_cache.dtype == torch.float32
+    assert mem.get_k_cache(1).shape == (10, 4, 16) and mem.get_cos_sin_cache().shape == (32, 16)
+    same = mem.init_model_cache_storage(2, 10, 4, 16, torch.float32, "cpu", max_seq_len=32)
+    assert torch.equal(same.cos_sin_cache, store.cos_sin_cache)
+    mem.Model_Cache = None
