@@ -27,12 +27,18 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16
 
-# HBM traffic of one suffix-kernel launch at this workload, measured with rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE in two runs of this file and scaled by the same counters' readings for a plain 1 GiB copy
-# (profiles/bench_config2_hbm_traffic.txt): 285.5 MB read + 7.4 MB written.
-SUFFIX_TRAFFIC_BYTES = 293.0e6
-# same for the kernel that runs the prefix and suffix phases in one launch: 354.1 MB read + 13.8 MB written
-FUSED_TRAFFIC_BYTES = 367.9e6
+# HBM traffic per launch of this workload's kernels and the matrix-pipe counters of the prefix kernel come from
+# rocprofv3 --pmc passes over this file; their summary (python -m parrotserve_amd.profile_summary) is kept in
+# profiles/counters.json together with the commit it was taken at, and is read from there -- nothing is typed in.
+COUNTERS_JSON = os.path.join(ROOT, "profiles", "counters.json")
+
+
+def measured_counters():
+    try:
+        with open(COUNTERS_JSON) as f:
+            return json.load(f)
+    except (OSError, ValueError):
+        return {}
 
 
 class HipEvents:
@@ -74,7 +80,8 @@ def cpu_baseline(case, sample_reqs: int, budget_s: float = 12.0):
 
     from oracle.ref_ops import ref_decode_attention
 
-    cores = min(os.cpu_count() or 1, 16)
+    host_cores = os.cpu_count() or 1
+    cores = min(host_cores, 16)  # the GPU box's CPU share for one GPU
     torch.set_num_threads(cores)
     lists = case.full_lists()[:sample_reqs]
     q = case.q[:sample_reqs]
@@ -90,6 +97,7 @@ def cpu_baseline(case, sample_reqs: int, budget_s: float = 12.0):
         "value": sample_reqs / t,
         "unit": "tokens/s/layer",
         "cores": cores,
+        "host_cores": host_cores,
         "kind": "port",
         "sample": f"{sample_reqs} of {case.num_reqs} requests of the same workload (fp32 math on fp16-rounded inputs), "
                   f"median of {len(times)} passes ({time.perf_counter() - t_begin:.1f} s of host work)",
@@ -140,6 +148,13 @@ def extras(torch, dev):
     nbytes = 2 * src.numel() * H * D * 2
     out["c3_token_move"] = {"rows": src.numel(), "row_bytes": H * D * 2, "us": t * 1e6, "GB/s": nbytes / t / 1e9,
                             "frac_hbm": nbytes / t / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": nbytes}
+    # the same kernel as a plain copy of as many rows in order (what a read + write stream of this size reaches on
+    # this device: the ceiling a move of scattered rows can approach)
+    ident = torch.arange(src.numel(), device=dev)
+    half = pool // 2
+    t_copy = _time_gpu(torch, lambda: kernels.discontinuous_move_tokens(kc[:half], kc[half:], ident, ident))
+    out["c3_token_move"]["same_rows_in_order_us"] = t_copy * 1e6
+    out["c3_token_move"]["same_rows_in_order_frac_hbm"] = nbytes / t_copy / 1e9 / HBM_PEAK_GBS
     # --- the same 65,536 rows gathered out of the block-structured layouts (block 16, x 8) of a 4M-slot cache:
     # whole blocks in random order (a context that owns its blocks) and fully random slots -----------------------
     bs, x = 16, 8
@@ -686,21 +701,22 @@ def main():
         ev.destroy(s)
     # the prefix pair stays unrecorded when the library runs the prefix and suffix phases in one launch
     fused = all(x is None for x in ph[0])
-    t_prefix, t_suffix, t_merge = (None if any(v is None for v in x) else sum(x) / len(x) * 1e-3 for x in ph)
+    _, t_suffix, t_merge = (None if any(v is None for v in x) else sum(x) / len(x) * 1e-3 for x in ph)
 
     e = 2  # bytes per fp16 element
     suffix_bytes = 2 * sum_s * H * D * e
     prefix_bytes = 2 * P * H * D * e
     prefix_flops = 4 * B * H * P * D
+    counters = measured_counters()
     if fused:
         # one kernel streams the prefix K/V (through the matrix cores) and every request's suffix K/V
         kernel_name = "decode_fused_kernel (prefix + suffix phases)"
         kernel_bytes = prefix_bytes + suffix_bytes
-        traffic = FUSED_TRAFFIC_BYTES
+        traffic = counters.get("hbm_traffic_bytes", {}).get("decode_fused_kernel")
     else:
         kernel_name = "decode_items_kernel (suffix phase)"
         kernel_bytes = suffix_bytes
-        traffic = SUFFIX_TRAFFIC_BYTES
+        traffic = counters.get("hbm_traffic_bytes", {}).get("decode_items_kernel")
     kernel_gbs = kernel_bytes / t_suffix / 1e9
 
     result = {
@@ -729,6 +745,7 @@ def main():
             "unit": "GB/s",
             "frac": kernel_gbs / HBM_PEAK_GBS,
             "traffic": traffic,
+            "traffic_measured_at_commit": counters.get("commit") if traffic is not None else None,
             "algorithmic_bytes": kernel_bytes,
             "avg_launch_us": t_suffix * 1e6,
         },
@@ -736,34 +753,61 @@ def main():
         "step_us_percentiles": pct,
         "warm_single_kv_set": {"value": B / t_warm, "ms_per_step": t_warm * 1e3},
     }
-    if fused:
-        # the prefix phase on its own (the same batch with empty suffixes: prefix kernel, then merge), for its
-        # matrix-core figures; in the step proper it runs inside the fused launch
-        ptabs = [kernels.DecodeTables.build([perm[l * n_used:(l + 1) * n_used][p].tolist() for p in case.prefix_lists],
-                                            case.group_req_cu, [[] for _ in range(B)], dev) for l in range(NL)]
-        for i in range(8):
-            kernels.decode_attention(qs[i % NL], kc, vc, ptabs[i % NL], out=out)
-        sets = [ev.create(6) for _ in range(64)]
+    def kernel_time(tabs_of, which, launches=64, warm=8):
+        """Average dispatch time (start/stop events attached to the launch) of kernel `which` (0 prefix, 1 suffix)
+        over `launches` calls; tabs_of(i) picks the tables and query of call i."""
+        for i in range(warm):
+            t, q = tabs_of(i)
+            kernels.decode_attention(q, kc, vc, t, out=out)
+        sets = [ev.create(6) for _ in range(launches)]
         for i, s6 in enumerate(sets):
-            kernels.decode_attention(qs[i % NL], kc, vc, ptabs[i % NL], out=out, events6=s6)
+            t, q = tabs_of(i)
+            kernels.decode_attention(q, kc, vc, t, out=out, events6=s6)
         torch.cuda.synchronize()
-        tp = [ev.elapsed_ms(s6[0], s6[1]) for s6 in sets]
+        ts = [ev.elapsed_ms(s6[2 * which], s6[2 * which + 1]) for s6 in sets]
         for s6 in sets:
             ev.destroy(s6)
-        if all(v is not None for v in tp):
-            t_prefix = sum(tp) / len(tp) * 1e-3
-        del ptabs
-    if t_prefix is not None:
-        prefix_tflops = prefix_flops / t_prefix / 1e12
-        prefix_bound_tflops = min(MFMA_F16_PEAK_TFLOPS, B * HBM_PEAK_GBS / 1e3)  # AI = B FLOP per KV byte
-        result["prefix_phase"] = {
-            "kernel": "prefix_mfma8_kernel" + (" (run on its own: empty suffixes)" if fused else ""),
-            "avg_launch_us": t_prefix * 1e6,
-            "tflops": prefix_tflops,
-            "frac_mfma_peak": prefix_tflops / MFMA_F16_PEAK_TFLOPS,
-            "frac_of_min_mfma_hbm_bound": prefix_tflops / prefix_bound_tflops,
-            "kv_gbs": prefix_bytes / t_prefix / 1e9,
+        return None if any(v is None for v in ts) else sum(ts) / len(ts) * 1e-3
+
+    # The two phases on their own, each against the roofline that bounds it.
+    # Prefix phase: the same batch with empty suffixes (prefix kernel, then merge).  It is a dense contraction with
+    # exactly B FLOP per K/V byte, so from HBM its ceiling is min(MFMA peak, B x HBM peak) = 0.51 PFLOP/s at B = 64
+    # (20 % of the matrix peak): "cold" rotates over the KV sets as the step does and is measured against that bound;
+    # "warm" re-reads one 67 MB set, which stays in the 256 MB memory-side cache, and is measured against the
+    # matrix peak itself (the figure the reference quotes for its kernel, shared_flash_decoding.py:407-416).
+    ptabs = [kernels.DecodeTables.build([perm[l * n_used:(l + 1) * n_used][p].tolist() for p in case.prefix_lists],
+                                        case.group_req_cu, [[] for _ in range(B)], dev) for l in range(NL)]
+    prefix_bound_tflops = min(MFMA_F16_PEAK_TFLOPS, B * HBM_PEAK_GBS / 1e3)  # AI = B FLOP per KV byte
+    phase = {"kernel": "prefix_mfma8_kernel (run on its own: the batch with empty suffixes)",
+             "flops": prefix_flops, "kv_bytes": prefix_bytes}
+    for label, pick in (("cold", lambda i: (ptabs[i % NL], qs[i % NL])), ("warm", lambda i: (ptabs[0], qs[0]))):
+        tp = kernel_time(pick, 0)
+        if tp is None:
+            continue
+        tf = prefix_flops / tp / 1e12
+        phase[label] = {"avg_launch_us": tp * 1e6, "tflops": tf, "frac_mfma_peak": tf / MFMA_F16_PEAK_TFLOPS,
+                        "frac_of_min_mfma_hbm_bound": tf / prefix_bound_tflops, "kv_gbs": prefix_bytes / tp / 1e9}
+    if "cold" in phase:
+        # matrix-pipe utilisation of the kernel from the profiler's counters (profiles/counters.json):
+        # SQ_VALU_MFMA_BUSY_CYCLES / (GRBM_GUI_ACTIVE per XCD x SIMDs)
+        pc = counters.get("prefix_mfma8_kernel", {})
+        phase["mfma_pipe_utilisation_from_counters"] = pc.get("mfma_pipe_utilisation")
+        phase["mfma_pipe_utilisation_by_trace_duration"] = pc.get("mfma_pipe_utilisation_by_trace_duration")
+        phase["counters_measured_at_commit"] = counters.get("commit")
+        result["prefix_phase"] = phase
+    del ptabs
+    # Suffix phase: the same requests without the shared prefix (P = 0) through decode_items_kernel, against HBM.
+    stabs = [kernels.DecodeTables.build([], [], [perm[l * n_used:(l + 1) * n_used][sx].tolist()
+                                                 for sx in case.suffix_lists], dev) for l in range(NL)]
+    ts_ = kernel_time(lambda i: (stabs[i % NL], qs[i % NL]), 1)
+    if ts_ is not None:
+        result["suffix_phase"] = {
+            "kernel": "decode_items_kernel (run on its own: the batch without its shared prefix)",
+            "avg_launch_us": ts_ * 1e6, "algorithmic_bytes": suffix_bytes, "GB/s": suffix_bytes / ts_ / 1e9,
+            "frac_hbm": suffix_bytes / ts_ / 1e9 / HBM_PEAK_GBS,
+            "traffic": counters.get("hbm_traffic_bytes", {}).get("decode_items_kernel"),
         }
+    del stabs
     if not args.no_extras:
         del kc, vc, tables, qs
         torch.cuda.empty_cache()

@@ -450,6 +450,17 @@ int ph_sample_top_p(const void* logits, int64_t row_stride, const float* tempera
                     const float* top_p, const float* uniform, int64_t* out_ids, int64_t rows,
                     int64_t vocab, int dtype, void* stream);
 
+/* The same temperature and top-p filter without the draw: probs[r, i] = the
+ * renormalised soft-max probability of token i of row r, 0 for tokens the
+ * filter drops -- the tensor the reference hands to torch.multinomial
+ * (parrot/engine/builtin/models/sampler.py:58-64).  A caller that wants the
+ * reference's own draw (the library's random stream: same seed, same kind of
+ * call) runs torch.multinomial(probs, 1, replacement=True) on it.
+ * probs: float32 [rows, vocab], probs_stride floats between rows. */
+int ph_top_p_probs(const void* logits, int64_t row_stride, const float* temperature,
+                   const float* top_p, float* probs, int64_t probs_stride, int64_t rows,
+                   int64_t vocab, int dtype, void* stream);
+
 /* ------------------------------------------------------------------------ */
 /* Instrumentation (no counterpart in the reference, which times whole
  * iterations from Python, parrot/engine/builtin/builtin_runner.py:158-175).

@@ -46,6 +46,7 @@ SIGNATURES: Dict[str, Tuple[object, List[object]]] = {
     "ph_decode_attention_timed": (I, [P, P, P, P, L, L, L, I, L, L, L, F, L, P, P, P, P, L, P, P, L, L, P, L, L, P, P, Z, P, P]),
     "ph_suffix_plan_build": (I, [P, L, L, L, P, P, P, P]),
     "ph_sample_top_p": (I, [P, L, P, P, P, P, L, L, I, P]),
+    "ph_top_p_probs": (I, [P, L, P, P, P, L, L, L, I, P]),
     "ph_prefill_workspace_bytes": (Z, [L, L, L, I, L]),
     "ph_prefill_attention": (I, [P, P, P, P, L, L, L, L, I, L, L, L, F, P, P, P, L, L, P, Z, P]),
 }

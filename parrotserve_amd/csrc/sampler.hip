@@ -90,6 +90,8 @@ struct SampArgs {
   const float* uniform;
   int64_t* out;
   int V;
+  float* probs;          // set: no draw, the filtered and renormalised probabilities of every row go here
+  int64_t probs_stride;  // floats between rows
 };
 
 template <typename E, bool LDSX>
@@ -228,6 +230,13 @@ __global__ __launch_bounds__(kSampThreads) void sample_top_p_kernel(const SampAr
     kept += sh.fpart[i];
   }
   base += finc - s;
+  if (a.probs) {  // the distribution itself instead of a draw from it: zero for dropped tokens, e / (kept mass) else
+    float* prow = a.probs + row * a.probs_stride;
+    const float inv = 1.f / kept;
+    for (int i = b0; i < b1; ++i) prow[i] = 0.f;
+    walk([&](int i, float e) { prow[i] = e * inv; });
+    return;
+  }
   const float goal = a.uniform[row] * kept;
   int found = INT_MAX, last = -1;
   float running = base;
@@ -530,9 +539,38 @@ extern "C" int ph_sample_top_p(const void* logits, int64_t row_stride, const flo
   if (rows == 0) return PH_OK;
   if (!logits || !uniform || !out_ids) return PH_ERR_ARG;
   if (rows > 0x7fffffff) return PH_ERR_ARG;
-  const SampArgs a{logits, row_stride, temperature, top_p, uniform, out_ids, (int)vocab};
+  const SampArgs a{logits, row_stride, temperature, top_p, uniform, out_ids, (int)vocab, nullptr, 0};
   hipStream_t st = (hipStream_t)stream;
   if (dtype == PH_F16) return launch_sample<F16>(a, rows, st);
   if (dtype == PH_BF16) return launch_sample<BF16>(a, rows, st);
   return launch_sample<F32>(a, rows, st);
+}
+
+template <typename E>
+static int launch_probs(const SampArgs& a, int64_t rows, hipStream_t st) {
+  dim3 grid((unsigned)rows), block(kSampThreads);
+  if (a.V <= kSampLdsFloats) {
+    const size_t lds = (size_t)a.V * sizeof(float);
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&sample_top_p_kernel<E, true>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, kSampLdsFloats * (int)sizeof(float));
+    hipLaunchKernelGGL((sample_top_p_kernel<E, true>), grid, block, lds, st, a);
+  } else {
+    hipLaunchKernelGGL((sample_top_p_kernel<E, false>), grid, block, 0, st, a);
+  }
+  return launch_status();
+}
+
+extern "C" int ph_top_p_probs(const void* logits, int64_t row_stride, const float* temperature, const float* top_p,
+                              float* probs, int64_t probs_stride, int64_t rows, int64_t vocab, int dtype,
+                              void* stream) {
+  if (rows < 0 || vocab <= 0 || vocab >= ((int64_t)1 << 30) || row_stride < vocab || probs_stride < vocab)
+    return PH_ERR_ARG;
+  if (dtype != PH_F16 && dtype != PH_BF16 && dtype != PH_F32) return PH_ERR_DTYPE;
+  if (rows == 0) return PH_OK;
+  if (!logits || !probs || rows > 0x7fffffff) return PH_ERR_ARG;
+  const SampArgs a{logits, row_stride, temperature, top_p, nullptr, nullptr, (int)vocab, probs, probs_stride};
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == PH_F16) return launch_probs<F16>(a, rows, st);
+  if (dtype == PH_BF16) return launch_probs<BF16>(a, rows, st);
+  return launch_probs<F32>(a, rows, st);
 }

@@ -310,6 +310,24 @@ def sample_top_p(logits: torch.Tensor, temperature: Optional[torch.Tensor], top_
     return out
 
 
+def top_p_probs(logits: torch.Tensor, temperature: Optional[torch.Tensor], top_p: Optional[torch.Tensor]) -> torch.Tensor:
+    """The distribution the reference's sampler draws from (models/sampler.py:33-64 up to the ``torch.multinomial``
+    call): temperature in the element type, top-p filter, soft-max of the survivors in fp32; dropped tokens get 0.
+    ``torch.multinomial(top_p_probs(...), 1, replacement=True)`` is then the reference's own draw."""
+    _require_gpu(logits, temperature, top_p)
+    assert logits.dim() == 2 and logits.stride(1) == 1
+    B, V = logits.shape
+    code = _dtype_code(logits)
+    for name, v in (("temperature", temperature), ("top_p", top_p)):
+        if v is not None and (v.dtype != torch.float32 or v.numel() != B or not v.is_contiguous()):
+            raise ValueError(f"{name} must be a contiguous float32 tensor of {B} elements")
+    probs = torch.empty((B, V), dtype=torch.float32, device=logits.device)
+    check(_lib.load().ph_top_p_probs(_ptr(logits), logits.stride(0) if B > 1 else max(logits.stride(0), V),
+                                     _ptr(temperature), _ptr(top_p), _ptr(probs), probs.stride(0), B, V, code,
+                                     _stream()), "top_p_probs")
+    return probs
+
+
 def silu_and_mul(out: torch.Tensor, input: torch.Tensor) -> None:
     """vLLM's form (3rdparty/vllm/csrc/activation.cpp:3-6): ``input`` is ``[T, 2d]`` = gate | up."""
     d = input.shape[-1] // 2

@@ -83,6 +83,10 @@ class Sampler(nn.Module):
     in torch's generator (same seed, same tokens from run to run) and follow the reference's distribution, but for a
     given seed they are NOT the ids the reference's ``torch.multinomial`` call would draw."""
 
+    # True: the draw is the reference's own call, ``torch.multinomial`` on the filtered probabilities (the library's
+    # random stream; one more launch and a [B, V] fp32 tensor), instead of the kernel's inverse-CDF draw
+    reference_draw = False
+
     def __init__(self, config: LlamaConfig, embd_weight: torch.Tensor):
         super().__init__()
         self.embd_weight = embd_weight
@@ -98,6 +102,9 @@ class Sampler(nn.Module):
         top_ps = [sc.top_p for sc in sampling_config]
         t_dev = torch.tensor(temperature, dtype=torch.float, device=dev) if any(t != 1.0 for t in temperature) else None
         p_dev = torch.tensor(top_ps, dtype=torch.float, device=dev) if any(p < 1.0 for p in top_ps) else None
+        if self.reference_draw:
+            probs = kernels.top_p_probs(logits, t_dev, p_dev)
+            return torch.multinomial(probs, num_samples=1, replacement=True).squeeze(-1)
         uniform = torch.rand(logits.shape[0], dtype=torch.float, device=dev)
         return kernels.sample_top_p(logits, t_dev, p_dev, uniform)
 

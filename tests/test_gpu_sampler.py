@@ -157,3 +157,59 @@ def test_sampler_module_uses_the_kernel():
     b = s(h, [SamplingConfig(temperature=0.8, top_p=0.9)] * 8)
     assert torch.equal(a, b) and int(a.min()) >= 0 and int(a.max()) < 4096
     assert s(h[:0], []).shape == (0,)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
+@pytest.mark.parametrize("B,V", [(16, 32000), (3, 1003), (2, 50257)])
+def test_filtered_probabilities_match_oracle(dtype, B, V):
+    """ph_top_p_probs: the tensor the reference hands to torch.multinomial (models/sampler.py:58-64) -- soft-max of
+    the tokens the top-p filter keeps, zero elsewhere -- against the float64 oracle, on rows whose cut is clear of
+    rounding noise: same support, probabilities to fp32 accuracy."""
+    x, temps, tops, _ = _case(31 + V, B, V, dtype)
+    dev = torch.device("cuda:0")
+    probs = kernels.top_p_probs(x.to(dev), temps.to(dev), tops.to(dev)).cpu().double().numpy()
+    assert probs.shape == (B, V)
+    compared = 0
+    for b in range(B):
+        want, margin = rs.kept_probs(x[b].double().numpy(), float(temps[b]), float(tops[b]), dtype)
+        np.testing.assert_allclose(probs[b].sum(), 1.0, rtol=1e-5)
+        if margin < MARGIN:
+            continue
+        compared += 1
+        assert ((probs[b] > 0) == (want > 0)).all(), f"row {b}: support differs"
+        np.testing.assert_allclose(probs[b], want, rtol=2e-5, atol=1e-9)
+    assert compared >= 0.8 * B
+
+
+def test_reference_draw_mode_of_the_sampler_module():
+    """Sampler.reference_draw: torch.multinomial on the kernel's filtered probabilities -- the reference's own call
+    sequence from there on (models/sampler.py:63-64), so for one seed the ids equal torch.multinomial's on the oracle
+    path of torch ops (division, sort, cumulative sum, mask, soft-max) whenever the two probability tensors agree."""
+    from parrotserve_amd.runner import LlamaConfig, Sampler, SamplingConfig
+
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(4)
+    W = (torch.randn(4096, 256, generator=g) * 0.3).half().to(dev)  # logits of a few units: a nucleus of tens of tokens
+    h = torch.randn(16, 256, generator=g).half().to(dev)
+    s = Sampler(LlamaConfig(vocab_size=4096, hidden_size=256), W)
+    s.reference_draw = True
+    cfgs = [SamplingConfig(temperature=0.8, top_p=0.9)] * 16
+    torch.manual_seed(11)
+    ids = s(h, cfgs)
+    assert ids.shape == (16,) and ids.dtype == torch.int64
+    # the reference's sequence of torch calls on the same logits, same seed
+    logits = torch.matmul(h, W.t())
+    logits.div_(torch.full((16, 1), 0.8, dtype=logits.dtype, device=dev))
+    sl, si = logits.sort(dim=-1, descending=True)
+    pr = sl.softmax(dim=-1)
+    mask = (pr.cumsum(dim=-1) - pr) > torch.full((16, 1), 0.9, dtype=logits.dtype, device=dev)
+    sl[mask] = -float("inf")
+    logits = torch.gather(sl, dim=-1, index=torch.argsort(si, dim=-1))
+    probs = torch.softmax(logits, dim=-1, dtype=torch.float)
+    torch.manual_seed(11)
+    want = torch.multinomial(probs, num_samples=1, replacement=True).squeeze(-1)
+    mine = kernels.top_p_probs(torch.matmul(h, W.t()), torch.full((16,), 0.8, device=dev), torch.full((16,), 0.9, device=dev))
+    same_support = ((mine > 0) == (probs > 0)).all(dim=-1)
+    # (the torch path rounds its probabilities and their running sums to fp16, which can move a cut by a token)
+    assert same_support.float().mean() >= 0.75
+    assert torch.equal(ids[same_support], want[same_support])
