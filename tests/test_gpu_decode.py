@@ -378,9 +378,9 @@ def test_unsupported_inputs_raise(dev):
     t = kernels.DecodeTables.build([], [], [[0, 1], [2]], dev)
     with pytest.raises(RuntimeError, match="head size"):
         kernels.decode_attention(q, kc, kc, t)
-    q32 = torch.zeros(2, 2, 128, dtype=torch.float32, device=dev)
+    q64 = torch.zeros(2, 2, 128, dtype=torch.float64, device=dev)  # float16 / bfloat16 / float32 are the element types
     with pytest.raises(RuntimeError, match="data type"):
-        kernels.decode_attention(q32, q32.new_zeros(8, 2, 128), q32.new_zeros(8, 2, 128), t)
+        kernels.decode_attention(q64, q64.new_zeros(8, 2, 128), q64.new_zeros(8, 2, 128), t)
 
 
 def test_balanced_and_grid_suffix_forms_agree(dev):
