@@ -236,6 +236,26 @@ def extras(torch, dev):
     out["c4_prefill"] = {"tokens": T, "chunks": len(c4.q_lens), "ms": t_pre * 1e3, "flops": flops,
                          "TFLOP/s": flops / t_pre / 1e12, "frac_mfma_peak": flops / t_pre / 1e12 / MFMA_F16_PEAK_TFLOPS,
                          "tokens/s/layer": T / t_pre}
+    # Where the distance between the chunk figure and the matrix peak lies: the tile loop alone, measured as the
+    # time one 1024-query chunk (160 workgroups, all resident at once, K/V warm in the last-level cache) gains
+    # when its parent grows by 4096 tokens = 64 steps of 64 tokens for every workgroup.
+    n1, pool1 = 1024, kc4.shape[0]
+    g1 = torch.Generator().manual_seed(11)
+    q1 = torch.randn((n1, H4, D), device=dev, dtype=torch.bfloat16)
+    o1 = torch.empty_like(q1)
+    ts = {}
+    for par1 in (2048, 6144):
+        slots1 = torch.randperm(pool1, generator=g1)[: par1 + n1].tolist()
+        tab1 = kernels.PrefillTables.build([n1], [slots1], dev)
+        ts[par1] = _time_gpu(torch, lambda: kernels.prefill_attention(q1, kc4, vc4, tab1, out=o1), iters=10)
+    step_s = (ts[6144] - ts[2048]) / 64
+    step_flops = 4 * 256 * 64 * D  # one 256-query workgroup, one head, one step
+    out["c4_prefill"]["tile_loop"] = {
+        "what": "one 1024-query chunk, parent 2048 -> 6144 tokens: time gained / 64 steps",
+        "us_per_64_token_step": step_s * 1e6,
+        "frac_mfma_peak_if_every_cu_ran_the_loop":
+            step_flops * torch.cuda.get_device_properties(dev).multi_processor_count / step_s / 1e12 / MFMA_F16_PEAK_TFLOPS,
+        "us_parent_2048": ts[2048] * 1e6, "us_parent_6144": ts[6144] * 1e6}
     del kc4, vc4, qkvs
     # --- config 5: full LLaMA-13B decoder layer, 4 prefix groups x 32 branches, prefix 6000 ------------------
     out["c5_layer"] = config5_layer(torch, dev)
