@@ -155,6 +155,11 @@ def extras(torch, dev):
     t_copy = _time_gpu(torch, lambda: kernels.discontinuous_move_tokens(kc[:half], kc[half:], ident, ident))
     out["c3_token_move"]["same_rows_in_order_us"] = t_copy * 1e6
     out["c3_token_move"]["same_rows_in_order_frac_hbm"] = nbytes / t_copy / 1e9 / HBM_PEAK_GBS
+    # one side scattered, the other in order: which side of a scattered move costs what
+    t_sr = _time_gpu(torch, lambda: kernels.discontinuous_move_tokens(kc, kc[half:], src, ident))
+    t_dr = _time_gpu(torch, lambda: kernels.discontinuous_move_tokens(kc[:half], kc, ident, dst))
+    out["c3_token_move"]["scattered_reads_ordered_writes_us"] = t_sr * 1e6
+    out["c3_token_move"]["ordered_reads_scattered_writes_us"] = t_dr * 1e6
     # --- the same 65,536 rows gathered out of the block-structured layouts (block 16, x 8) of a 4M-slot cache:
     # whole blocks in random order (a context that owns its blocks) and fully random slots -----------------------
     bs, x = 16, 8
@@ -203,6 +208,18 @@ def extras(torch, dev):
 
     t_rope = _time_gpu(torch, rope_step)
     rope_bytes = 2 * T * 2 * H4 * D * 2 + T * D * 2
+    # the same kernel on q and k rows that lie side by side without the v third between them, and the library's
+    # element-wise in-place kernel over the same bytes: what an in-place pass of this size reaches on this device
+    qks = [torch.randn((T, 2 * H4 * D), device=dev, dtype=torch.bfloat16) for _ in range(6)]
+    rot2 = _Rotor(len(qks))
+
+    def rope_dense_step():
+        qi, ki = qks[rot2.next()].chunk(2, dim=-1)
+        kernels.vllm_rotary_emb(pos, qi, ki, cache, D)
+
+    t_rope_dense = _time_gpu(torch, rope_dense_step)
+    t_rmw = _time_gpu(torch, lambda: qks[rot2.next()].mul_(1.0001))
+    del qks
     new_slots = torch.cat([c4.used_slots[n] for n in c4.new_lists]).to(torch.int32).to(dev)
     k3, v3 = k4.view(T, H4, D), v4.view(T, H4, D)
 
@@ -225,7 +242,10 @@ def extras(torch, dev):
     par = c4.parent_lists[0].numel()
     flops = 4 * H4 * D * sum(n * par + n * (n + 1) // 2 for n in c4.q_lens)
     out["c4_rope"] = {"tokens": T, "us": t_rope * 1e6, "GB/s": rope_bytes / t_rope / 1e9,
-                      "frac_hbm": rope_bytes / t_rope / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": rope_bytes}
+                      "frac_hbm": rope_bytes / t_rope / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": rope_bytes,
+                      "q_k_rows_without_v_between_us": t_rope_dense * 1e6,
+                      "q_k_rows_without_v_between_frac_hbm": rope_bytes / t_rope_dense / 1e9 / HBM_PEAK_GBS,
+                      "torch_mul_in_place_same_bytes_us": t_rmw * 1e6}
     app_bytes = 2 * 2 * T * H4 * D * 2
     out["c4_kv_append"] = {"tokens": T, "us": t_app * 1e6, "GB/s": app_bytes / t_app / 1e9,
                            "frac_hbm": app_bytes / t_app / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": app_bytes}
