@@ -234,6 +234,12 @@ def extras(torch, dev):
         kernels.rope_and_cache(pos, qi, ki, vi, cache, D, kc4, vc4, new_slots)
 
     t_fused = _time_gpu(torch, fused_step)
+
+    def fused_cache_only_step():  # the layer's form: attention reads K from the cache, k is not written back
+        qi, ki, vi = qkvs[rot.next()].chunk(3, dim=-1)
+        kernels.rope_and_cache(pos, qi, ki, vi, cache, D, kc4, vc4, new_slots, key_in_place=False)
+
+    t_fused_co = _time_gpu(torch, fused_cache_only_step)
     ctx = [c4.used_slots[torch.cat([p, n])].tolist() for p, n in zip(c4.parent_lists, c4.new_lists)]
     ptab = kernels.PrefillTables.build(c4.q_lens, ctx, dev)
     qc = q4.reshape(T, H4, D).contiguous()
@@ -253,6 +259,11 @@ def extras(torch, dev):
     out["c4_rope_append_fused"] = {"tokens": T, "us": t_fused * 1e6, "GB/s": fused_bytes / t_fused / 1e9,
                                    "frac_hbm": fused_bytes / t_fused / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": fused_bytes,
                                    "unfused_us": (t_rope + t_app) * 1e6}
+    co_bytes = fused_bytes - T * H4 * D * 2
+    out["c4_rope_append_fused_k_to_cache_only"] = {
+        "tokens": T, "us": t_fused_co * 1e6, "GB/s": co_bytes / t_fused_co / 1e9,
+        "frac_hbm": co_bytes / t_fused_co / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": co_bytes,
+        "unfused_us": (t_rope + t_app) * 1e6}
     out["c4_prefill"] = {"tokens": T, "chunks": len(c4.q_lens), "ms": t_pre * 1e3, "flops": flops,
                          "TFLOP/s": flops / t_pre / 1e12, "frac_mfma_peak": flops / t_pre / 1e12 / MFMA_F16_PEAK_TFLOPS,
                          "tokens/s/layer": T / t_pre}

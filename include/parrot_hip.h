@@ -381,7 +381,13 @@ int ph_prefill_attention(void* out, const void* q, const void* k_cache, const vo
  * the rotated k rows and the v rows go to their slots (as ph_kv_append) --
  * one pass over k instead of two.  Replaces rotary_embedding_neox +
  * reshape_and_cache (pos_encoding_kernels.cu:38-104, cache_kernels.cu:142-224)
- * as called back to back in models/llama.py:122-129 / attn_func.py:143-155. */
+ * as called back to back in models/llama.py:122-129 / attn_func.py:143-155.
+ * k_in_place = 1: k holds the rotated rows afterwards, as after the reference's
+ * two calls.  k_in_place = 0: the rotated k rows go to the cache only and the
+ * contents of k after the call are unspecified -- for a caller whose attention
+ * reads K from the cache (the model code does: attn_func.py:143-155 appends, then
+ * every kernel gathers from the cache); the pass then skips the write-back of
+ * the k rows. */
 int ph_add_rms_norm(void* out, void* residual, const void* x, const void* weight, float eps,
                     int64_t rows, int64_t n, int64_t x_stride, int64_t residual_stride,
                     int64_t out_stride, int dtype, int round_before_weight, void* stream);
@@ -394,7 +400,7 @@ int ph_rope_append(const int64_t* positions, void* q, void* k, const void* v,
                    const void* slot_mapping, int index_type, int64_t num_tokens,
                    int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim, int64_t rot_dim,
                    int64_t q_stride, int64_t k_stride, int64_t v_stride, int64_t cache_stride_n,
-                   int dtype, void* stream);
+                   int dtype, int k_in_place, void* stream);
 
 /* ------------------------------------------------------------------------ */
 /* Incremental suffix tables.  The reference rebuilds paged_block_tables /

@@ -39,7 +39,7 @@ SIGNATURES: Dict[str, Tuple[object, List[object]]] = {
     "ph_prefix_post_attention": (I, [P, P, P, P, P, P, L, L, L, I, L, L, L, F, P, L, P, Z, P]),
     "ph_add_rms_norm": (I, [P, P, P, P, F, L, L, L, L, L, I, I, P]),
     "ph_silu_mul": (I, [P, P, P, L, L, L, L, L, I, P]),
-    "ph_rope_append": (I, [P, P, P, P, P, P, P, P, I, L, L, L, L, L, L, L, L, L, I, P]),
+    "ph_rope_append": (I, [P, P, P, P, P, P, P, P, I, L, L, L, L, L, L, L, L, L, I, I, P]),
     "ph_suffix_tables_append": (I, [P, L, P, P, P, L, P]),
     "ph_decode_static_scratch_bytes": (Z, []),
     "ph_decode_attention_static": (I, [P, P, P, P, L, L, L, I, L, L, L, F, L, P, P, P, P, L, P, P, L, L, P, L, L, P, P]),

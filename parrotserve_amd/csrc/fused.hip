@@ -186,15 +186,17 @@ static int launch_silu_mul(void* out, const void* gate, const void* up, int64_t 
   return launch_status();
 }
 
-// One workgroup per token: rotate q and k heads in place (whole head rotated: rot_dim == head_dim), write the
-// rotated k row and the v row to the token's slot.
+// One workgroup per token: rotate q and k heads (whole head rotated: rot_dim == head_dim), q in place, write the
+// rotated k row and the v row to the token's slot; k itself is rewritten only when the caller wants it
+// (k_in_place): a caller that reads K from the cache from here on saves the read-modify-write of the k rows,
+// a quarter of the pass's time.
 template <typename E, typename IDX>
 __global__ __launch_bounds__(256) void rope_append_vec(const int64_t* __restrict__ positions, uint16_t* q, uint16_t* k,
                                                        const uint16_t* __restrict__ v,
                                                        const uint16_t* __restrict__ cos_sin, uint16_t* k_cache,
                                                        uint16_t* v_cache, const IDX* __restrict__ slot_mapping, int hq,
                                                        int hk, int D, int64_t q_stride, int64_t k_stride,
-                                                       int64_t v_stride, int64_t cache_stride) {
+                                                       int64_t v_stride, int64_t cache_stride, int k_in_place) {
   const int64_t t = blockIdx.x;
   const int64_t p = positions[t];
   const int64_t slot = (int64_t)slot_mapping[t];
@@ -206,25 +208,51 @@ __global__ __launch_bounds__(256) void rope_append_vec(const int64_t* __restrict
   const int v_units = hk * (D >> 3);
   uint16_t* kc = k_cache + slot * cache_stride;
   uint16_t* vc = v_cache + slot * cache_stride;
-  for (int u = threadIdx.x; u < rot_units + v_units; u += 256) {
-    if (u < rot_units) {
-      const int h = u / upd;
-      const int c = (u - h * upd) * 8;
-      const bool is_k = h >= hq;
-      uint16_t* base = is_k ? k + t * k_stride + (int64_t)(h - hq) * D : q + t * q_stride + (int64_t)h * D;
-      u32x4 x = ld16_nt(base + c), y = ld16_nt(base + half + c);
-      rotate8<E>(x, y, ld16(cr + c), ld16(sr + c));
-      st16(base + c, x);
-      st16(base + half + c, y);
-      if (is_k) {
-        uint16_t* dst = kc + (int64_t)(h - hq) * D;
-        st16(dst + c, x);
-        st16(dst + half + c, y);
+  // UN units per thread and pass, every load of the pass issued before the first rotation or store (a thread
+  // keeps up to 4 UN 16-byte loads in flight); rotation units first, then the v row's copy units
+  constexpr int UN = 3;
+  for (int u0 = threadIdx.x; u0 < rot_units; u0 += 256 * UN) {
+    uint16_t* base[UN];
+    int cc[UN], hh[UN];
+    u32x4 x[UN], y[UN], cs[UN], sn[UN];
+#pragma unroll
+    for (int j = 0; j < UN; ++j) {
+      const int u = u0 + j * 256;
+      if (u < rot_units) {
+        const int h = u / upd;
+        hh[j] = h;
+        cc[j] = (u - h * upd) * 8;
+        base[j] = h >= hq ? k + t * k_stride + (int64_t)(h - hq) * D : q + t * q_stride + (int64_t)h * D;
+        x[j] = ld16_nt(base[j] + cc[j]);
+        y[j] = ld16_nt(base[j] + half + cc[j]);
+        cs[j] = ld16(cr + cc[j]);
+        sn[j] = ld16(sr + cc[j]);
       }
-    } else {
-      const int c = (u - rot_units) * 8;
-      st16(vc + c, ld16_nt(v + t * v_stride + c));
     }
+#pragma unroll
+    for (int j = 0; j < UN; ++j) {
+      if (u0 + j * 256 < rot_units) {
+        rotate8<E>(x[j], y[j], cs[j], sn[j]);
+        if (k_in_place || hh[j] < hq) {
+          st16(base[j] + cc[j], x[j]);
+          st16(base[j] + half + cc[j], y[j]);
+        }
+        if (hh[j] >= hq) {
+          uint16_t* dst = kc + (int64_t)(hh[j] - hq) * D;
+          st16(dst + cc[j], x[j]);
+          st16(dst + half + cc[j], y[j]);
+        }
+      }
+    }
+  }
+  for (int u0 = threadIdx.x; u0 < v_units; u0 += 256 * UN) {
+    u32x4 w[UN];
+#pragma unroll
+    for (int j = 0; j < UN; ++j)
+      if (u0 + j * 256 < v_units) w[j] = ld16_nt(v + t * v_stride + (u0 + j * 256) * 8);
+#pragma unroll
+    for (int j = 0; j < UN; ++j)
+      if (u0 + j * 256 < v_units) st16(vc + (u0 + j * 256) * 8, w[j]);
   }
 }
 
@@ -261,7 +289,7 @@ extern "C" int ph_rope_append(const int64_t* positions, void* q, void* k, const 
                               void* k_cache, void* v_cache, const void* slot_mapping, int index_type,
                               int64_t num_tokens, int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim,
                               int64_t rot_dim, int64_t q_stride, int64_t k_stride, int64_t v_stride,
-                              int64_t cache_stride_n, int dtype, void* stream) {
+                              int64_t cache_stride_n, int dtype, int k_in_place, void* stream) {
   if (num_tokens < 0 || num_q_heads <= 0 || num_kv_heads <= 0 || head_dim <= 0 || rot_dim <= 0 || rot_dim % 2 ||
       rot_dim > head_dim)
     return PH_ERR_ARG;
@@ -285,7 +313,7 @@ extern "C" int ph_rope_append(const int64_t* positions, void* q, void* k, const 
   hipLaunchKernelGGL((rope_append_vec<E, IDX>), grid, block, 0, st, positions, (uint16_t*)q, (uint16_t*)k,         \
                      (const uint16_t*)v, (const uint16_t*)cos_sin_cache, (uint16_t*)k_cache, (uint16_t*)v_cache,   \
                      (const IDX*)slot_mapping, (int)num_q_heads, (int)num_kv_heads, (int)head_dim, q_stride,       \
-                     k_stride, v_stride, cache_stride_n)
+                     k_stride, v_stride, cache_stride_n, k_in_place)
   if (dtype == PH_F16) {
     if (index_type == PH_IDX_I64) PH_GO(F16, int64_t); else PH_GO(F16, int32_t);
   } else {

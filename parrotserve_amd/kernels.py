@@ -334,9 +334,12 @@ def silu_and_mul(out: torch.Tensor, input: torch.Tensor) -> None:
     silu_mul(input[..., :d], input[..., d:], out=out)
 
 
-def rope_and_cache(positions, query, key, value, cos_sin_cache, head_size, key_cache, value_cache, slot_mapping):
+def rope_and_cache(positions, query, key, value, cos_sin_cache, head_size, key_cache, value_cache, slot_mapping,
+                   key_in_place=True):
     """``vllm_rotary_emb(positions, query, key, ...)`` followed by ``vllm_reshape_and_cache(key, value, ...)``
-    in one launch: q and k rotated in place, rotated k rows and v rows written to their slots."""
+    in one launch: q and k rotated in place, rotated k rows and v rows written to their slots.
+    ``key_in_place=False``: the caller reads K from the cache from here on, so ``key`` is not written back
+    (its contents afterwards are unspecified) and the pass is a quarter shorter."""
     _require_gpu(query, key, value, key_cache, value_cache, cos_sin_cache, positions, slot_mapping)
     assert positions.dtype == torch.int64 and positions.dim() == 1
     T = positions.shape[0]
@@ -351,7 +354,8 @@ def rope_and_cache(positions, query, key, value, cos_sin_cache, head_size, key_c
     check(_lib.load().ph_rope_append(_ptr(positions), _ptr(q2), _ptr(k2), _ptr(v2), _ptr(cos_sin_cache),
                                      _ptr(key_cache), _ptr(value_cache), _ptr(slot_mapping), _index_code(slot_mapping),
                                      T, hq, hk, head_size, cos_sin_cache.shape[-1], q2.stride(0), k2.stride(0),
-                                     v2.stride(0), key_cache.stride(0), _dtype_code(query), _stream()),
+                                     v2.stride(0), key_cache.stride(0), _dtype_code(query), 1 if key_in_place else 0,
+                                     _stream()),
           "rope_and_cache")
 
 

@@ -67,8 +67,9 @@ class LlamaAttention(nn.Module):
         qkv = self.qkv_proj(hidden_states)
         q, k, v = torch.chunk(qkv, 3, dim=-1)
         if self.fused_ops:
+            # attention reads K from the cache only (kv_appended below), so k need not be rotated in place
             rope_and_cache(positions, q, k, v, get_cos_sin_cache(), self.head_dim, get_k_cache(self.layer_idx),
-                           get_v_cache(self.layer_idx), iteration_state.slot_mapping)
+                           get_v_cache(self.layer_idx), iteration_state.slot_mapping, key_in_place=False)
         else:
             vllm_rotary_emb(positions, q, k, get_cos_sin_cache(), head_size=self.head_dim)
         q = q.view(-1, self.num_heads, self.head_dim)

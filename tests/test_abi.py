@@ -73,11 +73,11 @@ def test_argument_validation_needs_no_gpu():
     assert lib.ph_silu_mul(None, None, None, 4, 0, 8, 8, 8, 0, None) == _lib.PH_ERR_ARG
     assert lib.ph_silu_mul(None, None, None, 4, 8, 8, 8, 8, 5, None) == _lib.PH_ERR_DTYPE
     assert lib.ph_rope_append(None, None, None, None, None, None, None, None, 0, 4, 2, 2, 128, 130, 256, 256, 256, 256,
-                              0, None) == _lib.PH_ERR_ARG  # rotary size beyond the head size
+                              0, 1, None) == _lib.PH_ERR_ARG  # rotary size beyond the head size
     assert lib.ph_rope_append(None, None, None, None, None, None, None, None, 7, 4, 2, 2, 128, 128, 256, 256, 256, 256,
-                              0, None) == _lib.PH_ERR_ARG  # unknown index type
+                              0, 1, None) == _lib.PH_ERR_ARG  # unknown index type
     assert lib.ph_rope_append(None, None, None, None, None, None, None, None, 0, 0, 2, 2, 128, 128, 256, 256, 256, 256,
-                              0, None) == _lib.PH_OK       # no tokens
+                              0, 0, None) == _lib.PH_OK       # no tokens
     # gathers out of the block-structured layouts
     gk = lambda n, D, x, eb, idx=0: lib.ph_gather_blocked_k(None, None, None, None, idx, n, 2, D, 16, x, eb, 4096, 2048,
                                                             128, 8, 1, 256, 128, 1, None)

@@ -399,3 +399,10 @@ def test_rope_and_cache_equals_rope_then_append(dev, dtype, T, H, D, idx):
     assert torch.equal(_bits(kc1.cpu()), _bits(kc2.cpu())) and torch.equal(_bits(vc1.cpu()), _bits(vc2.cpu()))
     assert torch.equal(_bits(q1.cpu()), _bits(rq)) and torch.equal(_bits(k1.cpu()), _bits(rk))
     assert torch.equal(_bits(kc1.cpu()), _bits(kc_ref)) and torch.equal(_bits(vc1.cpu()), _bits(vc_ref))
+    # without the write-back of k: q, v and both pools as before (k itself is left to the op)
+    d3 = qkv.to(dev)
+    q3, k3, v3 = d3.chunk(3, dim=-1)
+    kc3, vc3 = kc0.to(dev), vc0.to(dev)
+    kernels.rope_and_cache(pos.to(dev), q3, k3, v3, cache.to(dev), D, kc3, vc3, sm.to(dev), key_in_place=False)
+    assert torch.equal(_bits(q3.cpu()), _bits(rq)) and torch.equal(_bits(v3.cpu()), _bits(qkv[:, 2 * H * D :]))
+    assert torch.equal(_bits(kc3.cpu()), _bits(kc_ref)) and torch.equal(_bits(vc3.cpu()), _bits(vc_ref))
