@@ -269,6 +269,58 @@ def test_head_mapping_must_be_identity(dev):
         fn(torch.arange(H, dtype=torch.int32, device=dev))
 
 
+def test_timed_call_is_the_same_call_with_timestamps(dev):
+    """``ph_decode_attention_timed`` launches what ``ph_decode_attention`` launches (same bits out) and stamps the
+    caller's events with its own dispatches: three begin / end pairs, each end after its begin, the merge after
+    the kernel that feeds it; a pair whose kernel the call does not launch (no separate prefix kernel when both
+    phases share one launch) stays unrecorded."""
+    import ctypes
+
+    from parrotserve_amd import kernels, synth
+
+    hip = ctypes.CDLL("libamdhip64.so")
+    hip.hipEventCreate.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
+    hip.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p, ctypes.c_void_p]
+    hip.hipEventDestroy.argtypes = [ctypes.c_void_p]
+    hip.hipEventSynchronize.argtypes = [ctypes.c_void_p]
+
+    def elapsed(a, b):
+        ms = ctypes.c_float()
+        rc = hip.hipEventElapsedTime(ctypes.byref(ms), a, b)
+        if rc != 0:
+            hip.hipGetLastError()
+            return None
+        return ms.value
+
+    g = torch.Generator().manual_seed(77)
+    for B, expect_prefix_pair in ((64, False), (16, True)):  # 64 requests: one launch for both phases; 16: two
+        s = torch.randint(1, 150, (B,), generator=g).tolist()
+        case = synth.make_decode_case("t", 500 + B, torch.float16, 1, B, 700, s, 8, 128, 1 << 14)
+        kc, vc = synth.pool_to_device(case.k_rows, case.v_rows, case.used_slots, case.pool_slots, dev)
+        tables = kernels.DecodeTables.build(case.pool_lists(case.prefix_lists), case.group_req_cu,
+                                            case.pool_lists(case.suffix_lists), dev, num_heads=8, head_dim=128)
+        q = case.q.to(dev)
+        plain = kernels.decode_attention(q, kc, vc, tables)
+        evs = (ctypes.c_void_p * 6)()
+        for i in range(6):
+            e = ctypes.c_void_p()
+            assert hip.hipEventCreate(ctypes.byref(e)) == 0
+            evs[i] = e
+        timed = kernels.decode_attention(q, kc, vc, tables, events6=evs)
+        torch.cuda.synchronize()
+        assert torch.equal(plain.view(torch.int16), timed.view(torch.int16))
+        t_prefix, t_suffix, t_merge = elapsed(evs[0], evs[1]), elapsed(evs[2], evs[3]), elapsed(evs[4], evs[5])
+        assert t_suffix is not None and 0 < t_suffix < 50 and t_merge is not None and 0 < t_merge < 50
+        assert elapsed(evs[3], evs[4]) >= 0  # the merge begins after the suffix kernel ended
+        assert (t_prefix is not None) == expect_prefix_pair
+        if expect_prefix_pair:
+            assert 0 < t_prefix < 50
+        for i in range(6):
+            hip.hipEventDestroy(evs[i])
+        ref = ref_decode_attention(case.q, case.k_rows, case.v_rows, case.full_lists())
+        torch.testing.assert_close(timed.cpu().float(), ref.float(), **TOL[torch.float16])
+
+
 @pytest.mark.parametrize("balanced", [True, False])
 def test_lengths_beyond_the_table_are_clamped(dev, balanced):
     """A context length larger than the table's width must not walk into the next request's row (or past the
