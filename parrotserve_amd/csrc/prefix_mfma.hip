@@ -500,7 +500,7 @@ struct NoMid {
   __device__ __forceinline__ void operator()() const {}
 };
 
-template <typename E, bool CAUSAL, int TQ, typename Mid = NoMid, int SUB = 1, bool HALF = false>
+template <typename E, bool CAUSAL, int TQ, typename Mid = NoMid, int SUB = 1, bool HALF = false, bool PRESC = false>
 __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* __restrict__ kc,
                                            const uint16_t* __restrict__ vc, int64_t row_stride, int head,
                                            float scale_log2e, char* smem, float16_t (&ofold)[4 / TQ], float& mfin,
@@ -609,9 +609,19 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
     for (int s = 0; s < 8; ++s) {
       u32x4 v = ld16(qp + 8 * s);
       if (!ok || !mine) v = u32x4{0, 0, 0, 0};
+      if (PRESC) {
+        // PRESC: q takes the factor scale * log2(e) here and is rounded to the element type again (what the
+        // reference's own prefix kernel does, shared_flash_decoding.py:100), and the exponent reference enters
+        // the score product as its initial accumulator: the product is the exponent's argument as it stands
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          v[j] = pack2<E>(Elem<E>::lo(v[j]) * scale_log2e, Elem<E>::hi(v[j]) * scale_log2e);
+      }
       qop[s] = v;
     }
   }
+  // PRESC: minus the exponent reference (0 while there is none) in all sixteen accumulator registers
+  float16_t cinit = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   // last token any query of this wave's block may see (none if the block has no live query)
   const int wave_last = 32 * qb >= wk.nq ? -1 : CAUSAL ? min(s1 - 1, wk.causal_off + 32 * qb + 31) : s1 - 1;
 
@@ -692,7 +702,7 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
       for (int s = 0; s < 8; ++s) ka[s] = lds_ld16_a(kaddr[shi][s] + slo);
       if (SUB == 1) __builtin_amdgcn_sched_barrier(0);
       const float16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-      sacc[sb] = Mfma32<E>::run(ka[0], qop[0], zero);
+      sacc[sb] = Mfma32<E>::run(ka[0], qop[0], PRESC ? cinit : zero);
 #pragma unroll
       for (int s = 1; s < 8; ++s) sacc[sb] = Mfma32<E>::run(ka[s], qop[s], sacc[sb]);
     }
@@ -737,14 +747,24 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
 #pragma unroll
       for (int r = 0; r < 16; r += 4)
         mloc = fmaxf(mloc, fmaxf(fmaxf(x[sb][r], x[sb][r + 1]), fmaxf(x[sb][r + 2], x[sb][r + 3])));
-    mloc = half_swap_max(mloc) * scale_log2e;  // scale > 0 keeps the order
+    const bool had = m != -INFINITY;
+    if (PRESC) mloc = half_swap_max(mloc) + (had ? m : 0.f);  // the scores are relative to the reference so far
+    else mloc = half_swap_max(mloc) * scale_log2e;              // scale > 0 keeps the order
     mtrue = fmaxf(mtrue, mloc);
     // lazy exponent reference: moves only when the maximum has outgrown it by more than kSlack
     const bool move = mloc > m + kSlack;
     const float mnew = move ? mloc : m;
     const float mref = (mnew == -INFINITY) ? 0.f : mnew;
-    const bool had = m != -INFINITY;
     const float alpha = (move && had) ? __builtin_amdgcn_exp2f(m - mref) : 1.f;
+    if (PRESC && __builtin_amdgcn_ballot_w64(move) != 0) {  // wave-uniform, rare: re-base the scores and the seed
+      const float delta = mref - (had ? m : 0.f);            // 0 on the lanes whose reference stays
+#pragma unroll
+      for (int sb = 0; sb < SUB; ++sb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) x[sb][r] -= delta;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) cinit[r] = -mref;
+    }
     m = mnew;
     if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {  // wave-uniform, rare
       // pinned in assembly so that the multiply stays inside this branch; wait states cover the matrix
@@ -761,7 +781,9 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
 #pragma unroll
     for (int sb = 0; sb < SUB; ++sb) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) x[sb][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(x[sb][r], scale_log2e, -mref));
+      for (int r = 0; r < 16; ++r)
+        x[sb][r] = PRESC ? __builtin_amdgcn_exp2f(x[sb][r])
+                         : __builtin_amdgcn_exp2f(__builtin_fmaf(x[sb][r], scale_log2e, -mref));
       u32x4 pop[2];
 #pragma unroll
       for (int u = 0; u < 2; ++u)
@@ -1018,7 +1040,8 @@ __global__ __launch_bounds__(512) void prefill_mfma8_kernel(PrefillArgs a) {
   wk.s1 = min(kvn, wk.causal_off + nq);  // the last live query sees tokens up to causal_off + nq - 1
   float16_t of[NDB];
   float m, l;
-  attn_tile8<E, true, TQ, NoMid, SUB, HALF>(wk, a.kc, a.vc, a.row_stride, head, a.scale_log2e, smem, of, m, l);
+  // the prefill loop is bound by instruction issue: the pre-scaled query saves it one multiply-add per score
+  attn_tile8<E, true, TQ, NoMid, SUB, HALF, true>(wk, a.kc, a.vc, a.row_stride, head, a.scale_log2e, smem, of, m, l);
   const int lane = threadIdx.x & 63, w8 = threadIdx.x >> 6, g = w8 / QB, qb = w8 % QB, h = lane >> 5, ql = lane & 31;
   const int q = 32 * qb + ql;
   if (q < nq) {
