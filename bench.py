@@ -348,6 +348,50 @@ def fused_timeline(torch, lib, step, launches=8):
     return out
 
 
+PREFILL_TIMELINE_MARKS = ["kernel entry", "slot window in LDS", "ring requested, q loaded", None,
+                          "step 0 (tile landed, workgroup barrier passed)", "step 1", "step 2", "step 3",
+                          "tile loop done", None, None, "kernel exit"]
+
+
+def prefill_timeline(torch, lib, dev, launches=6):
+    """The same marks in the prefill kernel: one 256-query chunk over a 2048-token parent, 40 heads = 40 workgroups
+    that all start at once, so a workgroup's prologue (entry to step 0) and epilogue (loop done to exit) can be
+    read off beside its tile loop."""
+    import numpy as np
+    from parrotserve_amd import kernels
+
+    H, D, pool, n, par = 40, 128, 1 << 15, 256, 2048
+    kc = torch.randn((pool, H, D), device=dev, dtype=torch.bfloat16)
+    vc = torch.randn_like(kc)
+    slots = torch.randperm(pool, generator=torch.Generator().manual_seed(7))[: par + n].tolist()
+    q = torch.randn((n, H, D), device=dev, dtype=torch.bfloat16)
+    o = torch.empty_like(q)
+    tab = kernels.PrefillTables.build([n], [slots], dev)
+    for _ in range(5):
+        kernels.prefill_attention(q, kc, vc, tab, out=o)
+    torch.cuda.synchronize()
+    runs = []
+    for _ in range(launches):
+        lib.ph_timeline_clear()
+        torch.cuda.synchronize()
+        kernels.prefill_attention(q, kc, vc, tab, out=o)
+        torch.cuda.synchronize()
+        buf = np.zeros(4096 * 12, dtype=np.uint64)
+        assert lib.ph_timeline_read(buf.ctypes.data_as(ctypes.c_void_p), buf.nbytes) == 0
+        t = buf.reshape(4096, 12).astype(np.float64)[: H * 8]
+        runs.append(np.where(t > 0, (t - t[:, 0][t[:, 0] > 0].min()) / 100.0, np.nan))
+    rel = np.nanmedian(np.stack(runs), axis=0)
+    out = {"waves": int(rel.shape[0]), "steps": (par + n) // 64, "unit": "us from the first wave's entry", "marks": {}}
+    for i, name in enumerate(PREFILL_TIMELINE_MARKS):
+        c = rel[:, i]
+        c = c[~np.isnan(c)]
+        if name is None or c.size == 0:
+            continue
+        out["marks"][name] = {k: round(float(v), 2) for k, v in
+                              zip(("min", "p10", "p50", "p90", "max"), np.percentile(c, [0, 10, 50, 90, 100]))}
+    return out
+
+
 def head_size_64_step(torch, dev):
     """Config 2's batch with 64-wide heads (32 x 64, the OPT-1.3B shape): the prefix phase runs on head pairs through
     the 128-wide matrix-core kernel, the suffix phase and the merge at the native width.  Warm (one KV set)."""
@@ -721,7 +765,8 @@ def main():
         return (time.perf_counter() - t0) / steps
 
     if args.timeline:
-        print(json.dumps({"fused_kernel_timeline": fused_timeline(torch, lib, step)}))
+        print(json.dumps({"fused_kernel_timeline": fused_timeline(torch, lib, step),
+                          "prefill_kernel_timeline": prefill_timeline(torch, lib, dev)}))
         return
 
     t_step = timed(step, args.steps, args.warmup)

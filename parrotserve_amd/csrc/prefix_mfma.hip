@@ -1012,6 +1012,7 @@ template <typename E, int TQ, int SUB, bool HALF = false>
 __global__ __launch_bounds__(512) void prefill_mfma8_kernel(PrefillArgs a) {
   constexpr int QB = 8 / TQ, NDB = 4 / TQ, QT = 32 * QB;
   extern __shared__ __attribute__((aligned(16))) char smem[];
+  PH_TL(0);
   if ((int)blockIdx.x >= a.H) return;
   // 64-wide heads: workgroup x is head x = half (x & 1) of pair x >> 1, whose K/V rows are one 128-wide row
   const int head = a.pair ? blockIdx.x >> 1 : blockIdx.x;
@@ -1062,6 +1063,7 @@ __global__ __launch_bounds__(512) void prefill_mfma8_kernel(PrefillArgs a) {
       }
     }
   }
+  PH_TL(11);
 }
 
 // tile_cu[c] = number of 64-query tiles before chunk c (serial scan; chunk counts are small)

@@ -24,7 +24,7 @@ Collection (on the GPU box, from /tmp with TMPDIR=/tmp; one rocprofv3 run per li
     pf2        rocprofv3 --pmc SQ_LDS_BANK_CONFLICT SQ_LDS_IDX_ACTIVE SQ_INSTS_LDS SQ_INSTS_VALU_TRANS_F32
                               SQ_INSTS_VMEM_RD SQ_INSTS_SALU SQ_WAIT_ANY SQ_WAVES -- python3 bench.py --prefill-only
     pf3        rocprofv3 --pmc GRBM_GUI_ACTIVE GRBM_COUNT -- python3 bench.py --prefill-only
-    timeline.json   python3 bench.py --timeline > <dir>/timeline.json   (no profiler)
+    timeline.json   python3 bench.py --timeline > <dir>/timeline.json   (no profiler; fused decode and prefill kernels)
 
 A missing run only leaves its summary out.  The profiler sums SQ / GRBM counters over the chip's 8 XCDs;
 FETCH_SIZE / WRITE_SIZE are KiB per dispatch and are scaled by what the same counters read for a plain copy of known
@@ -238,10 +238,28 @@ def main(d):
     # ---- timeline of the fused decode kernel ---------------------------------------------------------------------
     tl = os.path.join(d, "timeline.json")
     if os.path.exists(tl):
-        j = None
+        j = pj = None
         for line in open(tl):
             if line.startswith("{"):
-                j = json.loads(line)["fused_kernel_timeline"]
+                both = json.loads(line)
+                j = both["fused_kernel_timeline"]
+                pj = both.get("prefill_kernel_timeline")
+        if pj:
+            m = pj["marks"]
+            t = ["Where the waves of prefill_mfma8_kernel<bf16, 256-query tiles, 64-token steps> spend a launch: one 256-query chunk "
+                 f"over a 2048-token parent, 40 heads = 40 workgroups resident at once, {pj['steps']} steps each (per-wave timestamps at "
+                 "marks inside the kernel, profiling variant of the library; microseconds from the first wave's entry; median over 6 "
+                 "launches per wave, then the spread over the launch's 320 waves)",
+                 head + "command (on the GPU box; no profiler):\n  python3 bench.py --timeline", "",
+                 f"{'mark':50s} {'min':>7s} {'p10':>7s} {'p50':>7s} {'p90':>7s} {'max':>7s}"]
+            for k, v in m.items():
+                t.append(f"{k:50s} {v['min']:7.2f} {v['p10']:7.2f} {v['p50']:7.2f} {v['p90']:7.2f} {v['max']:7.2f}")
+            first = m["step 0 (tile landed, workgroup barrier passed)"]["p50"]
+            done, end = m["tile loop done"]["p50"], m["kernel exit"]["p50"]
+            t += ["", f"median wave: prologue (entry to step 0) {first - m['kernel entry']['p50']:.1f} us, tile loop {done - first:.1f} us = "
+                  f"{(done - first) / pj['steps']:.2f} us per step, epilogue (loop done to exit) {end - done:.1f} us"]
+            out["prefill_kernel_timeline"] = m
+            _write("prefill_tile_timeline.txt", "\n".join(t))
         if j:
             t = ["Where the waves of decode_fused_kernel spend a launch at config 2 (per-wave timestamps at marks inside the kernel, "
                  "profiling variant of the library; microseconds from the first wave's entry; median over 8 launches per wave, then "
