@@ -232,6 +232,21 @@ size_t ph_decode_workspace_bytes(int64_t num_reqs, int64_t num_heads, int64_t he
                                  int64_t num_groups, int64_t max_prefix_len,
                                  int64_t max_suffix_len, int64_t chunk_tokens, int64_t num_items);
 
+/* Number of pieces (num_lanes) a caller's balanced suffix plan should be cut
+ * into for a ph_decode_attention call of this shape: one round of waves, two
+ * per SIMD, on the compute units the suffix phase runs on.  That is every
+ * compute unit of the device, except where the library runs the prefix and
+ * suffix phases of a call in one launch with workgroups of their own (16-bit
+ * elements, head size 128 or paired 64, a suffix that moves about as many
+ * bytes as the prefixes or more): there the prefix keeps the compute units a
+ * cost model gives it and the suffix takes the rest.  A plan cut into more or
+ * fewer pieces stays correct (pieces beyond one round are taken in further
+ * rounds by the same waves); it is only slower.  Host-only, no launch.  The
+ * reference has no counterpart (fixed (request, block) grids,
+ * attention_post_kernels.cu:395-418). */
+int64_t ph_decode_suffix_lanes(int64_t num_reqs, int64_t num_heads, int64_t head_dim, int dtype,
+                               int64_t num_groups, int64_t max_prefix_len, int64_t max_suffix_len);
+
 int ph_decode_attention(void* out, const void* q, const void* k_cache, const void* v_cache,
                         int64_t num_reqs, int64_t num_heads, int64_t head_dim, int dtype,
                         int64_t q_stride, int64_t out_stride, int64_t cache_stride_n,

@@ -267,6 +267,9 @@ class HipSharedPrefixAttn(AttnFunc):
     @classmethod
     def init_iteration_state(cls, iteration_state, builtin_config, jobs, num_heads: int, head_size: int):
         device = builtin_config.device
+        dtype = getattr(builtin_config, "dtype", torch.float16)
+        if not isinstance(dtype, torch.dtype):
+            dtype = torch.float16
         st = iteration_state
         cached = cls.table_cache.advance(jobs, device) if cls.incremental else None
         if cached is not None:
@@ -295,7 +298,7 @@ class HipSharedPrefixAttn(AttnFunc):
                                             cls.forked_fill_pay_ratio)
             if forked is not None:
                 st.fill_decode_tables = kernels.DecodeTables.build(*forked, device, num_heads=num_heads,
-                                                                   head_dim=head_size)
+                                                                   head_dim=head_size, dtype=dtype)
             else:
                 st.fill_tables = kernels.PrefillTables.build(tabs.fill_q_lens, tabs.fill_slot_lists, device)
         st.decode_tables = None
@@ -311,7 +314,8 @@ class HipSharedPrefixAttn(AttnFunc):
             order.extend(i for i in range(tabs.num_generates) if i not in grouped)
             suffix = [tabs.paged_block_tables[i] for i in order]
             st.decode_tables = kernels.DecodeTables.build([p for p, _ in tabs.groups], gcu if tabs.groups else [],
-                                                          suffix, device, num_heads=num_heads, head_dim=head_size)
+                                                          suffix, device, num_heads=num_heads, head_dim=head_size,
+                                                          dtype=dtype)
             if order != list(range(tabs.num_generates)):
                 perm = torch.tensor(order, dtype=torch.int64, device=device)
                 inv = torch.empty_like(perm)
@@ -319,7 +323,7 @@ class HipSharedPrefixAttn(AttnFunc):
                 st.decode_perm = (perm, inv)
             if cls.incremental:
                 cls.table_cache.store(jobs, order, [len(x) for x in suffix], st.decode_tables, st.decode_perm,
-                                      tabs.flash_context_len, num_heads, head_size, device)
+                                      tabs.flash_context_len, num_heads, head_size, device, dtype)
         elif cls.incremental:
             cls.table_cache.clear()
 

@@ -2,7 +2,8 @@
 
 Run ``python -m parrotserve_amd.build`` or call ``build()``; the shared library
 lands next to the sources' package (parrotserve_amd/libparrot_hip.so) so it
-travels with the tree.
+travels with the tree.  ``python -m parrotserve_amd.build --timeline`` also links the
+profiling variant (libparrot_hip_timeline.so, what ``bench.py --timeline`` loads).
 """
 from __future__ import annotations
 
@@ -43,7 +44,8 @@ def _compile(src: str, obj_dir: str, timeline: bool = False) -> str:
     return obj
 
 
-def build(verbose: bool = True) -> str:
+def build(verbose: bool = True, timeline: bool = False) -> str:
+    """Compile and link the product library; ``timeline=True`` also links the profiling variant."""
     obj_dir = os.path.join(PKG_DIR, "build")
     os.makedirs(obj_dir, exist_ok=True)
     with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as ex:
@@ -54,6 +56,8 @@ def build(verbose: bool = True) -> str:
         raise RuntimeError(f"link failed:\n{r.stdout}\n{r.stderr}")
     if verbose:
         print(f"built {LIB_PATH}")
+    if not timeline:
+        return LIB_PATH
     # the profiling variant shares every object but the one that holds the marks
     tl_obj = _compile("prefix_mfma.hip", obj_dir, timeline=True)
     tl_objs = [tl_obj if o.endswith("prefix_mfma.o") else o for o in objs]
@@ -67,5 +71,5 @@ def build(verbose: bool = True) -> str:
 
 
 if __name__ == "__main__":
-    build()
+    build(timeline="--timeline" in sys.argv[1:])
     sys.exit(0)

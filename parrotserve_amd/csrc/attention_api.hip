@@ -3,6 +3,8 @@
 // enqueued on the caller's stream.
 #include "decode.hpp"
 
+#include <algorithm>
+#include <cstdlib>
 #include <mutex>
 
 namespace ph {
@@ -40,6 +42,7 @@ struct DecodePlan {
   int64_t items;     // suffix items (balanced form), 0 in the grid form
   int dev_lanes;     // lanes of a plan the library builds on the device into the workspace (0: the caller's plan or none)
   bool paired;       // D == 64: the prefix phase runs on head pairs through the 128-wide matrix-core kernel
+  int prefix_wgs;    // fused launch: workgroups that run only prefix units (0: every workgroup runs both phases)
   int parts() const { return n_chunks + n_splits; }
   // partial rows (one row = one head's (O, m, l)): [parts][B][H] then [items][H]
   size_t rows(int64_t B, int64_t H) const { return (size_t)parts() * B * H + (size_t)items * H; }
@@ -64,20 +67,110 @@ static int device_cus() {
   return cached[dev];
 }
 
+// How the fused launch divides the compute units (see decode_fused_kernel): a suffix that moves at least half as
+// many bytes as the prefixes (and 64 MB) gets workgroups of its own (roles), a shorter one rides inside the prefix
+// workgroups (shared); measured at batch 64 over 4096- and 8192-token prefixes, roles win from there on (by 11 %
+// at half the prefix's bytes over 8192 tokens, a tie at equal bytes over 4096) and lose below.  The suffix volume
+// is an estimate from what the host knows -- half the longest list per request.
+struct FusedShape {
+  int64_t units_per_split;  // prefix units (head x group x query tile) per split of the prefix
+  double prefix_mb, suffix_mb;
+  bool roles;
+};
+static FusedShape fused_shape(int64_t B, int64_t H, int64_t D, int64_t groups, int64_t max_prefix, int64_t max_suffix,
+                              bool paired) {
+  FusedShape f{};
+  if (groups <= 0 || max_prefix <= 0) return f;
+  const int64_t rows_b = paired ? 2 * B : B, rows_h = paired ? H / 2 : H;  // what the matrix-core kernel sees
+  const int64_t per_group = cdiv(rows_b, groups);
+  const int64_t qtile = per_group <= 64 ? 64 : per_group <= 128 ? 128 : 256;
+  const int64_t mtiles = cdiv(per_group, qtile);
+  f.units_per_split = groups * rows_h * (mtiles > 0 ? mtiles : 1);
+  const double row_mb = (double)H * D * 4 / 1e6;  // K and V of one token, 16-bit elements
+  f.prefix_mb = (double)groups * max_prefix * row_mb;
+  f.suffix_mb = (double)B * max_suffix / 2 * row_mb;
+  f.roles = f.suffix_mb >= 64.0 && f.suffix_mb >= 0.5 * f.prefix_mb;
+  return f;
+}
+
+// Roles: the split count and the number of prefix-only workgroups.  A prefix workgroup is latency-bound next to
+// the suffix stream -- one 128-token step (64 KB) in flight ahead of the one it multiplies, about 2.7 us per step
+// with the memory system saturated, 12 us from launch to its first step -- so the prefix wants enough workgroups
+// to be done a little before the stream, and the stream wants the rest (it holds about 40 GB/s per compute unit).
+// Both end no earlier than the bytes of the launch take at the rate the device sustains.
+struct RoleChoice {
+  int splits, prefix_wgs;
+};
+static RoleChoice choose_roles(const FusedShape& f, int64_t max_prefix, int64_t cus) {
+  constexpr double kHbm = 6.9, kCu = 0.040;  // MB per us: the device under this access mix, one compute unit streaming
+  constexpr double kStep = 2.7, kFirst = 12.0, kFold = 2.0, kNext = 6.0, kMargin = 3.0;
+  const double floor_us = 4.0 + (f.prefix_mb + f.suffix_mb) / kHbm;
+  RoleChoice best{1, 1};
+  double best_cost = -1.0;
+  const int64_t max_splits = std::max<int64_t>(1, cdiv(max_prefix, 4 * kPrefixTile));
+  for (int64_t s = 1; s <= 64 && s <= max_splits; ++s) {
+    const int64_t tok = round_up(cdiv(max_prefix, s), 2 * kPrefixTile);
+    if (cdiv(max_prefix, tok) != s) continue;  // rounding left a split empty: the same plan as a smaller s
+    const double steps = (double)cdiv(tok, 2 * kPrefixTile);
+    const int64_t units = f.units_per_split * s;
+    for (int64_t r = 1; r <= 8; ++r) {
+      const int64_t np = cdiv(units, r);
+      if (np > cus - 1) continue;
+      const double t_prefix = kFirst + r * (steps * kStep + kFold) + (r - 1) * kNext + kMargin;
+      const double t_suffix = 6.0 + f.suffix_mb / std::min(kHbm, (double)(cus - np) * kCu);
+      const double cost = std::max(std::max(t_prefix, t_suffix), floor_us) + 0.25 * s;
+      if (best_cost < 0 || cost < best_cost) {
+        best_cost = cost;
+        best = RoleChoice{(int)s, (int)np};
+      }
+    }
+  }
+  return best;
+}
+
 // plan_head_dim > 0: a caller without a plan of its own that leaves the chunk size to the library gets the
 // balanced form from a plan built on the device (up to kPlanMaxReqs requests); an explicit chunk size keeps the
-// plain (request, chunk) grid.
+// plain (request, chunk) grid.  roles: the fused launch may give the two phases workgroups of their own.
 static DecodePlan plan_decode(int64_t B, int64_t H, int64_t groups, int64_t max_prefix, int64_t max_suffix,
                               int64_t chunk_tokens, int64_t num_items = 0, int64_t plan_head_dim = 0,
-                              bool paired = false) {
+                              bool paired = false, bool roles = false) {
   DecodePlan p{};
   p.items = num_items;
+  const int64_t cus = device_cus();
+  if (groups > 0 && max_prefix > 0) {
+    p.paired = paired;
+    const FusedShape f = fused_shape(B, H, plan_head_dim > 0 ? plan_head_dim : 128, groups, max_prefix, max_suffix, paired);
+    int64_t splits = 1;
+    if (roles && f.roles && max_suffix > 0) {
+      const RoleChoice rc = choose_roles(f, max_prefix, cus);
+      splits = rc.splits;
+      p.prefix_wgs = rc.prefix_wgs;
+    } else {
+      // One workgroup per CU at a time (the kernel uses most of the register file), so pick the
+      // split count whose workgroup total wastes the least of a whole number of rounds over the device's CUs.
+      // Cost model: rounds x (tokens per split + a fixed prologue/epilogue worth ~96 tokens).
+      const int64_t max_splits = cdiv(max_prefix, 4 * kPrefixTile);
+      int64_t best = -1;
+      for (int64_t s = 1; s <= 64 && s <= (max_splits > 0 ? max_splits : 1); ++s) {
+        const int64_t tok = round_up(cdiv(max_prefix, s), 2 * kPrefixTile);
+        const int64_t cost = cdiv(f.units_per_split * s, cus) * (tok + 96);
+        if (best < 0 || cost < best) {
+          best = cost;
+          splits = s;
+        }
+      }
+    }
+    const int64_t st = round_up(cdiv(max_prefix, splits), 2 * kPrefixTile);
+    p.split_tokens = (int)st;
+    p.n_splits = (int)cdiv(max_prefix, st);
+  }
   if (num_items > 0) {
     p.chunk = 32;
     p.n_chunks = 0;
   } else if (max_suffix > 0 && chunk_tokens <= 0 && plan_head_dim >= 8 && B <= kPlanMaxReqs) {
     const int64_t heads_per_wave = 64 / lanes_per_head((int)plan_head_dim) > 0 ? 64 / lanes_per_head((int)plan_head_dim) : 1;
-    const int64_t lanes = (int64_t)device_cus() * 4 * 2 / cdiv(H, heads_per_wave);  // two waves per SIMD
+    // two waves per SIMD on the compute units the suffix phase has to itself
+    const int64_t lanes = (cus - p.prefix_wgs) * 4 * 2 / cdiv(H, heads_per_wave);
     p.dev_lanes = (int)(lanes > 0 ? lanes : 1);
     p.items = p.dev_lanes + B;  // capacity: a cut at every lane mark and every request boundary
     p.chunk = 32;
@@ -96,32 +189,6 @@ static DecodePlan plan_decode(int64_t B, int64_t H, int64_t groups, int64_t max_
   } else {
     p.chunk = 32;
     p.n_chunks = 0;
-  }
-  if (groups > 0 && max_prefix > 0) {
-    // One workgroup per CU at a time (the kernel uses most of the register file), so pick the
-    // split count whose workgroup total wastes the least of a whole number of rounds over the device's CUs.
-    // Cost model: rounds x (tokens per split + a fixed prologue/epilogue worth ~96 tokens).
-    // the kernel takes 64-, 128- or 256-query tiles by the largest group; the mean group size stands in here
-    p.paired = paired;
-    const int64_t rows_b = paired ? 2 * B : B, rows_h = paired ? H / 2 : H;  // what the kernel sees
-    const int64_t per_group = cdiv(rows_b, groups);
-    const int64_t qtile = per_group <= 64 ? kPrefixQueryTile : per_group <= 128 ? 2 * kPrefixQueryTile : 4 * kPrefixQueryTile;
-    const int64_t mtiles = cdiv(per_group, qtile);
-    const int64_t base = groups * rows_h * (mtiles > 0 ? mtiles : 1);
-    const int64_t max_splits = cdiv(max_prefix, 4 * kPrefixTile);
-    int64_t splits = 1, best = -1;
-    const int64_t cus = device_cus();
-    for (int64_t s = 1; s <= 64 && s <= (max_splits > 0 ? max_splits : 1); ++s) {
-      const int64_t tok = round_up(cdiv(max_prefix, s), 2 * kPrefixTile);
-      const int64_t cost = cdiv(base * s, cus) * (tok + 96);
-      if (best < 0 || cost < best) {
-        best = cost;
-        splits = s;
-      }
-    }
-    const int64_t st = round_up(cdiv(max_prefix, splits), 2 * kPrefixTile);
-    p.split_tokens = (int)st;
-    p.n_splits = (int)cdiv(max_prefix, st);
   }
   return p;
 }
@@ -274,10 +341,35 @@ extern "C" size_t ph_decode_workspace_bytes(int64_t num_reqs, int64_t num_heads,
                                             int64_t num_groups, int64_t max_prefix_len, int64_t max_suffix_len,
                                             int64_t chunk_tokens, int64_t num_items) {
   if (num_reqs <= 0 || num_heads <= 0 || head_dim <= 0) return 0;
-  const DecodePlan p =
-      plan_decode(num_reqs, num_heads, num_groups, max_prefix_len, max_suffix_len, chunk_tokens, num_items, head_dim,
-                  pair_heads(head_dim, num_heads));
-  return plan_bytes(p, num_reqs, num_heads, head_dim);
+  // the call picks one of two layouts (prefix and suffix workgroups of their own, or not) by what the element type
+  // and the group sizes allow, which this query does not see: large enough for either
+  size_t need = 0;
+  for (int roles = 0; roles < 2; ++roles) {
+    const DecodePlan p = plan_decode(num_reqs, num_heads, num_groups, max_prefix_len, max_suffix_len, chunk_tokens,
+                                     num_items, head_dim, pair_heads(head_dim, num_heads), roles != 0);
+    need = std::max(need, plan_bytes(p, num_reqs, num_heads, head_dim));
+  }
+  return need;
+}
+
+// can the prefix and suffix phases of this call share one launch with workgroups of their own?
+static bool roles_possible(int64_t B, int64_t H, int64_t D, int dtype, bool has_prefix, bool has_suffix, bool planned,
+                           int64_t chunk_tokens) {
+  if (!has_prefix || !has_suffix) return false;
+  if (!planned && !(chunk_tokens <= 0 && B <= kPlanMaxReqs)) return false;  // no balanced plan: the grid form
+  return pair_heads(D, H) ? decode_fused_supported(dtype, 128) : decode_fused_supported(dtype, (int)D);
+}
+
+extern "C" int64_t ph_decode_suffix_lanes(int64_t num_reqs, int64_t num_heads, int64_t head_dim, int dtype,
+                                          int64_t num_groups, int64_t max_prefix_len, int64_t max_suffix_len) {
+  if (num_reqs <= 0 || num_heads <= 0 || head_dim < 8) return 1;
+  const bool has_prefix = num_groups > 0 && max_prefix_len > 0;
+  const bool roles = roles_possible(num_reqs, num_heads, head_dim, dtype, has_prefix, max_suffix_len > 0, true, 0);
+  const DecodePlan p = plan_decode(num_reqs, num_heads, has_prefix ? num_groups : 0, max_prefix_len, max_suffix_len, 0,
+                                   1, head_dim, pair_heads(head_dim, num_heads), roles);
+  const int64_t heads_per_wave = std::max(1, 64 / lanes_per_head((int)head_dim));
+  const int64_t lanes = ((int64_t)device_cus() - p.prefix_wgs) * 4 * 2 / cdiv(num_heads, heads_per_wave);
+  return lanes > 0 ? lanes : 1;
 }
 
 // events6: null, or (start, stop) event pairs for the prefix, suffix and merge kernels of this call
@@ -311,8 +403,9 @@ static int decode_attention_impl(void* out, const void* q, const void* k_cache, 
                   plan->num_items > (int64_t)1 << 30))
     return PH_ERR_ARG;
   const bool paired = pair_heads(D, H) && prefix_mfma_supported(dtype, 128);
+  const bool roles = roles_possible(num_reqs, num_heads, head_dim, dtype, has_prefix, has_suffix, planned, chunk_tokens);
   const DecodePlan p = plan_decode(num_reqs, num_heads, has_prefix ? num_groups : 0, max_prefix_len, max_suffix_len,
-                                   chunk_tokens, planned ? plan->num_items : 0, head_dim, pair_heads(D, H));
+                                   chunk_tokens, planned ? plan->num_items : 0, head_dim, pair_heads(D, H), roles);
   if (plan_bytes(p, B, H, D) > workspace_bytes || ((p.parts() > 0 || p.items > 0) && !workspace))
     return PH_ERR_WORKSPACE;
   if (((uintptr_t)workspace & 255u) != 0) return PH_ERR_ALIGN;
@@ -359,8 +452,9 @@ static int decode_attention_impl(void* out, const void* q, const void* k_cache, 
     pa.B = B;
     pa.H = H;
     pa.scale_log2e = sl2;
-    fuse = planned && (paired ? decode_fused_supported(dtype, 128, 2 * max_group_reqs)
-                              : decode_fused_supported(dtype, D, max_group_reqs));
+    // roles for groups of any size; the shared form only where its eight-wave tile is at least half full
+    fuse = planned && (paired ? decode_fused_supported(dtype, 128) : decode_fused_supported(dtype, D)) &&
+           (p.prefix_wgs > 0 || (paired ? 2 : 1) * max_group_reqs > 32);
     if (fuse) {
       fused_pa = paired ? pair_args(pa, ws) : pa;
       fused_groups = (int)num_groups;
@@ -389,7 +483,8 @@ static int decode_attention_impl(void* out, const void* q, const void* k_cache, 
     ia.ml = ws.ml + item_base * 2;
     ia.H = H;
     ia.scale_log2e = sl2;
-    rc = fuse ? launch_decode_fused(fused_pa, ia, dtype, fused_groups, fused_max_reqs, device_cus(), st, ev_suffix)
+    rc = fuse ? launch_decode_fused(fused_pa, ia, dtype, fused_groups, fused_max_reqs, device_cus(), p.prefix_wgs, st,
+                                      ev_suffix)
               : launch_items(ia, dtype, D, st, ev_suffix);
     if (rc != PH_OK) return rc;
   } else if (has_suffix) {

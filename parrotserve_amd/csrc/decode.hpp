@@ -128,9 +128,11 @@ int launch_suffix_plan(const int32_t* lens, int B, int max_len, int lanes, int32
 int launch_prefix_mfma(const PrefixArgs& a, int dtype, int D, int num_groups, int max_group_reqs, hipStream_t st,
                        const KernelEvents& ev = KernelEvents());
 bool prefix_mfma_supported(int dtype, int D);
-// Prefix + suffix phases in one launch (see decode_fused_kernel); cus = compute units of the device.
-bool decode_fused_supported(int dtype, int D, int max_group_reqs);
+// Prefix + suffix phases in one launch (see decode_fused_kernel); cus = compute units of the device;
+// prefix_wgs > 0: that many workgroups run only prefix units and the others only suffix pieces, 0: every
+// workgroup runs both.
+bool decode_fused_supported(int dtype, int D);
 int launch_decode_fused(const PrefixArgs& a, const ItemArgs& ia, int dtype, int num_groups, int max_group_reqs, int cus,
-                        hipStream_t st, const KernelEvents& ev = KernelEvents());
+                        int prefix_wgs, hipStream_t st, const KernelEvents& ev = KernelEvents());
 
 }  // namespace ph

@@ -27,6 +27,7 @@
 //
 // Math restated from parrot/engine/builtin/kernels/shared_flash_decoding.py:34-134.
 #include "stream_item.hpp"
+#include <cstdlib>
 
 namespace ph {
 
@@ -97,6 +98,11 @@ struct TileWork {
   //   0 / 1: every row of the tile is that half, qrow0 points at the half's 64 values;
   //   2: rows alternate, row q = request q >> 1 (rows of q_stride from qrow0, the pair's first value), half q & 1
   int pair_half = -1;
+  // decode form: shares at most two steps longer than the ring touch the lines beyond it during their first two
+  // steps.  Off for the prefix-only workgroups of the fused launch: next to a suffix stream that saturates the
+  // memory system the touches (at any distance, at every step) made the steps slower, not faster (cold K/V:
+  // 70 us against 63 us per launch at config 2 with 64 prefix workgroups)
+  bool touch_ahead = true;
 };
 
 // Runs the tile on all four waves.  On return wave w holds, for the 32 dims [32w, 32w+32) of every
@@ -569,7 +575,8 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
                    : reinterpret_cast<const char*>(kc + (int64_t)head * kPD + ((c ^ ((4 * (r0 + i) + tl) & 15)) * 8));
   const uint32_t dst0 = lds_addr_of(gl) + sub0 * kStage + (isv ? kVtOff : 0) + r0 * 1024;
   const uint32_t pf_lds = lds_addr_of(smem + kPfOff) + w8 * 256;
-  const int pf_steps = (PREFETCH && (s1 - s0 + STEP * TQ - 1) / (STEP * TQ) <= NST + kPfSteps) ? kPfSteps : 0;
+  const int pf_steps =
+      (PREFETCH && wk.touch_ahead && (s1 - s0 + STEP * TQ - 1) / (STEP * TQ) <= NST + kPfSteps) ? kPfSteps : 0;
   // rows of the group's tile that starts at token tb, into ring stage `stage`
   auto fetch_rows = [&](int tb, int stage) {
     uint32_t sl[LPT];
@@ -888,7 +895,7 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
 // whole workgroup; writes one (O, m, l) part per request of the tile.
 template <typename E, int TQ, typename Mid = NoMid>
 __device__ __forceinline__ void prefix_unit8(const PrefixArgs& a, int split, int head, int z, int mtiles, char* smem,
-                                             Mid mid = Mid()) {
+                                             Mid mid = Mid(), bool touch_ahead = true) {
   constexpr int QB = 8 / TQ, QT = 32 * QB, NDB = 4 / TQ;  // query blocks, queries per tile, dim blocks per wave
   const int g = z / mtiles, mt = z - g * mtiles;
   int r0 = 0, r1 = a.B, poff = 0, plen = a.fixed_prefix_len;
@@ -926,6 +933,7 @@ __device__ __forceinline__ void prefix_unit8(const PrefixArgs& a, int split, int
   wk.s0 = s0;
   wk.s1 = s1;
   wk.causal_off = 0;
+  wk.touch_ahead = touch_ahead;
   float16_t of[NDB];
   float m, l;
   attn_tile8<E, false, TQ>(wk, a.kc, a.vc, a.row_stride, head, a.scale_log2e, smem, of, m, l, mid);
@@ -957,22 +965,49 @@ __global__ __launch_bounds__(512) void prefix_mfma8_kernel(PrefixArgs a, int mti
   prefix_unit8<E, TQ>(a, blockIdx.x, blockIdx.y, blockIdx.z, mtiles, smem);
 }
 
-// Prefix and suffix phases of one decode step in one launch.  Workgroup b owns the prefix units b,
-// b + grid, ... (normally at most one: the planner sizes the splits to the CU count) and its eight waves
-// one suffix piece each of the host-planned balanced form, (piece, head group) per wave.  Order inside a
-// workgroup: suffix records requested, prefix prologue (slot window, first K/V tiles sent on their way into
-// LDS, Q), then the suffix stream (it needs no LDS and runs at the same rate on two waves per SIMD as on
-// more), then the prefix main loop on tiles that landed long ago, then the fold.  Against two launches this
-// removes one launch, hides the prefix prologue behind the suffix stream and keeps the memory system busy
-// from the first microseconds.  The merge stays a separate launch: it needs every part.
+// Prefix and suffix phases of one decode step in one launch, in one of two forms.
+//
+// Roles (np > 0): workgroups [0, np) are prefix-only -- workgroup b walks the prefix units b, b + np, ... back to
+// back -- and workgroups [np, grid) are suffix-only: their eight waves take one (piece, head group) of the balanced
+// form each, the pieces cut for 8 (grid - np) waves.  Whole compute units belong to the matrix product for the
+// whole launch while the others stream, so neither phase waits for the other inside a workgroup and the memory
+// system sees both from the first microseconds to the last.  Consecutive workgroup ids land on different XCDs, so
+// both kinds spread evenly over the chip.
+//
+// Shared (np == 0): workgroup b owns the prefix units b, b + grid, ... (normally at most one) and its eight waves one
+// suffix piece each.  Order inside a workgroup: suffix records requested, prefix prologue (slot window, first K/V
+// tiles sent on their way into LDS, Q), then the suffix stream (it needs no LDS), then the prefix main loop on tiles
+// that landed long ago, then the fold.  Taken when the suffix is too short to keep separate workgroups busy.
+//
+// The merge stays a separate launch: it needs every part.
 // DS = head size of the suffix phase: 128, or 64 when the prefix phase runs on head pairs (pa.req_shift == 1).
 template <typename E, int TQ, int DS = kPD>
-__global__ __launch_bounds__(512) void decode_fused_kernel(PrefixArgs pa, int mtiles, int n_units, ItemArgs ia) {
+__global__ __launch_bounds__(512) void decode_fused_kernel(PrefixArgs pa, int mtiles, int n_units, int np,
+                                                           ItemArgs ia) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   PH_TL(0);
   constexpr int HPW = HeadLanes<DS>::HPW;
   const int hgroups = (ia.H + HPW - 1) / HPW;
   const int slots = ia.num_lanes * hgroups;
+  if (np > 0) {
+    if ((int)blockIdx.x < np) {
+      for (int u = blockIdx.x; u < n_units; u += np) {
+        if (u != (int)blockIdx.x) __syncthreads();  // the fold scratch of the last unit is the staging ring of the next
+        const int split = u % pa.n_splits;
+        const int rest = u / pa.n_splits;
+        prefix_unit8<E, TQ>(pa, split, rest % pa.H, rest / pa.H, mtiles, smem, NoMid(), false);
+      }
+    } else {
+      const int stride = ((int)gridDim.x - np) * 8;
+      const int wave = __builtin_amdgcn_readfirstlane(((int)blockIdx.x - np) * 8 + (int)(threadIdx.x >> 6));
+      for (int s = wave; s < slots; s += stride) {
+        const int piece = s / hgroups;
+        run_piece<E, DS, 4, 2>(ia, piece, s - piece * hgroups);
+      }
+    }
+    PH_TL(11);
+    return;
+  }
   const int wave = __builtin_amdgcn_readfirstlane(blockIdx.x * 8 + (threadIdx.x >> 6));
   // this wave's first suffix piece: its record is requested before anything else
   const int piece0 = wave < slots ? wave / hgroups : -1;
@@ -1132,47 +1167,54 @@ static int launch_prefill_t(const PrefillArgs& a, int64_t num_tokens, hipStream_
 
 template <typename E, int TQ, int DS>
 static int launch_fused_tq(const PrefixArgs& a, const ItemArgs& ia, int num_groups, int max_group_reqs, int cus,
-                           hipStream_t st, const KernelEvents& ev) {
+                           int np, hipStream_t st, const KernelEvents& ev) {
   constexpr int QT = 32 * (8 / TQ);
   constexpr int HPW = HeadLanes<DS>::HPW;
   const int mtiles = (max_group_reqs + QT - 1) / QT;
   const int n_units = a.n_splits * a.H * num_groups * mtiles;
   const int hgroups = (ia.H + HPW - 1) / HPW;
   const int wave_slots = ia.num_lanes * hgroups;
-  int grid = (wave_slots + 7) / 8;
-  const int unit_grid = n_units < cus ? n_units : cus;
-  if (grid < unit_grid) grid = unit_grid;
+  int grid;
+  if (np > 0) {
+    // roles: np prefix-only workgroups, then one round of suffix-only workgroups on the other compute units
+    if (np > n_units) np = n_units;
+    int swg = (wave_slots + 7) / 8;
+    const int room = cus - np > 1 ? cus - np : 1;
+    if (swg > room) swg = room;
+    grid = np + swg;
+  } else {
+    grid = (wave_slots + 7) / 8;
+    const int unit_grid = n_units < cus ? n_units : cus;
+    if (grid < unit_grid) grid = unit_grid;
+  }
   if (grid <= 0) return PH_OK;
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&decode_fused_kernel<E, TQ, DS>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, kTile8Lds);
   PH_LAUNCH_TIMED((decode_fused_kernel<E, TQ, DS>), dim3(grid), dim3(512), kTile8Lds, st, ev, a, mtiles,
-                        n_units, ia);
+                        n_units, np, ia);
   return launch_status();
 }
 
 // query tile by the largest group: 64, 128 or 256 requests share each K/V tile of the prefix
 template <typename E, int DS>
-static int launch_fused_t(const PrefixArgs& a, const ItemArgs& ia, int num_groups, int max_group_reqs, int cus,
+static int launch_fused_t(const PrefixArgs& a, const ItemArgs& ia, int num_groups, int max_group_reqs, int cus, int np,
                           hipStream_t st, const KernelEvents& ev) {
-  if (max_group_reqs <= 64) return launch_fused_tq<E, 4, DS>(a, ia, num_groups, max_group_reqs, cus, st, ev);
-  if (max_group_reqs <= 128) return launch_fused_tq<E, 2, DS>(a, ia, num_groups, max_group_reqs, cus, st, ev);
-  return launch_fused_tq<E, 1, DS>(a, ia, num_groups, max_group_reqs, cus, st, ev);
+  if (max_group_reqs <= 64) return launch_fused_tq<E, 4, DS>(a, ia, num_groups, max_group_reqs, cus, np, st, ev);
+  if (max_group_reqs <= 128) return launch_fused_tq<E, 2, DS>(a, ia, num_groups, max_group_reqs, cus, np, st, ev);
+  return launch_fused_tq<E, 1, DS>(a, ia, num_groups, max_group_reqs, cus, np, st, ev);
 }
 
-// One launch for the prefix and suffix phases: head size 128, groups of more than 32 requests (the
-// eight-wave prefix form), balanced suffix plan present.
-bool decode_fused_supported(int dtype, int D, int max_group_reqs) {
-  return D == kPD && (dtype == PH_F16 || dtype == PH_BF16) && max_group_reqs > 32;
-}
+// One launch for the prefix and suffix phases: head size 128 (the eight-wave prefix form), balanced suffix plan present.
+bool decode_fused_supported(int dtype, int D) { return D == kPD && (dtype == PH_F16 || dtype == PH_BF16); }
 
 int launch_decode_fused(const PrefixArgs& a, const ItemArgs& ia, int dtype, int num_groups, int max_group_reqs, int cus,
-                        hipStream_t st, const KernelEvents& ev) {
+                        int prefix_wgs, hipStream_t st, const KernelEvents& ev) {
   if (a.req_shift) {  // 64-wide heads: the prefix phase on head pairs, the suffix phase at its own width
-    return dtype == PH_F16 ? launch_fused_t<F16, 64>(a, ia, num_groups, max_group_reqs, cus, st, ev)
-                           : launch_fused_t<BF16, 64>(a, ia, num_groups, max_group_reqs, cus, st, ev);
+    return dtype == PH_F16 ? launch_fused_t<F16, 64>(a, ia, num_groups, max_group_reqs, cus, prefix_wgs, st, ev)
+                           : launch_fused_t<BF16, 64>(a, ia, num_groups, max_group_reqs, cus, prefix_wgs, st, ev);
   }
-  return dtype == PH_F16 ? launch_fused_t<F16, kPD>(a, ia, num_groups, max_group_reqs, cus, st, ev)
-                         : launch_fused_t<BF16, kPD>(a, ia, num_groups, max_group_reqs, cus, st, ev);
+  return dtype == PH_F16 ? launch_fused_t<F16, kPD>(a, ia, num_groups, max_group_reqs, cus, prefix_wgs, st, ev)
+                         : launch_fused_t<BF16, kPD>(a, ia, num_groups, max_group_reqs, cus, prefix_wgs, st, ev);
 }
 
 bool prefix_mfma_supported(int dtype, int D) { return D == kPD && (dtype == PH_F16 || dtype == PH_BF16); }

@@ -490,11 +490,11 @@ class DecodeTables:
     @staticmethod
     def build(prefix_lists: Sequence[Sequence[int]], group_req_cu: Sequence[int],
               suffix_lists: Sequence[Sequence[int]], device, num_heads: int = 32, head_dim: int = 128,
-              balanced: bool = True) -> "DecodeTables":
+              balanced: bool = True, dtype: torch.dtype = torch.float16) -> "DecodeTables":
         """From python lists: ``prefix_lists[g]`` is group g's slot list shared by
         requests ``group_req_cu[g] .. group_req_cu[g+1]-1``; ``suffix_lists[b]`` is
-        request b's own slot list.  ``balanced`` adds the host-planned item list of the
-        suffix phase, sized for ``num_heads x head_dim``."""
+        request b's own slot list.  ``balanced`` adds the item list of the
+        suffix phase, cut for ``num_heads x head_dim`` heads of ``dtype`` elements."""
         B = len(suffix_lists)
         t = DecodeTables(num_reqs=B)
         G = len(prefix_lists)
@@ -538,10 +538,12 @@ class DecodeTables:
                 chunk *= 2
             t.chunk_tokens = chunk
             if balanced:
+                shape = dict(num_reqs=B, num_groups=t.num_groups, max_prefix_len=t.max_prefix_len,
+                             max_suffix_len=t.max_suffix_len, dtype=dtype)
                 if B <= PLAN_MAX_REQS and t.suffix_offsets is None:
-                    t.plan_on_device(suffix_lane_capacity(device, num_heads, head_dim), device)
+                    t.plan_on_device(suffix_lane_capacity(device, num_heads, head_dim, **shape), device)
                 else:
-                    t.set_plan(lens, suffix_lanes(device, num_heads, head_dim, total), device)
+                    t.set_plan(lens, suffix_lanes(device, num_heads, head_dim, total, **shape), device)
         return t
 
 
@@ -594,22 +596,27 @@ def _heads_per_wave(head_dim: int) -> int:
     return max(1, 64 // lanes)
 
 
-def suffix_lane_capacity(device, num_heads: int, head_dim: int) -> int:
-    """Lanes of the device-built plan: one launch-wide round of waves at two waves per SIMD (see suffix_lanes)."""
-    heads_per_wave = _heads_per_wave(head_dim)
-    hgroups = (num_heads + heads_per_wave - 1) // heads_per_wave
-    return max(1, _cu_count(device) * 4 * 2 // hgroups)
+def suffix_lane_capacity(device, num_heads: int, head_dim: int, num_reqs: int = 0, num_groups: int = 0,
+                         max_prefix_len: int = 0, max_suffix_len: int = 0, dtype: torch.dtype = torch.float16) -> int:
+    """Lanes the balanced suffix plan should be cut into (``ph_decode_suffix_lanes``): one launch-wide round of waves
+    at two waves per SIMD on the compute units the suffix phase runs on -- all of them, or, for a batch whose
+    prefix and suffix phases get workgroups of their own inside one launch, the ones the prefix leaves."""
+    if num_reqs <= 0 or str(device) == "cpu" or not torch.cuda.is_available():
+        heads_per_wave = _heads_per_wave(head_dim)
+        hgroups = (num_heads + heads_per_wave - 1) // heads_per_wave
+        return max(1, _cu_count(device) * 4 * 2 // hgroups)
+    code = {torch.float16: _lib.PH_F16, torch.bfloat16: _lib.PH_BF16, torch.float32: _lib.PH_F32}[dtype]
+    with torch.cuda.device(device):
+        return int(_lib.load().ph_decode_suffix_lanes(num_reqs, num_heads, head_dim, code, num_groups, max_prefix_len,
+                                                      max_suffix_len))
 
 
-def suffix_lanes(device, num_heads: int, head_dim: int, total_tokens: int) -> int:
-    """Pieces of the balanced suffix phase: one launch-wide round of waves at two waves per SIMD (a piece is
-    streamed by one wave per `_heads_per_wave(head_dim)` heads; measured: one to three waves per SIMD stream at the same rate,
-    and fewer, longer pieces pay the start-up chain less often), and no piece under 4 tokens (one round of the
-    streaming body's register pipeline)."""
-    heads_per_wave = _heads_per_wave(head_dim)
-    hgroups = (num_heads + heads_per_wave - 1) // heads_per_wave
-    cus = _cu_count(device)
-    lanes = max(1, cus * 4 * 2 // hgroups)
+def suffix_lanes(device, num_heads: int, head_dim: int, total_tokens: int, **shape) -> int:
+    """Pieces of the host-planned balanced suffix phase: ``suffix_lane_capacity`` (a piece is streamed by one wave
+    per `_heads_per_wave(head_dim)` heads; measured: one to three waves per SIMD stream at the same rate, and fewer,
+    longer pieces pay the start-up chain less often), and no piece under 4 tokens (one round of the streaming body's
+    register pipeline)."""
+    lanes = suffix_lane_capacity(device, num_heads, head_dim, **shape)
     return max(1, min(lanes, (total_tokens + 3) // 4))
 
 

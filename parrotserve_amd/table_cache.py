@@ -41,6 +41,7 @@ class _Cached:
     flash_context_len: int
     num_heads: int
     head_dim: int
+    dtype: Any = torch.float16     # element type of the caches (the library's launch choice depends on it)
     slot_mapping: Any = None       # device int32 [B], job order: this iteration's new slots
 
 
@@ -91,16 +92,21 @@ class DecodeTableCache:
         c.slot_mapping = torch.from_numpy(np.asarray(new_slots, dtype=np.int32)).to(device)
         kernels.suffix_tables_append(t.suffix_slots, t.suffix_lens, c.rows, c.slot_mapping)
         t.max_suffix_len = need
+        shape = dict(num_reqs=t.num_reqs, num_groups=t.num_groups, max_prefix_len=t.max_prefix_len,
+                     max_suffix_len=need, dtype=c.dtype)
         if t.num_reqs <= kernels.PLAN_MAX_REQS:  # the cut points move with the lengths: a fresh plan, built on the device
-            t.plan_on_device(kernels.suffix_lane_capacity(device, c.num_heads, c.head_dim), device)
+            # (the lane count follows the library's launch choice for the batch's shape: it moves at a few thresholds
+            # of the growing lengths, and the plan's arrays are laid out anew when it does)
+            lanes = kernels.suffix_lane_capacity(device, c.num_heads, c.head_dim, **shape)
+            t.plan_on_device(lanes, device)
         else:
             total = int(c.lens_host.sum())
-            t.set_plan(c.lens_host, kernels.suffix_lanes(device, c.num_heads, c.head_dim, total), device)
+            t.set_plan(c.lens_host, kernels.suffix_lanes(device, c.num_heads, c.head_dim, total, **shape), device)
         self.hits += 1
         return c
 
     def store(self, jobs: Sequence[Any], order: List[int], suffix_lens: Sequence[int], tables, decode_perm,
-              flash_context_len: int, num_heads: int, head_dim: int, device) -> None:
+              flash_context_len: int, num_heads: int, head_dim: int, device, dtype=torch.float16) -> None:
         """Remember a batch that was just built from scratch.  ``order[r]`` = job whose suffix is table
         row r; ``suffix_lens`` in table-row order."""
         self.rebuilds += 1
@@ -118,7 +124,7 @@ class DecodeTableCache:
         self.state = _Cached(ctxs, parents, [len(c.token_kv_block_ids) for c in ctxs],
                              [p.get_context_len() if p is not None else 0 for p in parents], rows,
                              np.asarray(list(suffix_lens), dtype=np.int64), tables, decode_perm, flash_context_len,
-                             num_heads, head_dim)
+                             num_heads, head_dim, dtype)
 
 
 def _widen(t, need: int, device) -> None:

@@ -15,7 +15,8 @@ def _run_case(case, dev, chunk_tokens=None):
 
     kc, vc = synth.pool_to_device(case.k_rows, case.v_rows, case.used_slots, case.pool_slots, dev)
     tables = kernels.DecodeTables.build(case.pool_lists(case.prefix_lists), case.group_req_cu,
-                                        case.pool_lists(case.suffix_lists), dev)
+                                        case.pool_lists(case.suffix_lists), dev, num_heads=case.q.shape[1],
+                                        head_dim=case.q.shape[2], dtype=case.dtype)
     if chunk_tokens is not None:
         tables.chunk_tokens = chunk_tokens
     out = kernels.decode_attention(case.q.to(dev), kc, vc, tables)
@@ -83,6 +84,76 @@ def test_config5_full_size_attention(dev):
     pick = [0, 31, 32, 50, 64, 95, 100, 127]
     ref = ref_decode_attention(case.q[pick], case.k_rows, case.v_rows, [full[i] for i in pick])
     torch.testing.assert_close(out[pick].cpu().float(), ref.float(), **TOL[torch.float16])
+
+
+def _role_split(dev, case):
+    """(prefix-only workgroups, compute units) the library gives a batch of this shape, read off the lane count it
+    asks a plan to be cut into: lanes = 8 waves x (compute units - prefix workgroups) / head groups."""
+    from parrotserve_amd import kernels
+
+    B, H, D = case.q.shape
+    P = max(len(p) for p in case.prefix_lists)
+    S = max(len(x) for x in case.suffix_lists)
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    lanes = kernels.suffix_lane_capacity(dev, H, D, num_reqs=B, num_groups=len(case.prefix_lists), max_prefix_len=P,
+                                         max_suffix_len=S, dtype=case.dtype)
+    hgroups = (H + 3) // 4
+    return cus - (lanes * hgroups + 7) // 8, cus
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_prefix_and_suffix_workgroups_of_their_own(dev, dtype):
+    """A suffix-heavy batch (config 2's proportions at a quarter of its heads): the library gives the prefix phase
+    workgroups of its own inside the one launch, the plan is cut for the rest, and the result equals the oracle --
+    also with a plan cut for the whole device (more pieces than suffix waves: further rounds) and for a handful of
+    lanes (fewer pieces than suffix workgroups)."""
+    from parrotserve_amd import kernels, synth
+
+    g = torch.Generator().manual_seed(21)
+    s = torch.randint(300, 1100, (64,), generator=g).tolist()
+    case = synth.make_decode_case("roles", 21, dtype, 1, 64, 2048, s, 8, 128, 1 << 17)
+    np_, cus = _role_split(dev, case)
+    assert 0 < np_ < cus, "this shape is meant to take the two-role launch"
+    out = _check(case, dev)
+    kc, vc = synth.pool_to_device(case.k_rows, case.v_rows, case.used_slots, case.pool_slots, dev)
+    for lanes in (kernels.suffix_lane_capacity(dev, 8, 128), 5):
+        tables = kernels.DecodeTables.build(case.pool_lists(case.prefix_lists), case.group_req_cu,
+                                            case.pool_lists(case.suffix_lists), dev, num_heads=8, head_dim=128,
+                                            dtype=dtype)
+        tables.plan_on_device(lanes, dev)
+        other = kernels.decode_attention(case.q.to(dev), kc, vc, tables).cpu()
+        torch.testing.assert_close(other.float(), out.float(), **TOL[dtype])
+
+
+def test_prefix_workgroups_walk_several_units_each(dev):
+    """Eight groups x 32 heads are 256 prefix units per split -- more than the prefix-only workgroups of a device
+    with that many compute units or fewer -- so every prefix workgroup walks several units back to back (the fold
+    scratch of one is the staging ring of the next).  Groups of eight requests: the 64-query tile mostly empty."""
+    from parrotserve_amd import synth
+
+    g = torch.Generator().manual_seed(22)
+    s = torch.randint(120, 400, (64,), generator=g).tolist()
+    case = synth.make_decode_case("units", 22, torch.float16, 8, 8, 520, s, 32, 128, 1 << 16)
+    np_, cus = _role_split(dev, case)
+    assert 0 < np_ < 8 * 32, "prefix workgroups must be fewer than the prefix units"
+    _check(case, dev)
+
+
+def test_two_role_launch_with_empty_suffixes(dev):
+    """Requests whose own list is empty inside a batch that takes the two-role launch (their output is the prefix
+    part alone), and, with every list empty, the prefix phase on its own."""
+    from parrotserve_amd import synth
+
+    g = torch.Generator().manual_seed(23)
+    s = torch.randint(500, 1200, (48,), generator=g).tolist()
+    for b in (0, 7, 8, 30, 47):
+        s[b] = 0
+    case = synth.make_decode_case("empty", 23, torch.float16, 1, 48, 1500, s, 8, 128, 1 << 17)
+    np_, cus = _role_split(dev, case)
+    assert 0 < np_ < cus
+    _check(case, dev)
+    none = synth.make_decode_case("none", 24, torch.float16, 1, 48, 1500, [0] * 48, 8, 128, 1 << 17)
+    _check(none, dev)
 
 
 def test_multi_group_prefixes(dev):
