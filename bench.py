@@ -292,6 +292,8 @@ def extras(torch, dev):
     out["c5_layer"] = config5_layer(torch, dev)
     out["c2_iteration_tables"] = iteration_tables_cost(torch, dev)
     out["prefix_length_sweep"] = prefix_length_sweep(torch, dev)
+    out["prefix_regimes"] = prefix_regimes(torch, dev)
+    out["bench_kernel_shape"] = bench_kernel_shape(torch, dev)
     out["e2e_decode_13b"] = e2e_decode(torch, dev)
     out["e2e_decode_13b_fused_ops"] = e2e_decode(torch, dev, fused_ops=True)
     # --- RMSNorm at a bandwidth-sized row count (LLaMA-13B hidden) -----------------------------------------
@@ -500,6 +502,101 @@ def prefix_length_sweep(torch, dev):
     return res
 
 
+def _event_time_us(torch, ev, call, which, launches=24, warm=4):
+    """Median dispatch time (start / stop events attached to the launch) of kernel `which` (0 prefix, 1 suffix or
+    fused, 2 merge) of `call(i, events6)` over `launches` calls."""
+    for i in range(warm):
+        call(i, None)
+    sets = [ev.create(6) for _ in range(launches)]
+    for i, s6 in enumerate(sets):
+        call(i, s6)
+    torch.cuda.synchronize()
+    ts = [ev.elapsed_ms(s6[2 * which], s6[2 * which + 1]) for s6 in sets]
+    for s6 in sets:
+        ev.destroy(s6)
+    if any(t is None for t in ts):
+        return None
+    return sorted(ts)[len(ts) // 2] * 1e3
+
+
+def prefix_regimes(torch, dev):
+    """The prefix phase (matrix-core kernel alone: empty suffixes) from the bandwidth-bound to the matrix-bound regime:
+    one group of B requests over a P-token prefix, 32 x 128 fp16.  The contraction has B FLOP per K/V byte, so its
+    ceiling is min(matrix peak, B x HBM peak); cold = the launches rotate over K/V sets that do not fit the
+    memory-side cache together, warm = one set re-read."""
+    from parrotserve_amd import kernels
+
+    ev = HipEvents()
+    H, D, pool = 32, 128, 1 << 16
+    g = torch.Generator(device=dev).manual_seed(11)
+    kc = torch.randn((pool, H, D), generator=g, device=dev, dtype=torch.float16)
+    vc = torch.randn((pool, H, D), generator=g, device=dev, dtype=torch.float16)
+    perm = torch.randperm(pool, generator=torch.Generator().manual_seed(11))
+    res = {"heads": H, "head_dim": D, "dtype": "f16", "points": []}
+    for P in (4096, 8192):
+        nsets = pool // P
+        for B in (64, 128, 256, 512, 1024):
+            q = torch.randn((B, H, D), generator=g, device=dev, dtype=torch.float16)
+            o = torch.empty_like(q)
+            tabs = [kernels.DecodeTables.build([perm[i * P:(i + 1) * P].tolist()], [0, B], [[] for _ in range(B)], dev,
+                                               num_heads=H, head_dim=D) for i in range(nsets)]
+            flops = 4 * B * H * P * D
+            kv = 2 * P * H * D * 2
+            bound = min(MFMA_F16_PEAK_TFLOPS, B * HBM_PEAK_GBS / 1e3)
+            pt = {"batch": B, "prefix_len": P, "flops": flops, "kv_bytes": kv, "bound_tflops": bound}
+            for label, pick in (("cold", lambda i: tabs[i % nsets]), ("warm", lambda i: tabs[0])):
+                t = _event_time_us(torch, ev, lambda i, e6: kernels.decode_attention(q, kc, vc, pick(i), out=o,
+                                                                                     events6=e6), 0)
+                if t is None:
+                    continue
+                tf = flops / t / 1e6
+                pt[label] = {"us": t, "tflops": tf, "frac_mfma_peak": tf / MFMA_F16_PEAK_TFLOPS,
+                             "frac_of_min_mfma_hbm_bound": tf / bound, "kv_GB/s": kv / t / 1e3}
+            res["points"].append(pt)
+            del tabs
+    return res
+
+
+def bench_kernel_shape(torch, dev):
+    """The one shape the reference's own kernel benchmark runs (benchmark/bench_kernel.py:11-83): batch 64 sharing an
+    8192-token prefix, 40 x 128 heads, ten to twenty diverged tokens per request.  The launch that runs the prefix and
+    suffix phases against the HBM roofline (K/V of the prefix once, of every suffix once), and the merge beside it."""
+    from parrotserve_amd import kernels, synth
+
+    ev = HipEvents()
+    B, P, H, D = 64, 8192, 40, 128
+    g = torch.Generator().manual_seed(1)
+    lens = torch.randint(10, 21, (B,), generator=g).tolist()
+    nsets = 4
+    case = synth.make_decode_case("bk", 1, torch.float16, 1, B, P, lens, H, D, 1 << 16)
+    n_used = case.k_rows.shape[0]
+    kc, vc = synth.pool_to_device(case.k_rows, case.v_rows, case.used_slots, case.pool_slots, dev)
+    perm = torch.randperm(case.pool_slots, generator=torch.Generator().manual_seed(2))
+    dgen = torch.Generator(device=dev).manual_seed(2)
+    tabs = []
+    for i in range(nsets):  # K/V sets at other slots of the pool, device-generated rows
+        used = perm[i * n_used:(i + 1) * n_used]
+        idx = used.to(dev)
+        kc[idx] = torch.randn((n_used, H, D), generator=dgen, device=dev, dtype=torch.float16)
+        vc[idx] = torch.randn((n_used, H, D), generator=dgen, device=dev, dtype=torch.float16)
+        tabs.append(kernels.DecodeTables.build([used[p].tolist() for p in case.prefix_lists], case.group_req_cu,
+                                               [used[x].tolist() for x in case.suffix_lists], dev, num_heads=H,
+                                               head_dim=D))
+    q = case.q.to(dev)
+    o = torch.empty_like(q)
+    call = lambda i, e6: kernels.decode_attention(q, kc, vc, tabs[i % nsets], out=o, events6=e6)
+    t_k = _event_time_us(torch, ev, call, 1)
+    t_m = _event_time_us(torch, ev, call, 2)
+    t_step = _time_gpu(torch, lambda: call(0, None), iters=10)
+    nbytes = 2 * (P + sum(lens)) * H * D * 2
+    return {"batch": B, "prefix_len": P, "heads": H, "sum_suffix_len": sum(lens), "kv_sets": nsets,
+            "step_us_one_set": t_step * 1e6, "merge_us": t_m,
+            "roofline": {"kernel": "decode_fused_kernel (prefix + suffix phases)", "bound": "hbm",
+                         "algorithmic_bytes": nbytes, "avg_launch_us": t_k,
+                         "achieved": None if t_k is None else nbytes / t_k / 1e3, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": None if t_k is None else nbytes / t_k / 1e3 / HBM_PEAK_GBS}}
+
+
 def iteration_tables_cost(torch, dev):
     """Host time per decode iteration of producing the device index tables (slot tables, lengths, suffix plan)
     for config 2's batch, 64 Generate jobs forked from one 4096-token parent, own contexts U[16,512]: rebuilt
@@ -670,6 +767,9 @@ def main():
     ap.add_argument("--timeline", action="store_true",
                     help="only record where the waves of the fused decode kernel spend their time (needs the "
                          "profiling variant of the library, built beside the product one) and exit")
+    ap.add_argument("--prefix-regimes-only", action="store_true",
+                    help="only run the prefix phase over batch sizes from the bandwidth-bound to the matrix-bound "
+                         "regime, and the reference benchmark's shape, and exit")
     ap.add_argument("--prefill-only", action="store_true",
                     help="only run config 4's prefill kernel a few times (for profiler counter passes) and exit")
     args = ap.parse_args()
@@ -695,6 +795,11 @@ def main():
         return
     if args.e2e_only:
         print(json.dumps({"e2e_decode_13b_fused_ops": e2e_decode(torch, dev, fused_ops=True)}))
+        return
+
+    if args.prefix_regimes_only:
+        print(json.dumps({"prefix_regimes": prefix_regimes(torch, dev),
+                          "bench_kernel_shape": bench_kernel_shape(torch, dev)}))
         return
 
     if args.prefill_only:

@@ -82,6 +82,8 @@ def load() -> ctypes.CDLL:
     if hasattr(lib, "ph_timeline_read"):  # profiling variant of the library (build.TIMELINE_LIB_PATH)
         lib.ph_timeline_read.restype = c_int
         lib.ph_timeline_read.argtypes = [c_void_p, c_size_t]
+        lib.ph_timeline_read_clocks.restype = c_int
+        lib.ph_timeline_read_clocks.argtypes = [c_void_p, c_size_t]
         lib.ph_timeline_clear.restype = c_int
         lib.ph_timeline_clear.argtypes = []
     _lib = lib

@@ -268,11 +268,12 @@ static PrefixArgs pair_args(const PrefixArgs& pa, const Carve& ws) {
 }
 
 static int run_prefix(PrefixArgs& pa, int dtype, int D, int num_groups, const int32_t* group_req_cu_host,
-                      int max_group_reqs, hipStream_t st, const Carve* pairs = nullptr,
+                      int max_group_reqs, bool internal_ml, hipStream_t st, const Carve* pairs = nullptr,
                       const KernelEvents& ev = KernelEvents()) {
   if (pairs && pairs->opart_pairs)
-    return launch_prefix_mfma(pair_args(pa, *pairs), dtype, 128, num_groups, 2 * max_group_reqs, st, ev);
-  if (prefix_mfma_supported(dtype, D)) return launch_prefix_mfma(pa, dtype, D, num_groups, max_group_reqs, st, ev);
+    return launch_prefix_mfma(pair_args(pa, *pairs), dtype, 128, num_groups, 2 * max_group_reqs, internal_ml, st, ev);
+  if (prefix_mfma_supported(dtype, D))
+    return launch_prefix_mfma(pa, dtype, D, num_groups, max_group_reqs, internal_ml, st, ev);
   int rc = launch_clear_ml(pa.ml, (int64_t)pa.n_splits * pa.B * pa.H, st);
   if (rc != PH_OK) return rc;
   for (int g = 0; g < num_groups; ++g) {
@@ -460,8 +461,8 @@ static int decode_attention_impl(void* out, const void* q, const void* k_cache, 
       fused_groups = (int)num_groups;
       fused_max_reqs = paired ? 2 * max_group_reqs : max_group_reqs;
     } else {
-      rc = run_prefix(pa, dtype, D, (int)num_groups, group_req_cu_host, max_group_reqs, st, paired ? &ws : nullptr,
-                      ev_prefix);
+      rc = run_prefix(pa, dtype, D, (int)num_groups, group_req_cu_host, max_group_reqs, true, st,
+                      paired ? &ws : nullptr, ev_prefix);
       if (rc != PH_OK) return rc;
     }
   }
@@ -635,7 +636,7 @@ static int prefix_phase(void* out, const float* prev_m, const float* prev_l, flo
     pa.B = B;
     pa.H = H;
     pa.scale_log2e = scale * kLog2e;
-    rc = run_prefix(pa, dtype, D, 1, nullptr, B, st, paired ? &ws : nullptr);
+    rc = run_prefix(pa, dtype, D, 1, nullptr, B, m_out == nullptr, st, paired ? &ws : nullptr);
     if (rc != PH_OK) return rc;
   }
   MergeArgs ma{};

@@ -124,9 +124,10 @@ constexpr int kPlanMaxReqs = 8192;
 // lengths are clamped to [0, max_len]
 int launch_suffix_plan(const int32_t* lens, int B, int max_len, int lanes, int32_t* items, int32_t* lane_rec,
                        int32_t* req_item_cu, hipStream_t st);
-// MFMA shared-prefix kernel: grid (split, head, group x m-tile).
-int launch_prefix_mfma(const PrefixArgs& a, int dtype, int D, int num_groups, int max_group_reqs, hipStream_t st,
-                       const KernelEvents& ev = KernelEvents());
+// MFMA shared-prefix kernel: grid (split, head, group x m-tile).  internal_ml: the parts' (m, l) only feed the
+// call's own merge (not exported to the caller), which frees the kernel to pre-scale and re-round the query.
+int launch_prefix_mfma(const PrefixArgs& a, int dtype, int D, int num_groups, int max_group_reqs, bool internal_ml,
+                       hipStream_t st, const KernelEvents& ev = KernelEvents());
 bool prefix_mfma_supported(int dtype, int D);
 // Prefix + suffix phases in one launch (see decode_fused_kernel); cus = compute units of the device;
 // prefix_wgs > 0: that many workgroups run only prefix units and the others only suffix pieces, 0: every
