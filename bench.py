@@ -28,8 +28,9 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16
 
 # HBM traffic per launch of this workload's kernels and the matrix-pipe counters of the prefix kernel come from
-# rocprofv3 --pmc passes over this file; their summary (python -m parrotserve_amd.profile_summary) is kept in
-# profiles/counters.json together with the commit it was taken at, and is read from there -- nothing is typed in.
+# rocprofv3 --pmc passes over this file (the commands stand at the top of each profiles/*.txt); their figures are
+# kept in profiles/counters.json together with the commit they were taken at, and are read from there -- nothing
+# is typed in.
 COUNTERS_JSON = os.path.join(ROOT, "profiles", "counters.json")
 
 

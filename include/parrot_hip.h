@@ -182,11 +182,21 @@ int ph_rotary_embedding(void* state, const void* cos, const void* sin,
  *                 paged_block_tables [B, max]).
  *   suffix_slots_count: number of int32 entries readable behind suffix_slots
  *                 (the kernel prefetches slot ids before it knows a list's
- *                 length and clamps those reads to this bound);
+ *                 length and clamps those reads to this bound).  A padded
+ *                 table must hold max_suffix_len entries in every row:
+ *                 suffix_slots_count >= (B - 1) * suffix_table_stride +
+ *                 max_suffix_len, else PH_ERR_ARG;
  *   suffix_lens:  int32 [B] (DEVICE); max_suffix_len: host upper bound -- the
- *                 kernels read a length as min(max(len, 0), max_suffix_len),
- *                 so a bad entry cannot walk into another request's slots
- *                 (for a padded table pass at most its width).
+ *                 kernels read a length as min(max(len, 0), max_suffix_len)
+ *                 (and no further than the table's end), so a bad entry
+ *                 cannot walk into another request's slots (for a padded
+ *                 table pass at most its width).  This is a clamp, not only a
+ *                 sizing hint: tokens beyond max_suffix_len are not attended
+ *                 to.  A call captured into a graph and replayed while the
+ *                 lists grow must therefore be captured with the largest
+ *                 length a replay will see (the table's width, say) -- also
+ *                 when the library builds the plan itself, whose arguments
+ *                 are recorded with the call.
  * chunk_tokens: suffix split size of the plain (request, chunk) grid form
  *   (multiple of 16); 0 = leave the decomposition to the library.
  * plan (HOST struct of DEVICE pointers, may be NULL): a caller that knows the
@@ -274,7 +284,9 @@ int ph_decode_attention(void* out, const void* q, const void* k_cache, const voi
  * needs 13.9 MB; config 5, 128 x 40 x 128 in four groups, 15 MB).  All calls on
  * one device share the array: calls that overlap on one device (two streams,
  * two threads) race on it -- serialise them, or use ph_decode_attention with a
- * workspace per stream. */
+ * workspace per stream.  The first call on a device asks the runtime for the
+ * array's address (hipGetSymbolAddress, once per device): make that call
+ * outside stream capture; later calls only launch kernels. */
 size_t ph_decode_static_scratch_bytes(void);
 
 int ph_decode_attention_static(void* out, const void* q, const void* k_cache, const void* v_cache,

@@ -38,36 +38,32 @@ ATTN_FUNCS = [
 # host-side index tables (pure python, no device)
 # --------------------------------------------------------------------------- #
 def _lca(context1, context2):
-    """Lowest common ancestor of two context nodes, ``None`` if the trees differ
-    (attn_func.py:412-439)."""
-    if context1 is context2:
-        return context1
-    if context1 is None or context2 is None:
+    """Lowest common ancestor of two context nodes, ``None`` if they sit in different trees (what
+    attn_func.py:412-439 computes).  The deeper node is lifted to the other's depth, then both climb together."""
+    a, b = context1, context2
+    if a is None or b is None:
         return None
-    while context1 is not None:
-        if context1 is context2:
-            return context1
-        if context1.depth > context2.depth:
-            context1 = context1.parent_context
-        elif context1.depth < context2.depth:
-            context2 = context2.parent_context
-        else:
-            context1 = context1.parent_context
-            context2 = context2.parent_context
-    return None
+    if a.depth < b.depth:
+        a, b = b, a
+    for _ in range(a.depth - b.depth):
+        a = a.parent_context
+    while a is not b:
+        if a is None or b is None:
+            return None
+        a, b = a.parent_context, b.parent_context
+    return a
 
 
 def get_shared_context_len(jobs: Sequence[Any]) -> int:
-    """Length of the context shared by ALL jobs (attn_func.py:441-459)."""
+    """Tokens of context shared by ALL jobs: the context length of the lowest common ancestor of every job's
+    context, 0 when there is none (attn_func.py:441-459)."""
     assert len(jobs) > 0
-    if len(jobs) == 1:
-        return jobs[0].context.get_context_len()
-    lca = _lca(jobs[0].context, jobs[1].context)
-    for job in jobs[2:]:
-        if lca is None:
-            break
-        lca = _lca(lca, job.context)
-    return lca.get_context_len() if lca is not None else 0
+    common = jobs[0].context
+    for job in jobs[1:]:
+        common = _lca(common, job.context)
+        if common is None:
+            return 0
+    return common.get_context_len()
 
 
 @dataclasses.dataclass

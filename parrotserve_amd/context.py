@@ -19,34 +19,47 @@ class ParrotError(Exception):
 
 
 class RecyclePool:
+    """Ids 0, 1, 2, ... with recycling.  The pool's state is the recycled ids -- a queue in the order they came
+    back and a set for membership -- plus the number of fresh ids issued so far; everything else is derived or
+    bookkeeping.  Behaviour kept from the reference because callers and tests can see it: recycled ids go out
+    oldest first and before any fresh id (unless ``debug_mode``, which only ever issues fresh ones); a bounded
+    pool never issues its last id (``pool_size - 1``); the allocation count moves before the failure checks (an
+    exhausted ``allocate`` and a double ``free`` both leave it changed); the high-water mark is only sampled when a
+    recycled id goes out."""
+
     def __init__(self, pool_name: str = "pool", pool_size: Optional[int] = None, debug_mode: bool = False) -> None:
         self.pool_name = pool_name
         self.pool_size = pool_size
-        self.allocated_num = 0
-        self.cur_max_id = 0
-        self.free_ids: Deque[int] = deque()
-        self._free_set = set()  # O(1) double-free check; free_ids keeps the FIFO order
-        self.history_max = 0
         self.debug_mode = debug_mode
+        self.free_ids: Deque[int] = deque()   # recycled ids, oldest first
+        self._recycled = set()                # the same ids, for the double-free check
+        self.cur_max_id = 0                   # fresh ids issued so far (the next fresh id)
+        self.allocated_num = 0
+        self.history_max = 0
+
+    def _fresh(self) -> int:
+        issued = self.cur_max_id
+        self.cur_max_id = issued + 1
+        if self.pool_size is not None and issued + 1 >= self.pool_size:
+            raise ParrotError(f"No free ids in Pool: {self.pool_name} (pool_size={self.pool_size}).")
+        return issued
 
     def allocate(self) -> int:
         self.allocated_num += 1
-        if not self.free_ids or self.debug_mode:
-            self.cur_max_id += 1
-            if self.pool_size is not None and self.cur_max_id >= self.pool_size:
-                raise ParrotError(f"No free ids in Pool: {self.pool_name} (pool_size={self.pool_size}).")
-            return self.cur_max_id - 1
-        allocated_id = self.free_ids.popleft()
-        self._free_set.discard(allocated_id)
-        self.history_max = max(self.history_max, self.get_allocated_num())
-        return allocated_id
+        if self.debug_mode or not self.free_ids:
+            return self._fresh()
+        reused = self.free_ids.popleft()
+        self._recycled.remove(reused)
+        if self.allocated_num > self.history_max:
+            self.history_max = self.allocated_num
+        return reused
 
     def free(self, id: int) -> None:
         self.allocated_num -= 1
-        if id in self._free_set:
+        if id in self._recycled:
             raise ValueError("The id is already free.")
+        self._recycled.add(id)
         self.free_ids.append(id)
-        self._free_set.add(id)
 
     def get_allocated_num(self) -> int:
         return self.allocated_num

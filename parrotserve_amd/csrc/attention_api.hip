@@ -399,6 +399,11 @@ static int decode_attention_impl(void* out, const void* q, const void* k_cache, 
   const bool has_suffix = max_suffix_len > 0;
   if (has_prefix && (!prefix_slots || !prefix_cu || !group_req_cu || !group_req_cu_host)) return PH_ERR_ARG;
   if (has_suffix && (!suffix_slots || !suffix_lens || suffix_slots_count <= 0)) return PH_ERR_ARG;
+  // padded table: every row must hold max_suffix_len entries inside the table (the balanced form walks a row up to
+  // its clamped length without knowing where the table ends)
+  if (has_suffix && !suffix_offsets &&
+      (suffix_table_stride < 0 || suffix_slots_count < (num_reqs - 1) * suffix_table_stride + max_suffix_len))
+    return PH_ERR_ARG;
   bool planned = has_suffix && plan != nullptr && plan->num_items > 0;
   if (planned && (!plan->items || !plan->lane_rec || !plan->req_item_cu || plan->num_lanes <= 0 ||
                   plan->num_items > (int64_t)1 << 30))
@@ -531,6 +536,9 @@ static int decode_attention_impl(void* out, const void* q, const void* k_cache, 
   ma.baseB = p.n_splits;
   ma.lens = has_suffix ? suffix_lens : nullptr;
   ma.max_len = (int)max_suffix_len;
+  ma.offsets = suffix_offsets;
+  ma.table_stride = suffix_table_stride;
+  ma.slots_total = suffix_slots_count;
   ma.chunk = p.chunk;
   ma.req_item_cu = planned ? plan->req_item_cu : nullptr;
   ma.item_base = item_base;
@@ -700,6 +708,11 @@ static int suffix_phase(void* out, const float* prev_m, const float* prev_l, flo
   if (max_suffix_len < 0 || max_suffix_len > INT32_MAX) return PH_ERR_ARG;
   const bool has_suffix = max_suffix_len > 0;
   if (has_suffix && (!suffix_slots || !suffix_lens || suffix_slots_count <= 0)) return PH_ERR_ARG;
+  // padded table: every row must hold max_suffix_len entries inside the table (the balanced form walks a row up to
+  // its clamped length without knowing where the table ends)
+  if (has_suffix && !suffix_offsets &&
+      (suffix_table_stride < 0 || suffix_slots_count < (num_reqs - 1) * suffix_table_stride + max_suffix_len))
+    return PH_ERR_ARG;
   const DecodePlan p = plan_decode(num_reqs, num_heads, 0, 0, max_suffix_len, chunk_tokens, 0, head_dim);
   if (plan_bytes(p, B, H, D) > workspace_bytes || ((p.parts() > 0 || p.items > 0) && !workspace))
     return PH_ERR_WORKSPACE;
@@ -766,6 +779,9 @@ static int suffix_phase(void* out, const float* prev_m, const float* prev_l, flo
   ma.baseB = 0;
   ma.lens = has_suffix ? suffix_lens : nullptr;
   ma.max_len = (int)max_suffix_len;
+  ma.offsets = suffix_offsets;
+  ma.table_stride = suffix_table_stride;
+  ma.slots_total = suffix_slots_count;
   ma.chunk = p.chunk;
   ma.req_item_cu = has_suffix && p.dev_lanes > 0 ? ws.req_item_cu : nullptr;
   ma.item_base = 0;
@@ -895,6 +911,8 @@ extern "C" int ph_prefill_attention(void* out, const void* q, const void* k_cach
   ma.baseB = 0;
   ma.lens = lens;
   ma.max_len = (int)max_kv_len;
+  ma.offsets = offsets;
+  ma.slots_total = ctx_slots_count;
   ma.chunk = p.chunk;
   return launch_merge(ma, dtype, D, st);
 }

@@ -56,7 +56,7 @@ __global__ __launch_bounds__(256) void decode_partial_kernel(PartialArgs a) {
   const int32_t* slots = a.slots + off;
   const int myslot = slots[min((int64_t)(t0 + lane), last)];
   // a length beyond the host's bound (or the table's end) would walk into other requests' slots
-  if (len < 0) len = (int)min((int64_t)min(max(a.lens[b], 0), a.max_len), last + 1);
+  if (len < 0) len = clamped_list_len(a.lens, b, a.max_len, off, a.slots_total);
 
   const int head = hg * HPW + lane / LPH;
   const bool head_ok = head < a.H;
@@ -124,7 +124,12 @@ __global__ __launch_bounds__(256) void merge_kernel(MergeArgs a) {
     it0 = a.req_item_cu[b];
     nB = a.req_item_cu[b + 1] - it0;
   } else {
-    nB = a.lens ? (min(max(a.lens[b], 0), a.max_len) + a.chunk - 1) / a.chunk : 0;
+    int len = 0;
+    if (a.lens && a.slots_total > 0)
+      len = clamped_list_len(a.lens, b, a.max_len, a.offsets ? a.offsets[b] : (int64_t)b * a.table_stride, a.slots_total);
+    else if (a.lens)
+      len = min(max(a.lens[b], 0), a.max_len);
+    nB = (len + a.chunk - 1) / a.chunk;
   }
   const int total = a.nA + nB;
 #pragma unroll 2

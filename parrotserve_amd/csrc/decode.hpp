@@ -65,7 +65,10 @@ struct MergeArgs {
   int nA;                   // parts [0, nA) are candidates for every request
   int baseB;                // parts [baseB, baseB + ceil(lens[b]/chunk)) likewise
   const int32_t* lens;      // may be null (no B range)
-  int max_len;              // lengths read from `lens` are clamped to [0, max_len]
+  int max_len;              // lengths read from `lens` are clamped to [0, max_len] ...
+  const int64_t* offsets;   // ... and, when slots_total > 0, to the entries behind the request's list start
+  int64_t table_stride;     //     (offsets[b], or b * table_stride): the clamp of the kernel that wrote the parts
+  int64_t slots_total;
   int chunk;
   const int32_t* req_item_cu; // balanced form: request b owns items [cu[b], cu[b+1]) ...
   int64_t item_base;          // ... whose partial rows start at item_base (rows of H)
@@ -74,6 +77,16 @@ struct MergeArgs {
   float* m_out;             // optional export of the merged m / l
   float* l_out;
 };
+
+// Length of request b's slot list as every kernel reads it: the device value clamped to [0, max_len] and to the
+// entries the table holds behind the list's start (a corrupt length then reads a wrong token of the same table
+// instead of unmapped memory, and the kernels that write parts and the one that merges them agree on the count).
+__device__ __forceinline__ int clamped_list_len(const int32_t* lens, int b, int max_len, int64_t off,
+                                                int64_t slots_total) {
+  const int64_t len = min(max(lens[b], 0), max_len);
+  const int64_t room = slots_total - off;
+  return (int)max((int64_t)0, min(len, room));
+}
 
 struct PrefixArgs {
   const uint16_t* q;

@@ -1059,17 +1059,13 @@ __global__ __launch_bounds__(512) void decode_fused_kernel(PrefixArgs pa, int mt
 // Prefill with parent context, eight waves: workgroup = (head, tile of 32 * (8 / TQ) queries of one chunk)
 // HALF (64-wide heads, 256-query tiles): only this head's half of the pair's output is computed
 template <typename E, int TQ, int SUB, bool HALF = false>
-__global__ __launch_bounds__(512) void prefill_mfma8_kernel(PrefillArgs a) {
+__device__ __forceinline__ void prefill_tile8(const PrefillArgs& a, int tile_row, char* smem) {
   constexpr int QB = 8 / TQ, NDB = 4 / TQ, QT = 32 * QB;
-  extern __shared__ __attribute__((aligned(16))) char smem[];
-  PH_TL(0);
-  if ((int)blockIdx.x >= a.H) return;
   // 64-wide heads: workgroup x is head x = half (x & 1) of pair x >> 1, whose K/V rows are one 128-wide row
   const int head = a.pair ? blockIdx.x >> 1 : blockIdx.x;
   const int half = a.pair ? (int)(blockIdx.x & 1) : -1;
-  if ((int)blockIdx.y >= a.tile_cu[a.num_chunks]) return;
   // later tiles of a chunk see more keys: hand them out first so the launch does not end on the longest ones
-  const int ti = a.tile_cu[a.num_chunks] - 1 - blockIdx.y;
+  const int ti = a.tile_cu[a.num_chunks] - 1 - tile_row;
   int lo = 0, hi = a.num_chunks;  // chunk with tile_cu[c] <= ti < tile_cu[c+1]
   while (hi - lo > 1) {
     const int mid = (lo + hi) >> 1;
@@ -1112,6 +1108,21 @@ __global__ __launch_bounds__(512) void prefill_mfma8_kernel(PrefillArgs a) {
         *reinterpret_cast<u32x2*>(op + 8 * j) = v;
       }
     }
+  }
+}
+
+// Prefill with parent context, eight waves: workgroup = (head, tile of 32 * (8 / TQ) queries of one chunk); grid.y
+// covers the tile rows, striding over them when there are more than the grid's y extent holds
+// HALF (64-wide heads, 256-query tiles): only this head's half of the pair's output is computed
+template <typename E, int TQ, int SUB, bool HALF = false>
+__global__ __launch_bounds__(512) void prefill_mfma8_kernel(PrefillArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  PH_TL(0);
+  if ((int)blockIdx.x >= a.H) return;
+  const int tiles = a.tile_cu[a.num_chunks];
+  for (int row = blockIdx.y; row < tiles; row += gridDim.y) {
+    if (row != (int)blockIdx.y) __syncthreads();  // the last tile's fold scratch is the next tile's staging ring
+    prefill_tile8<E, TQ, SUB, HALF>(a, row, smem);
   }
   PH_TL(11);
 }
@@ -1159,6 +1170,8 @@ static int launch_prefix_t(const PrefixArgs& a, int num_groups, int max_group_re
   return launch_status();
 }
 
+constexpr int64_t kMaxGridY = 65535;  // grid extent in y and z
+
 template <typename E, int TQ, int SUB, bool HALF = false>
 static int launch_prefill_tq(const PrefillArgs& a, int64_t num_tokens, hipStream_t st) {
   constexpr int QT = 32 * (8 / TQ);  // queries per workgroup tile
@@ -1166,7 +1179,8 @@ static int launch_prefill_tq(const PrefillArgs& a, int64_t num_tokens, hipStream
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_mfma8_kernel<E, TQ, SUB, HALF>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, kTile8Lds);
   const int hx = (a.H + 7) / 8 * 8;  // keeps head == linear id mod 8 for every tile row
-  const int64_t max_tiles = num_tokens / QT + a.num_chunks;  // >= sum of ceil(n_c / QT)
+  int64_t max_tiles = num_tokens / QT + a.num_chunks;  // >= sum of ceil(n_c / QT)
+  if (max_tiles > kMaxGridY) max_tiles = kMaxGridY;      // the kernel strides over the tile rows beyond the grid
   hipLaunchKernelGGL((prefill_mfma8_kernel<E, TQ, SUB, HALF>), dim3(hx, (unsigned)max_tiles), dim3(512), kTile8Lds, st,
                      a);
   return launch_status();

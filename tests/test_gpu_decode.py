@@ -810,6 +810,91 @@ def test_captured_decode_step_replays_while_contexts_grow(dev):
     torch.testing.assert_close(out_static.cpu().float(), ref.float(), **TOL[torch.float16])
 
 
+def test_captured_library_planned_step_replays_while_contexts_grow(dev):
+    """A caller without a plan of its own: the library builds the suffix plan inside the call, so the plan launch
+    and its length bound are part of what a graph records.  Captured with max_suffix_len = the table's width (the
+    largest length a replay will see), the replays follow the growing lists; each equals the eager result on
+    tables built from scratch."""
+    from parrotserve_amd import kernels, synth, table_cache
+
+    g = torch.Generator().manual_seed(30)
+    B, H, D, P = 48, 8, 128, 600
+    lens = torch.randint(1, 80, (B,), generator=g).tolist()
+    case = synth.make_decode_case("growlib", 30, torch.float16, 1, B, P, lens, H, D, 1 << 14)
+    kc, vc = synth.pool_to_device(case.k_rows, case.v_rows, case.used_slots, case.pool_slots, dev)
+    prefix = case.pool_lists(case.prefix_lists)
+    suffix = [list(l) for l in case.pool_lists(case.suffix_lists)]
+    used = set(case.used_slots.tolist())
+    spare = [s for s in range(case.pool_slots) if s not in used][: 5 * B]
+    tables = kernels.DecodeTables.build(prefix, case.group_req_cu, suffix, dev, num_heads=H, head_dim=D,
+                                        balanced=False)
+    assert tables.plan is None
+    tables.chunk_tokens = 0                                  # leave the decomposition to the library: it plans
+    table_cache._widen(tables, max(lens) + 8, dev)
+    tables.max_suffix_len = tables.suffix_table_stride       # what the captured call records as its bound
+    q_static = case.q.to(dev)
+    out_static = torch.empty_like(q_static)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        kernels.decode_attention(q_static, kc, vc, tables, out=out_static)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        kernels.decode_attention(q_static, kc, vc, tables, out=out_static)
+    gq = torch.Generator(device=dev).manual_seed(7)
+    for it in range(5):
+        new = spare[it * B:(it + 1) * B]
+        new_dev = torch.tensor(new, dtype=torch.int32, device=dev)
+        kc[new_dev.long()] = torch.randn((B, H, D), generator=gq, device=dev, dtype=torch.float16)
+        vc[new_dev.long()] = torch.randn((B, H, D), generator=gq, device=dev, dtype=torch.float16)
+        for b in range(B):
+            suffix[b].append(new[b])
+        kernels.suffix_tables_append(tables.suffix_slots, tables.suffix_lens, None, new_dev)
+        q_new = torch.randn(q_static.shape, generator=gq, device=dev, dtype=torch.float16)
+        fresh = kernels.DecodeTables.build(prefix, case.group_req_cu, suffix, dev, num_heads=H, head_dim=D)
+        eager = kernels.decode_attention(q_new, kc, vc, fresh)
+        torch.cuda.synchronize()
+        q_static.copy_(q_new)
+        out_static.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        torch.testing.assert_close(out_static.float(), eager.float(), **TOL[torch.float16])
+    full = [prefix[0] + l for l in suffix]
+    ref = ref_decode_attention(q_static.cpu(), kc.cpu(), vc.cpu(), [torch.tensor(l) for l in full])
+    torch.testing.assert_close(out_static.cpu().float(), ref.float(), **TOL[torch.float16])
+
+
+def test_inconsistent_table_extents(dev):
+    """A padded table that does not hold max_suffix_len entries in its last row is refused; a ragged table whose
+    last list runs past the table's end is read up to the end by the kernel that writes the parts and by the one
+    that merges them alike (the result is that of the truncated list)."""
+    from parrotserve_amd import kernels
+
+    g = torch.Generator().manual_seed(33)
+    B, H, D, W = 5, 4, 128, 40
+    k = torch.randn(B * W, H, D, generator=g).half()
+    v = torch.randn(B * W, H, D, generator=g).half()
+    q = torch.randn(B, H, D, generator=g).half()
+    rows = torch.randperm(B * W, generator=g).to(torch.int32)
+    lens = torch.tensor([W, 7, W, 20, W], dtype=torch.int32)
+    padded = kernels.DecodeTables(num_reqs=B, suffix_slots=rows[: B * W - 9].to(dev), suffix_table_stride=W,
+                                  suffix_lens=lens.to(dev), max_suffix_len=W, chunk_tokens=16)
+    padded.suffix_slots_count = lambda: B * W - 9  # the true extent: the last row is nine entries short
+    with pytest.raises(ValueError):
+        kernels.decode_attention(q.to(dev), k.to(dev), v.to(dev), padded)
+    # ragged: lists back to back, the last one claims W tokens but only W - 9 lie inside the table
+    offs = torch.tensor([0, W, W + 7, 2 * W + 7, 2 * W + 27], dtype=torch.int64)
+    total = int(offs[-1]) + W - 9
+    ragged = kernels.DecodeTables(num_reqs=B, suffix_slots=rows[:total].to(dev), suffix_offsets=offs.to(dev),
+                                  suffix_lens=lens.to(dev), max_suffix_len=W, chunk_tokens=16)
+    out = kernels.decode_attention(q.to(dev), k.to(dev), v.to(dev), ragged)
+    true_lens = [W, 7, W, 20, W - 9]
+    ref = ref_decode_attention(q, k, v, [rows[int(offs[b]): int(offs[b]) + true_lens[b]].long() for b in range(B)])
+    torch.testing.assert_close(out.cpu().float(), ref.float(), **TOL[torch.float16])
+
+
 @pytest.mark.parametrize("seed", range(12))
 def test_randomized_grouped_decode_shapes(dev, seed):
     """Seeded random batches: 1-3 prefix groups of 1-140 requests, prefixes of 1-1500 tokens (not multiples of

@@ -166,3 +166,20 @@ def test_randomized_prefill_shapes(dev, seed, D):
     case = synth.make_prefill_case("rnd", 2000 + seed, dtype, q_lens, ri(0, 700), ri(1, 6), D, 1 << 13)
     out, ref = run_prefill_case(case, dev)
     torch.testing.assert_close(out.float(), ref.float(), **TOL[dtype])
+
+
+def test_more_tile_rows_than_the_grid_holds(dev):
+    """70,000 one-token chunks without parents: more tile rows than a grid's y extent (65,535), so workgroups stride
+    over them.  A query that sees exactly one key returns that key's value row."""
+    from parrotserve_amd import kernels
+
+    C, H, D = 70000, 2, 128
+    g = torch.Generator(device=dev).manual_seed(12)
+    k = torch.randn((C, H, D), generator=g, device=dev, dtype=torch.bfloat16)
+    v = torch.randn((C, H, D), generator=g, device=dev, dtype=torch.bfloat16)
+    q = torch.randn((C, H, D), generator=g, device=dev, dtype=torch.bfloat16)
+    perm = torch.randperm(C, generator=torch.Generator().manual_seed(12))
+    tabs = kernels.PrefillTables.build([1] * C, [[int(s)] for s in perm.tolist()], dev)
+    out = kernels.prefill_attention(q, k, v, tabs)
+    torch.cuda.synchronize()
+    assert torch.equal(out, v[perm.to(dev)])

@@ -44,11 +44,18 @@ def _call_both(dev, dtype, seed, groups, per_group, P, H, D, smax):
     assert lib.ph_decode_attention(want.data_ptr(), q.data_ptr(), kc.data_ptr(), vc.data_ptr(), *common,
                                    ws.data_ptr(), nbytes, st) == 0
     got = torch.zeros_like(q)
+    # first call on the device outside the measured region: it looks the array's address up (hipGetSymbolAddress,
+    # which may load the code object)
+    assert lib.ph_decode_attention_static(got.data_ptr(), q.data_ptr(), kc.data_ptr(), vc.data_ptr(), *common, st) == 0
+    torch.cuda.synchronize()
+    got.zero_()
     torch.cuda.synchronize()
     before = torch.cuda.memory_allocated(dev)
+    free_before = torch.cuda.mem_get_info(dev)[0]  # the driver's own count: sees allocations torch's allocator does not
     assert lib.ph_decode_attention_static(got.data_ptr(), q.data_ptr(), kc.data_ptr(), vc.data_ptr(), *common, st) == 0
     torch.cuda.synchronize()
     assert torch.cuda.memory_allocated(dev) == before
+    assert torch.cuda.mem_get_info(dev)[0] == free_before
     ref = ref_decode_attention(case.q, case.k_rows, case.v_rows, case.full_lists())
     return got.cpu(), want.cpu(), ref
 
@@ -62,6 +69,40 @@ def test_static_scratch_entry_point_matches_workspace_entry_point(dev, dtype):
         torch.testing.assert_close(got.float(), want.float(), **TOL[dtype])
         assert torch.equal(got.view(torch.int16), want.view(torch.int16))  # same kernels, same order of sums
         torch.testing.assert_close(got.float(), ref.float(), **TOL[dtype])
+
+
+def test_static_scratch_entry_point_under_graph_capture(dev):
+    """The entry point recorded into a graph (after one eager call on the device, which resolves the array's
+    address) and replayed three times with eager work between the replays: every replay equals the workspace form."""
+    from parrotserve_amd import kernels, synth
+
+    g = torch.Generator().manual_seed(43)
+    B, H, D, P = 64, 8, 128, 500
+    s = torch.randint(0, 70, (B,), generator=g).tolist()
+    case = synth.make_decode_case("nag", 43, torch.float16, 1, B, P, s, H, D, 1 << 14)
+    kc, vc = synth.pool_to_device(case.k_rows, case.v_rows, case.used_slots, case.pool_slots, dev)
+    t = kernels.DecodeTables.build(case.pool_lists(case.prefix_lists), case.group_req_cu,
+                                   case.pool_lists(case.suffix_lists), dev, num_heads=H, head_dim=D)
+    q = case.q.to(dev)
+    out = torch.empty_like(q)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        kernels.decode_attention_static(q, kc, vc, t, out)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        kernels.decode_attention_static(q, kc, vc, t, out)
+    gq = torch.Generator(device=dev).manual_seed(8)
+    for _ in range(3):
+        q.copy_(torch.randn(q.shape, generator=gq, device=dev, dtype=torch.float16))
+        want = kernels.decode_attention(q, kc, vc, t)       # eager work between the replays, on its own workspace
+        torch.cuda.synchronize()
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want)
 
 
 def test_static_scratch_entry_point_refuses_what_does_not_fit(dev):
