@@ -12,6 +12,7 @@ is no PyTorch fallback.
 """
 from __future__ import annotations
 
+import collections
 import ctypes
 import dataclasses
 from typing import Dict, List, Optional, Sequence, Tuple
@@ -758,15 +759,52 @@ def _check_paged_args(query, key_cache, value_cache, head_mapping, context_lens,
     assert block_tables.shape[0] == query.shape[0]
 
 
+# Device tables (with the balanced suffix plan) of recent calls of the reference-named ops.  Unchanged model code
+# calls these once per layer with the same tensors, and the plan depends on the lengths only: layer 1 of an
+# iteration builds it, layers 2..L find it here.  An entry is keyed by the tensors' addresses and torch's version
+# counter of the length tensor, and holds references to the tensors, so an address cannot come back for another
+# tensor while its entry lives; a length tensor rewritten in place through torch bumps the version and misses.
+# (Writes torch does not see -- a kernel of the caller's own -- are not detected: such a caller passes a new tensor.)
+_paged_tables_cache: "collections.OrderedDict[Tuple, Tuple[Tuple, DecodeTables]]" = collections.OrderedDict()
+_PAGED_TABLES_CACHE_ENTRIES = 8
+
+
+def _paged_tables(query, context_lens, block_tables, flash_context_len: int = 0, flash_block_table=None) -> DecodeTables:
+    B, H, D = query.shape
+    P = int(flash_context_len)
+    key = (context_lens.data_ptr(), context_lens._version, B, block_tables.data_ptr(), block_tables.stride(0),
+           block_tables.shape[1], H, D, query.dtype, P, 0 if flash_block_table is None else flash_block_table.data_ptr(),
+           str(query.device))
+    hit = _paged_tables_cache.get(key)
+    if hit is not None:
+        _paged_tables_cache.move_to_end(key)
+        return hit[1]
+    table = block_tables if block_tables.stride(1) == 1 else block_tables.contiguous()
+    lens = context_lens.contiguous()
+    t = DecodeTables(num_reqs=B, suffix_slots=table, suffix_offsets=None, suffix_table_stride=table.stride(0),
+                     suffix_lens=lens, max_suffix_len=table.shape[1])
+    if P > 0:
+        assert flash_block_table.dtype == torch.int32 and flash_block_table.numel() >= P
+        cu, gcu, gcu_host = _single_group_cu(P, B, query.device)
+        t.num_groups = 1
+        t.prefix_slots = flash_block_table.contiguous()
+        t.prefix_cu, t.group_req_cu, t.group_req_cu_host = cu, gcu, gcu_host
+        t.max_prefix_len = P
+    if 0 < B <= PLAN_MAX_REQS and t.max_suffix_len > 0:
+        t.plan_on_device(suffix_lane_capacity(query.device, H, D, num_reqs=B, num_groups=t.num_groups,
+                                              max_prefix_len=t.max_prefix_len, max_suffix_len=t.max_suffix_len,
+                                              dtype=query.dtype), query.device)
+    _paged_tables_cache[key] = ((context_lens, block_tables, flash_block_table), t)
+    while len(_paged_tables_cache) > _PAGED_TABLES_CACHE_ENTRIES:
+        _paged_tables_cache.popitem(last=False)
+    return t
+
+
 def vllm_paged_attention(query, key_cache, value_cache, head_mapping, context_lens, block_tables):
     """Non-shared ragged decode (parrot/engine/builtin/kernels/vllm/paged_attention.py:12-38):
     request i attends over ``block_tables[i, :context_lens[i]]``."""
     _check_paged_args(query, key_cache, value_cache, head_mapping, context_lens, block_tables)
-    block_tables = block_tables if block_tables.stride(1) == 1 else block_tables.contiguous()
-    t = DecodeTables(num_reqs=query.shape[0], suffix_slots=block_tables, suffix_offsets=None,
-                     suffix_table_stride=block_tables.stride(0), suffix_lens=context_lens.contiguous(),
-                     max_suffix_len=block_tables.shape[1])
-    return decode_attention(query, key_cache, value_cache, t)
+    return decode_attention(query, key_cache, value_cache, _paged_tables(query, context_lens, block_tables))
 
 
 def flash_paged_attention(query, key_cache, value_cache, head_mapping, flash_context_len, flash_block_table,
@@ -775,19 +813,7 @@ def flash_paged_attention(query, key_cache, value_cache, head_mapping, flash_con
     all requests attend over ``flash_block_table[:flash_context_len]`` plus their
     own ``paged_block_tables[i, :paged_context_lens[i]]``."""
     _check_paged_args(query, key_cache, value_cache, head_mapping, paged_context_lens, paged_block_tables)
-    B = query.shape[0]
-    P = int(flash_context_len)
-    paged_block_tables = paged_block_tables if paged_block_tables.stride(1) == 1 else paged_block_tables.contiguous()
-    t = DecodeTables(num_reqs=B, suffix_slots=paged_block_tables, suffix_offsets=None,
-                     suffix_table_stride=paged_block_tables.stride(0), suffix_lens=paged_context_lens.contiguous(),
-                     max_suffix_len=paged_block_tables.shape[1])
-    if P > 0:
-        assert flash_block_table.dtype == torch.int32 and flash_block_table.numel() >= P
-        cu, gcu, gcu_host = _single_group_cu(P, B, query.device)
-        t.num_groups = 1
-        t.prefix_slots = flash_block_table.contiguous()
-        t.prefix_cu, t.group_req_cu, t.group_req_cu_host = cu, gcu, gcu_host
-        t.max_prefix_len = P
+    t = _paged_tables(query, paged_context_lens, paged_block_tables, flash_context_len, flash_block_table)
     return decode_attention(query, key_cache, value_cache, t)
 
 

@@ -104,23 +104,26 @@ def test_attn_func_forward_matches_oracle(dev, name, n_groups, with_fills):
     assert torch.equal(store.v_cache[1].cpu().view(torch.int16), vc_ref.view(torch.int16))
 
 
-def test_decoder_layer_config5_scaled(dev):
-    """Config 5's recipe scaled down (fp16, weights N(0, 0.02), RMSNorm -> QKV -> RoPE -> prefix groups x
-    branches -> shared-prefix + suffix attention -> O-proj -> MLP): hidden 640, 5 heads x 128, FFN 1728,
-    2 groups x 8 branches, prefix 300, suffix U[4,40], seed 4."""
-    from parrotserve_amd import mem, synth
+def _check_config5_layer(dev, case, groups, branches, prefix, hidden, H, ffn, fused_ops, oracle_reqs=None,
+                         gemm_rows=None):
+    """One decoder layer of config 5's recipe on the GPU, stage by stage, each HIP op checked on the inputs it
+    really saw: RMSNorm, RoPE (bit-exact), append (bit-exact) and attention against the oracle; the stages behind
+    the library GEMMs against an fp32 CPU evaluation that takes the checked attention output.  ``oracle_reqs`` /
+    ``gemm_rows``: the requests (rows) the attention oracle / the CPU GEMMs are evaluated on (default: all)."""
+    from parrotserve_amd import mem
     from parrotserve_amd.attn_func import BuiltinConfig
     from parrotserve_amd.context import BlockContext, RecyclePool
     from parrotserve_amd.iter_state import IterationState
+    from parrotserve_amd.kernels import rope_and_cache, vllm_rotary_emb
+    from parrotserve_amd import synth
     from parrotserve_amd.llama_layer import LlamaDecoderLayer
     from parrotserve_amd.primitive_job import Generate
 
-    case = synth.config5(groups=2, branches=8, prefix=300, s_lo=4, s_hi=40, hidden=640, heads=5, ffn=1728,
-                         pool_slots=1 << 12)
     dec = case.decode
-    B, H, D, hidden = dec.num_reqs, 5, 128, 640
+    B, D = dec.num_reqs, 128
     slots = dec.pool_slots
-    store = mem.init_model_cache_storage(1, slots, H, D, torch.float16, dev, max_seq_len=1024, rope_theta=case.theta)
+    max_pos = int(case.positions.max()) + 1
+    store = mem.init_model_cache_storage(1, slots, H, D, torch.float16, dev, max_seq_len=max_pos, rope_theta=case.theta)
     kc, vc = synth.pool_to_device(dec.k_rows, dec.v_rows, dec.used_slots, slots, dev)
     store.k_cache[0].copy_(kc)
     store.v_cache[0].copy_(vc)
@@ -130,27 +133,29 @@ def test_decoder_layer_config5_scaled(dev):
         def __init__(self, ids):
             super().__init__(pool_size=None)
             self._ids = list(ids)
+            self._next = 0
 
         def allocate(self):
-            return self._ids.pop(0)
+            self._next += 1
+            return self._ids[self._next - 1]
 
     jobs = []
-    for gi in range(2):
+    for gi in range(groups):
         parent = BlockContext(gi, None, _Scripted(dec.used_slots[dec.prefix_lists[gi]].tolist()), 1)
-        parent.allocate(300)
-        for b in range(8):
-            r = gi * 8 + b
+        parent.allocate(prefix)
+        for b in range(branches):
+            r = gi * branches + b
             ids = dec.used_slots[dec.suffix_lists[r]].tolist()
-            child = BlockContext(100 + r, parent, _Scripted(ids), 1)
+            child = BlockContext(1000 + r, parent, _Scripted(ids), 1)
             child.allocate(len(ids))
             j = Generate(0, r, child.context_id, parent.context_id)
             j.context = child
             jobs.append(j)
     cfg = BuiltinConfig(num_kv_cache_blocks=slots, attn_func="hip_shared_prefix", dtype=torch.float16, device=dev)
     st = IterationState(jobs, type("C", (), dict(num_attention_heads=H, hidden_size=hidden))(), cfg)
-    assert st.decode_tables.num_groups == 2 and st.decode_perm is None
+    assert st.decode_tables.num_groups == groups and st.decode_perm is None
 
-    layer = LlamaDecoderLayer(hidden, H, 1728, case.eps, 0, cfg.attn_func).half().to(dev)
+    layer = LlamaDecoderLayer(hidden, H, ffn, case.eps, 0, cfg.attn_func, fused_ops=fused_ops).half().to(dev)
     w = case.weights
     with torch.no_grad():
         layer.self_attn.qkv_proj.weight.copy_(w["qkv_proj"])
@@ -161,16 +166,22 @@ def test_decoder_layer_config5_scaled(dev):
     x = case.x.to(dev)
     pos = case.positions.to(dev)
 
-    # GPU, stage by stage (same calls LlamaDecoderLayer.forward makes), so each HIP op is checked on the
-    # inputs it really saw
+    # GPU, stage by stage (the calls LlamaAttention.forward makes for this setting of fused_ops)
     with torch.inference_mode():
         h1 = layer.input_layernorm(x)
         qkv = layer.self_attn.qkv_proj(h1)
         qkv_before = qkv.clone()
         q, k, v = torch.chunk(qkv, 3, dim=-1)
-        from parrotserve_amd.kernels import vllm_rotary_emb
-        vllm_rotary_emb(pos, q, k, mem.get_cos_sin_cache(), head_size=D)
-        attn_out = layer.self_attn.attn_func(q.view(B, H, D), k.view(B, H, D), v.view(B, H, D), st)
+        if fused_ops:
+            rope_and_cache(pos, q, k, v, mem.get_cos_sin_cache(), D, mem.get_k_cache(0), mem.get_v_cache(0),
+                           st.slot_mapping, key_in_place=False)
+            attn_out = layer.self_attn.attn_func(q.view(B, H, D), k.view(B, H, D), v.view(B, H, D), st,
+                                                 kv_appended=True)
+        else:
+            vllm_rotary_emb(pos, q, k, mem.get_cos_sin_cache(), head_size=D)
+            attn_out = layer.self_attn.attn_func(q.view(B, H, D), k.view(B, H, D), v.view(B, H, D), st)
+        k_cache_after = mem.Model_Cache.k_cache[0].clone()
+        v_cache_after = mem.Model_Cache.v_cache[0].clone()
         mem.Model_Cache.k_cache[0].copy_(kc)  # undo the append, then run the whole layer in one go
         mem.Model_Cache.v_cache[0].copy_(vc)
         y = layer(x, pos, st)
@@ -179,23 +190,33 @@ def test_decoder_layer_config5_scaled(dev):
     ref_h1 = ref_rms_norm(case.x, w["input_layernorm"], case.eps)
     torch.testing.assert_close(h1.cpu().float(), ref_h1.float(), **TOL)
     # 2. RoPE on the GPU's own qkv (bit-exact with the reference kernel's arithmetic)
-    cache = ref_cos_sin_cache(1024, D, case.theta, torch.float16)
+    cache = ref_cos_sin_cache(max_pos, D, case.theta, torch.float16)
     torch.testing.assert_close(mem.get_cos_sin_cache().cpu().float(), cache.float(), atol=1e-3, rtol=0)
     qb, kb, vb = qkv_before.cpu().chunk(3, dim=-1)
     rq, rk = ref_rope_neox(case.positions, qb, kb, mem.get_cos_sin_cache().cpu(), D, elem_rounding=True)
     assert torch.equal(q.cpu().view(torch.int16), rq.contiguous().view(torch.int16))
-    assert torch.equal(k.cpu().view(torch.int16), rk.contiguous().view(torch.int16))
-    # 3. append + shared-prefix attention on those q/k/v
+    if not fused_ops:  # the fused pass writes the rotated k rows to the cache only
+        assert torch.equal(k.cpu().view(torch.int16), rk.contiguous().view(torch.int16))
+    # 3. append (bit-exact, only at the new tokens' slots) + shared-prefix attention on those q/k/v
     k_rows, v_rows = dec.k_rows.clone(), dec.v_rows.clone()
     for r in range(B):
         last = int(dec.suffix_lists[r][-1])
         k_rows[last] = rk.view(B, H, D)[r]
         v_rows[last] = vb.reshape(B, H, D)[r]
-    ref_attn = ref_decode_attention(rq.view(B, H, D), k_rows, v_rows, dec.full_lists())
-    torch.testing.assert_close(attn_out.cpu().view(B, H, D).float(), ref_attn.float(), **TOL)
+    used = dec.used_slots[: k_rows.shape[0]].to(dev)
+    assert torch.equal(k_cache_after[used].cpu().view(torch.int16), k_rows.view(torch.int16))
+    assert torch.equal(v_cache_after[used].cpu().view(torch.int16), v_rows.view(torch.int16))
+    untouched = torch.ones(slots, dtype=torch.bool, device=dev)
+    untouched[used] = False
+    assert not k_cache_after[untouched].any() and not v_cache_after[untouched].any()
+    pick = list(range(B)) if oracle_reqs is None else list(oracle_reqs)
+    full = dec.full_lists()
+    ref_attn = ref_decode_attention(rq.view(B, H, D)[pick], k_rows, v_rows, [full[i] for i in pick])
+    torch.testing.assert_close(attn_out.cpu().view(B, H, D)[pick].float(), ref_attn.float(), **TOL)
     # 4. whole layer vs an fp32 CPU evaluation that takes the checked attention output
-    a = attn_out.cpu().float()
-    hcpu = case.x.float() + (a @ w["o_proj"].float().t()).half().float()
+    rows = list(range(B)) if gemm_rows is None else list(gemm_rows)
+    a = attn_out.cpu().float()[rows]
+    hcpu = case.x.float()[rows] + (a @ w["o_proj"].float().t()).half().float()
     hcpu = hcpu.half()
     h2 = ref_rms_norm(hcpu, w["post_attention_layernorm"], case.eps).float()
     gate = (h2 @ w["gate_proj"].float().t()).half().float()
@@ -203,7 +224,43 @@ def test_decoder_layer_config5_scaled(dev):
     act = (torch.nn.functional.silu(gate).half().float() * up).half().float()
     mlp = (act @ w["down_proj"].float().t()).half().float()
     ref_y = (hcpu.float() + mlp).half()
-    torch.testing.assert_close(y.cpu().float(), ref_y.float(), atol=2e-2, rtol=2e-2)
+    torch.testing.assert_close(y.cpu()[rows].float(), ref_y.float(), atol=2e-2, rtol=2e-2)
+    mem.Model_Cache = None
+
+
+@pytest.mark.parametrize("fused_ops", [False, True])
+def test_decoder_layer_config5_scaled(dev, fused_ops):
+    """Config 5's recipe scaled down (fp16, weights N(0, 0.02), RMSNorm -> QKV -> RoPE -> prefix groups x
+    branches -> shared-prefix + suffix attention -> O-proj -> MLP): hidden 640, 5 heads x 128, FFN 1728,
+    2 groups x 8 branches, prefix 300, suffix U[4,40], seed 4."""
+    from parrotserve_amd import synth
+
+    case = synth.config5(groups=2, branches=8, prefix=300, s_lo=4, s_hi=40, hidden=640, heads=5, ffn=1728,
+                         pool_slots=1 << 12)
+    _check_config5_layer(dev, case, 2, 8, 300, 640, 5, 1728, fused_ops)
+
+
+_C5_FULL = {}
+
+
+@pytest.mark.parametrize("fused_ops", [False, True])
+def test_decoder_layer_config5_full_size(dev, fused_ops):
+    """Config 5 at full size: hidden 5120, 40 heads x 128, FFN 13824, 4 groups x 32 branches over 6000-token
+    prefixes, suffix U[32,1024], seed 4.  RMSNorm, RoPE and the append on all 128 rows; the attention oracle on
+    twelve requests (three per group, the shortest and longest suffix among them); the stages behind the GEMMs on
+    16 sampled rows."""
+    from parrotserve_amd import synth
+
+    if "case" not in _C5_FULL:
+        _C5_FULL["case"] = synth.config5()
+    case = _C5_FULL["case"]
+    lens = [l.numel() for l in case.decode.suffix_lists]
+    pick = sorted({min(range(128), key=lens.__getitem__), max(range(128), key=lens.__getitem__),
+                   0, 17, 31, 32, 50, 63, 64, 95, 100, 127})
+    rows = [0, 5, 13, 31, 32, 40, 47, 63, 64, 70, 77, 95, 96, 101, 120, 127]
+    _check_config5_layer(dev, case, 4, 32, 6000, 5120, 40, 13824, fused_ops, oracle_reqs=pick, gemm_rows=rows)
+    if fused_ops:
+        _C5_FULL.clear()
 
 
 @pytest.mark.parametrize("name,n_groups", [("xformers_fill_shared_prompts_generate", 1), ("hip_shared_prefix", 3)])

@@ -322,6 +322,44 @@ def test_reference_named_entry_points(dev):
     torch.testing.assert_close(out1.float(), ref.float(), **TOL[torch.float16])
 
 
+def test_reference_named_ops_reuse_the_plan_across_layers_and_notice_new_lengths(dev):
+    """The reference-named ops keep the device tables and suffix plan of a call for the next call with the same
+    tensors (the next layer of the iteration).  Lengths rewritten in place through torch must not find the old
+    plan: the second result is checked against the oracle on the new lengths."""
+    from parrotserve_amd import kernels, synth
+
+    g = torch.Generator().manual_seed(10)
+    B, P, H, D = 24, 260, 8, 128
+    s = torch.randint(20, 90, (B,), generator=g).tolist()
+    case = synth.make_decode_case("rc", 10, torch.float16, 1, B, P, s, H, D, 1 << 12)
+    kc, vc = synth.pool_to_device(case.k_rows, case.v_rows, case.used_slots, case.pool_slots, dev)
+    suf = case.pool_lists(case.suffix_lists)
+    mx = max(len(x) for x in suf)
+    table = torch.tensor([x + [0] * (mx - len(x)) for x in suf], dtype=torch.int32, device=dev)
+    lens = torch.tensor([len(x) for x in suf], dtype=torch.int32, device=dev)
+    flash = torch.tensor(case.pool_lists(case.prefix_lists)[0], dtype=torch.int32, device=dev)
+    hm = torch.arange(H, dtype=torch.int32, device=dev)
+    q = case.q.to(dev)
+    kernels._paged_tables_cache.clear()
+    out_a = kernels.flash_paged_attention(q, kc, vc, hm, P, flash, lens, table)
+    assert len(kernels._paged_tables_cache) == 1
+    tables_a = next(iter(kernels._paged_tables_cache.values()))[1]
+    out_b = kernels.flash_paged_attention(q, kc, vc, hm, P, flash, lens, table)  # "layer 2": same tensors
+    assert len(kernels._paged_tables_cache) == 1
+    assert next(iter(kernels._paged_tables_cache.values()))[1] is tables_a
+    assert torch.equal(out_a, out_b)
+    ref = ref_decode_attention(case.q, case.k_rows, case.v_rows, case.full_lists())
+    torch.testing.assert_close(out_a.cpu().float(), ref.float(), **TOL[torch.float16])
+    # the next iteration, written into the same tensor: every list one to nineteen tokens shorter
+    cut = torch.randint(1, 20, (B,), generator=g)
+    lens.sub_(cut.to(torch.int32).to(dev))
+    out_c = kernels.flash_paged_attention(q, kc, vc, hm, P, flash, lens, table)
+    assert len(kernels._paged_tables_cache) == 2
+    short = [torch.cat([case.prefix_lists[0], l[: l.numel() - int(c)]]) for l, c in zip(case.suffix_lists, cut)]
+    ref_c = ref_decode_attention(case.q, case.k_rows, case.v_rows, short)
+    torch.testing.assert_close(out_c.cpu().float(), ref_c.float(), **TOL[torch.float16])
+
+
 def test_head_mapping_must_be_identity(dev):
     """A mapping other than arange(H) (grouped KV heads) is refused, not silently ignored."""
     from parrotserve_amd import kernels
