@@ -271,6 +271,39 @@ int ph_decode_attention(void* out, const void* q, const void* k_cache, const voi
                         const ph_suffix_plan* plan,
                         void* workspace, size_t workspace_bytes, void* stream);
 
+/* ph_decode_attention for query heads that share KV heads (grouped / multi-query
+ * attention): the reference's native kernels read the KV head
+ * head_mapping[query head] (csrc/attention/attention_post_kernels.cu:79,101,
+ * attention_prev_kernels.cu, 3rdparty/vllm/csrc/attention/attention_kernels.cu:
+ * kv_head_idx = head_mapping[head_idx]).
+ *   k_cache, v_cache: [slots, num_kv_heads, D];
+ *   head_mapping: int32 [num_heads] (DEVICE), KV head of every query head, each
+ *                 in [0, num_kv_heads);
+ *   kv_group:     host statement about the mapping.  G > 0 asserts
+ *                 head_mapping[h] == h / G with num_heads == G * num_kv_heads
+ *                 (what repeat_interleave(arange(num_kv_heads), G) holds): for
+ *                 G a power of two up to 64, head size 128 and 16-bit elements
+ *                 the prefix phase then runs on the matrix cores with the G
+ *                 query heads of a KV head as G rows per request of one tile,
+ *                 so a group's prefix K/V is still read once -- and at G times
+ *                 the arithmetic per byte.  0 = any mapping: every phase runs
+ *                 per request.
+ * Everything else as ph_decode_attention (workspace: the same
+ * ph_decode_workspace_bytes). */
+int ph_decode_attention_gqa(void* out, const void* q, const void* k_cache, const void* v_cache,
+                            int64_t num_reqs, int64_t num_heads, int64_t num_kv_heads,
+                            const int32_t* head_mapping, int64_t kv_group, int64_t head_dim, int dtype,
+                            int64_t q_stride, int64_t out_stride, int64_t cache_stride_n,
+                            float scale,
+                            int64_t num_groups, const int32_t* prefix_slots, const int32_t* prefix_cu,
+                            const int32_t* group_req_cu, const int32_t* group_req_cu_host,
+                            int64_t max_prefix_len,
+                            const int32_t* suffix_slots, const int64_t* suffix_offsets,
+                            int64_t suffix_table_stride, int64_t suffix_slots_count,
+                            const int32_t* suffix_lens, int64_t max_suffix_len,
+                            int64_t chunk_tokens, const ph_suffix_plan* plan,
+                            void* workspace, size_t workspace_bytes, void* stream);
+
 /* ph_decode_attention without a workspace argument, for callers that cannot
  * allocate device memory (code under HIP graph capture, serving loops with a
  * fixed memory plan, harnesses that forbid hipMalloc).  No counterpart in the

@@ -34,6 +34,8 @@ SIGNATURES: Dict[str, Tuple[object, List[object]]] = {
     "ph_decode_workspace_bytes": (Z, [L, L, L, L, L, L, L, L]),
     "ph_decode_suffix_lanes": (L, [L, L, L, I, L, L, L]),
     "ph_decode_attention": (I, [P, P, P, P, L, L, L, I, L, L, L, F, L, P, P, P, P, L, P, P, L, L, P, L, L, P, P, Z, P]),
+    "ph_decode_attention_gqa": (I, [P, P, P, P, L, L, L, P, L, L, I, L, L, L, F, L, P, P, P, P, L, P, P, L, L, P, L, L, P, P, Z,
+                                    P]),
     "ph_prefix_attention": (I, [P, P, P, P, P, P, L, L, L, I, L, L, L, F, P, L, P, Z, P]),
     "ph_suffix_post_attention": (I, [P, P, P, P, P, P, L, L, L, I, L, L, L, F, P, P, L, L, P, L, L, P, Z, P]),
     "ph_suffix_prev_attention": (I, [P, P, P, P, P, P, L, L, L, I, L, L, L, F, P, P, L, L, P, L, L, P, Z, P]),

@@ -240,14 +240,23 @@ static Carve carve(void* ws, const DecodePlan& p, int64_t B, int64_t H, int64_t 
 // weights, is ignored).  Twice the matrix work, the same K/V traffic -- read once per group, not once per request.
 static bool pair_heads(int64_t D, int64_t H) { return D == 64 && H % 2 == 0; }
 
+// How the query heads of a decode call map onto the KV heads of the pools (grouped / multi-query attention,
+// csrc/attention/attention_post_kernels.cu:79,101).  map == null: query head h reads KV head h.
+struct KvHeads {
+  int64_t num_kv_heads = 0;       // 0: as many as query heads
+  const int32_t* map = nullptr;   // device, [H]: KV head of each query head
+  int64_t group = 0;              // host hint: > 0 asserts map[h] == h / group (H == group x num_kv_heads); 0: any map
+};
+
 static int check_common(const void* out, const void* q, const void* kc, const void* vc, int64_t B, int64_t H,
-                        int64_t D, int dtype, int64_t q_stride, int64_t out_stride, int64_t row_stride) {
+                        int64_t D, int dtype, int64_t q_stride, int64_t out_stride, int64_t row_stride,
+                        int64_t kv_heads = 0) {
   if (dtype != PH_F16 && dtype != PH_BF16 && dtype != PH_F32) return PH_ERR_DTYPE;
   if (D != 64 && D != 80 && D != 96 && D != 112 && D != 128 && D != 256) return PH_ERR_HEAD_DIM;
   if (B < 0 || H <= 0 || B > (1 << 24) || H > 4096) return PH_ERR_ARG;
   if (B == 0) return PH_OK;
   if (!out || !q || !kc || !vc) return PH_ERR_ARG;
-  if (q_stride < H * D || out_stride < H * D || row_stride < H * D) return PH_ERR_ARG;
+  if (q_stride < H * D || out_stride < H * D || row_stride < (kv_heads > 0 ? kv_heads : H) * D) return PH_ERR_ARG;
   if (!aligned16(out) || !aligned16(q) || !aligned16(kc) || !aligned16(vc) || q_stride % 8 || out_stride % 8 ||
       row_stride % 8)
     return PH_ERR_ALIGN;
@@ -267,12 +276,38 @@ static PrefixArgs pair_args(const PrefixArgs& pa, const Carve& ws) {
   return w;
 }
 
+// the prefix phase's arguments as the matrix-core kernel sees them when G = 1 << gshift query heads share each KV
+// head: G rows per request, one "head" per KV head
+static PrefixArgs gqa_args(const PrefixArgs& pa, int gshift) {
+  PrefixArgs w = pa;
+  w.B = pa.B << gshift;
+  w.H = pa.H >> gshift;
+  w.req_shift = gshift;
+  w.gqa = 1;
+  return w;
+}
+
+// log2 of the group size when the matrix-core kernel can take the query heads of a KV head as rows of one tile
+// (a power of two up to 64, the plain h -> h / G map, head size 128, 16-bit elements); -1 otherwise
+static int gqa_shift(const KvHeads& kv, int64_t H, int64_t D, int dtype) {
+  if (!kv.map || kv.group < 2 || kv.group > 64 || (kv.group & (kv.group - 1)) || D != 128 ||
+      !prefix_mfma_supported(dtype, 128) || kv.num_kv_heads * kv.group != H)
+    return -1;
+  int s = 0;
+  while ((1 << s) < kv.group) ++s;
+  return s;
+}
+
+// head_map != null with gshift < 0: any mapping, through the per-request kernel
 static int run_prefix(PrefixArgs& pa, int dtype, int D, int num_groups, const int32_t* group_req_cu_host,
                       int max_group_reqs, bool internal_ml, hipStream_t st, const Carve* pairs = nullptr,
-                      const KernelEvents& ev = KernelEvents()) {
+                      const KernelEvents& ev = KernelEvents(), const int32_t* head_map = nullptr, int gshift = -1) {
   if (pairs && pairs->opart_pairs)
     return launch_prefix_mfma(pair_args(pa, *pairs), dtype, 128, num_groups, 2 * max_group_reqs, internal_ml, st, ev);
-  if (prefix_mfma_supported(dtype, D))
+  if (head_map && gshift > 0)
+    return launch_prefix_mfma(gqa_args(pa, gshift), dtype, D, num_groups, max_group_reqs << gshift, internal_ml, st,
+                              ev);
+  if (!head_map && prefix_mfma_supported(dtype, D))
     return launch_prefix_mfma(pa, dtype, D, num_groups, max_group_reqs, internal_ml, st, ev);
   int rc = launch_clear_ml(pa.ml, (int64_t)pa.n_splits * pa.B * pa.H, st);
   if (rc != PH_OK) return rc;
@@ -296,6 +331,7 @@ static int run_prefix(PrefixArgs& pa, int dtype, int D, int num_groups, const in
     sa.req_begin = group_req_cu_host ? group_req_cu_host[g] : 0;
     sa.num_reqs = group_req_cu_host ? group_req_cu_host[g + 1] - group_req_cu_host[g] : pa.B;
     sa.scale_log2e = pa.scale_log2e;
+    sa.head_map = head_map;
     rc = launch_partial(sa, dtype, D, st);
     if (rc != PH_OK) return rc;
   }
@@ -383,7 +419,8 @@ static int decode_attention_impl(void* out, const void* q, const void* k_cache, 
                                  const int64_t* suffix_offsets, int64_t suffix_table_stride,
                                  int64_t suffix_slots_count, const int32_t* suffix_lens, int64_t max_suffix_len,
                                  int64_t chunk_tokens, const ph_suffix_plan* plan, void* workspace,
-                                 size_t workspace_bytes, void* stream, void* const* events6) {
+                                 size_t workspace_bytes, void* stream, void* const* events6,
+                                 const KvHeads& kv = KvHeads()) {
   const int B = (int)num_reqs, H = (int)num_heads, D = (int)head_dim;
   KernelEvents ev_prefix, ev_suffix, ev_merge;
   if (events6) {
@@ -391,13 +428,15 @@ static int decode_attention_impl(void* out, const void* q, const void* k_cache, 
     ev_suffix = KernelEvents{(hipEvent_t)events6[2], (hipEvent_t)events6[3]};
     ev_merge = KernelEvents{(hipEvent_t)events6[4], (hipEvent_t)events6[5]};
   }
+  if (kv.map && (kv.num_kv_heads <= 0 || kv.num_kv_heads > num_heads || kv.group < 0)) return PH_ERR_ARG;
   int rc = check_common(out, q, k_cache, v_cache, num_reqs, num_heads, head_dim, dtype, q_stride, out_stride,
-                        cache_stride_n);
+                        cache_stride_n, kv.map ? kv.num_kv_heads : 0);
   if (rc != PH_OK || num_reqs == 0) return rc;
   if (num_groups < 0 || max_prefix_len < 0 || max_suffix_len < 0 || max_suffix_len > INT32_MAX) return PH_ERR_ARG;
   const bool has_prefix = num_groups > 0 && max_prefix_len > 0;
   const bool has_suffix = max_suffix_len > 0;
   if (has_prefix && (!prefix_slots || !prefix_cu || !group_req_cu || !group_req_cu_host)) return PH_ERR_ARG;
+  const int gshift = gqa_shift(kv, num_heads, head_dim, dtype);  // > 0: the KV heads' query heads as matrix rows
   if (has_suffix && (!suffix_slots || !suffix_lens || suffix_slots_count <= 0)) return PH_ERR_ARG;
   // padded table: every row must hold max_suffix_len entries inside the table (the balanced form walks a row up to
   // its clamped length without knowing where the table ends)
@@ -408,8 +447,12 @@ static int decode_attention_impl(void* out, const void* q, const void* k_cache, 
   if (planned && (!plan->items || !plan->lane_rec || !plan->req_item_cu || plan->num_lanes <= 0 ||
                   plan->num_items > (int64_t)1 << 30))
     return PH_ERR_ARG;
-  const bool paired = pair_heads(D, H) && prefix_mfma_supported(dtype, 128);
-  const bool roles = roles_possible(num_reqs, num_heads, head_dim, dtype, has_prefix, has_suffix, planned, chunk_tokens);
+  // a head mapping takes the 64-wide head pairs out (a pair's heads need not share anything); it runs on the
+  // matrix cores as G rows per request when it is the plain h / G map at head size 128, else per request
+  const bool paired = !kv.map && pair_heads(D, H) && prefix_mfma_supported(dtype, 128);
+  const bool mfma_prefix = kv.map ? gshift > 0 : (paired || prefix_mfma_supported(dtype, D));
+  const bool roles = mfma_prefix && roles_possible(num_reqs, num_heads, head_dim, dtype, has_prefix, has_suffix,
+                                                   planned, chunk_tokens);
   const DecodePlan p = plan_decode(num_reqs, num_heads, has_prefix ? num_groups : 0, max_prefix_len, max_suffix_len,
                                    chunk_tokens, planned ? plan->num_items : 0, head_dim, pair_heads(D, H), roles);
   if (plan_bytes(p, B, H, D) > workspace_bytes || ((p.parts() > 0 || p.items > 0) && !workspace))
@@ -459,15 +502,16 @@ static int decode_attention_impl(void* out, const void* q, const void* k_cache, 
     pa.H = H;
     pa.scale_log2e = sl2;
     // roles for groups of any size; the shared form only where its eight-wave tile is at least half full
-    fuse = planned && (paired ? decode_fused_supported(dtype, 128) : decode_fused_supported(dtype, D)) &&
-           (p.prefix_wgs > 0 || (paired ? 2 : 1) * max_group_reqs > 32);
+    const int row_mult = paired ? 2 : gshift > 0 ? 1 << gshift : 1;  // rows of the matrix-core kernel per request
+    fuse = planned && mfma_prefix && (paired ? decode_fused_supported(dtype, 128) : decode_fused_supported(dtype, D)) &&
+           (p.prefix_wgs > 0 || row_mult * max_group_reqs > 32);
     if (fuse) {
-      fused_pa = paired ? pair_args(pa, ws) : pa;
+      fused_pa = paired ? pair_args(pa, ws) : gshift > 0 ? gqa_args(pa, gshift) : pa;
       fused_groups = (int)num_groups;
-      fused_max_reqs = paired ? 2 * max_group_reqs : max_group_reqs;
+      fused_max_reqs = row_mult * max_group_reqs;
     } else {
       rc = run_prefix(pa, dtype, D, (int)num_groups, group_req_cu_host, max_group_reqs, true, st,
-                      paired ? &ws : nullptr, ev_prefix);
+                      paired ? &ws : nullptr, ev_prefix, kv.map, gshift);
       if (rc != PH_OK) return rc;
     }
   }
@@ -489,6 +533,7 @@ static int decode_attention_impl(void* out, const void* q, const void* k_cache, 
     ia.ml = ws.ml + item_base * 2;
     ia.H = H;
     ia.scale_log2e = sl2;
+    ia.head_map = kv.map;
     rc = fuse ? launch_decode_fused(fused_pa, ia, dtype, fused_groups, fused_max_reqs, device_cus(), p.prefix_wgs, st,
                                       ev_suffix)
               : launch_items(ia, dtype, D, st, ev_suffix);
@@ -518,6 +563,7 @@ static int decode_attention_impl(void* out, const void* q, const void* k_cache, 
     sa.req_begin = 0;
     sa.num_reqs = B;
     sa.scale_log2e = sl2;
+    sa.head_map = kv.map;
     rc = launch_partial(sa, dtype, D, st, ev_suffix);
     if (rc != PH_OK) return rc;
   }
@@ -529,6 +575,7 @@ static int decode_attention_impl(void* out, const void* q, const void* k_cache, 
   ma.B = B;
   ma.H = H;
   ma.nA = has_prefix ? p.n_splits : 0;
+  ma.gshift = has_prefix && gshift > 0 ? gshift : 0;
   if (has_prefix && paired) {
     ma.opart_pairs = ws.opart_pairs;
     ma.ml_pairs = ws.ml_pairs;
@@ -560,6 +607,29 @@ extern "C" int ph_decode_attention(void* out, const void* q, const void* k_cache
                                group_req_cu_host, max_prefix_len, suffix_slots, suffix_offsets, suffix_table_stride,
                                suffix_slots_count, suffix_lens, max_suffix_len, chunk_tokens, plan, workspace,
                                workspace_bytes, stream, nullptr);
+}
+
+extern "C" int ph_decode_attention_gqa(void* out, const void* q, const void* k_cache, const void* v_cache,
+                                       int64_t num_reqs, int64_t num_heads, int64_t num_kv_heads,
+                                       const int32_t* head_mapping, int64_t kv_group, int64_t head_dim, int dtype,
+                                       int64_t q_stride, int64_t out_stride, int64_t cache_stride_n, float scale,
+                                       int64_t num_groups, const int32_t* prefix_slots, const int32_t* prefix_cu,
+                                       const int32_t* group_req_cu, const int32_t* group_req_cu_host,
+                                       int64_t max_prefix_len, const int32_t* suffix_slots,
+                                       const int64_t* suffix_offsets, int64_t suffix_table_stride,
+                                       int64_t suffix_slots_count, const int32_t* suffix_lens,
+                                       int64_t max_suffix_len, int64_t chunk_tokens, const ph_suffix_plan* plan,
+                                       void* workspace, size_t workspace_bytes, void* stream) {
+  if (!head_mapping) return PH_ERR_ARG;
+  KvHeads kv;
+  kv.num_kv_heads = num_kv_heads;
+  kv.map = head_mapping;
+  kv.group = kv_group;
+  return decode_attention_impl(out, q, k_cache, v_cache, num_reqs, num_heads, head_dim, dtype, q_stride, out_stride,
+                               cache_stride_n, scale, num_groups, prefix_slots, prefix_cu, group_req_cu,
+                               group_req_cu_host, max_prefix_len, suffix_slots, suffix_offsets, suffix_table_stride,
+                               suffix_slots_count, suffix_lens, max_suffix_len, chunk_tokens, plan, workspace,
+                               workspace_bytes, stream, nullptr, kv);
 }
 
 extern "C" size_t ph_decode_static_scratch_bytes(void) { return kStaticScratchBytes; }

@@ -61,12 +61,13 @@ __global__ __launch_bounds__(256) void decode_partial_kernel(PartialArgs a) {
   const int head = hg * HPW + lane / LPH;
   const bool head_ok = head < a.H;
   const int hclamp = head_ok ? head : a.H - 1;
-  const uint32_t lane_off = (uint32_t)(hclamp * D + HeadLanes<D>::chunk(lane) * 8);  // elements inside a token row
+  const uint32_t lane_off = (uint32_t)(hclamp * D + HeadLanes<D>::chunk(lane) * 8);  // elements inside a query row
+  const uint32_t kv_off = kv_lane_off<D>(a.head_map, hclamp, lane);                  // ... inside a K/V token row
   if (t0 >= len) return;
   const int t1 = min(len, t0 + a.chunk);
   const int64_t pr = ((int64_t)(a.part_base + c) * a.B + b) * a.H + hclamp;
   stream_request<E, D, TB, STAGES>(a.q, (int64_t)b * a.q_stride, a.kc, a.vc, a.row_stride, slots, myslot, t0, t1,
-                                   lane_off, a.scale_log2e, head_ok, a.opart, a.ml, pr);
+                                   lane_off, kv_off, a.scale_log2e, head_ok, a.opart, a.ml, pr);
 }
 
 // Balanced form: the host cut the batch's token stream into `num_lanes` near-equal pieces; a piece is
@@ -142,7 +143,10 @@ __global__ __launch_bounds__(256) void merge_kernel(MergeArgs a) {
       mlrow = a.ml_pairs + pr * 2;
       op = a.opart_pairs + pr * (2 * D) + (head & 1) * D + dl;
     } else {
-      if (i < a.nA)
+      if (i < a.nA && a.gshift > 0)  // grouped KV heads: the part of row b G + (head mod G), KV head head / G
+        pr = ((int64_t)i * ((int64_t)a.B << a.gshift) + ((int64_t)b << a.gshift) + (head & ((1 << a.gshift) - 1))) *
+                 (a.H >> a.gshift) + (head >> a.gshift);
+      else if (i < a.nA)
         pr = ((int64_t)i * a.B + b) * a.H + head;
       else if (a.req_item_cu)
         pr = a.item_base + (int64_t)(it0 + i - a.nA) * a.H + head;

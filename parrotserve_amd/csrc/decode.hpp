@@ -30,6 +30,7 @@ struct PartialArgs {
   int B, H;                 // full batch size / head count (workspace extents)
   int req_begin, num_reqs;  // requests covered by this launch
   float scale_log2e;
+  const int32_t* head_map;  // KV head of each query head (device, [H]); null = query head h reads KV head h
 };
 
 // Balanced (host-planned) suffix phase; partial rows are [item][H].
@@ -49,6 +50,7 @@ struct ItemArgs {
   float* ml;
   int H;
   float scale_log2e;
+  const int32_t* head_map;     // KV head of each query head (device, [H]); null = identity
 };
 
 struct MergeArgs {
@@ -62,6 +64,8 @@ struct MergeArgs {
   uint16_t* out;
   int64_t out_stride;
   int B, H;
+  int gshift;               // log2 G when parts [0, nA) were written on G rows per request and H / G KV heads
+                            // (grouped KV heads on the matrix-core kernel), 0 otherwise
   int nA;                   // parts [0, nA) are candidates for every request
   int baseB;                // parts [baseB, baseB + ceil(lens[b]/chunk)) likewise
   const int32_t* lens;      // may be null (no B range)
@@ -97,8 +101,12 @@ struct PrefixArgs {
   const int32_t* slots;        // all groups' prefix slots
   const int32_t* prefix_cu;    // [G+1] device
   const int32_t* group_req_cu; // [G+1] device
-  int req_shift;               // 1: 64-wide heads on head pairs -- B counts rows (two per request: row 2b + s is
-                               // request b, half s), H head pairs, q is the real [B][2 H][64] tensor
+  int req_shift;               // rows per request = 1 << req_shift; B counts rows and H what a row's heads are:
+                               //   gqa == 0, req_shift == 1: 64-wide heads on head pairs -- row 2b + s is request b,
+                               //     half s, H head pairs, q is the real [B][2 H][64] tensor;
+                               //   gqa == 1: G = 1 << req_shift query heads share each KV head -- row b G + j is
+                               //     request b, query head (KV head) G + j; H counts KV heads, q is [B][H G][128]
+  int gqa;
   int fixed_prefix_len;        // used when prefix_cu is null: one group, all requests, slots[0 .. len)
   int split_tokens;            // tokens per split (multiple of the tile)
   int n_splits;                // parts [0, n_splits)

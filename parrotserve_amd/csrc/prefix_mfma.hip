@@ -98,6 +98,9 @@ struct TileWork {
   //   0 / 1: every row of the tile is that half, qrow0 points at the half's 64 values;
   //   2: rows alternate, row q = request q >> 1 (rows of q_stride from qrow0, the pair's first value), half q & 1
   int pair_half = -1;
+  // grouped KV heads: row q of the tile is request q >> gshift, member q & (G - 1) of the G = 1 << gshift query
+  // heads that share this KV head; qrow0 points at the group's first query head of the tile's first request
+  int gshift = 0;
   // decode form: shares at most two steps longer than the ring touch the lines beyond it during their first two
   // steps.  Off for the prefix-only workgroups of the fused launch: next to a suffix stream that saturates the
   // memory system the touches (at any distance, at every step) made the steps slower, not faster (cold K/V:
@@ -612,6 +615,8 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
     } else if (wk.pair_half >= 0) {
       qp = wk.qrow0 + (int64_t)(ok ? q : 0) * wk.q_stride;
     }
+    if (wk.gshift > 0)
+      qp = wk.qrow0 + (int64_t)(ok ? q >> wk.gshift : 0) * wk.q_stride + (q & ((1 << wk.gshift) - 1)) * kPD + 64 * h;
     const bool mine = wk.pair_half < 0 || h == half;
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
@@ -927,9 +932,12 @@ __device__ __forceinline__ void prefix_unit8(const PrefixArgs& a, int split, int
     return;
   }
   TileWork wk;
-  // req_shift == 1: B and H count rows (two per request) and head pairs; q is the real [B][2 H][64] tensor
-  wk.qrow0 = a.q + (int64_t)(qbase >> a.req_shift) * a.q_stride + head * kPD;
-  wk.pair_half = a.req_shift ? 2 : -1;
+  // req_shift > 0: B counts rows (1 << req_shift per request).  Head pairs: H counts pairs, q is the real
+  // [B][2 H][64] tensor (a pair is 128 values wide).  Grouped KV heads: H counts KV heads, `head` is one, and its
+  // G query heads lie side by side in the query row.
+  wk.qrow0 = a.q + (int64_t)(qbase >> a.req_shift) * a.q_stride + (a.gqa ? (head << a.req_shift) : head) * kPD;
+  wk.pair_half = (a.req_shift && !a.gqa) ? 2 : -1;
+  wk.gshift = a.gqa ? a.req_shift : 0;
   wk.q_stride = a.q_stride;
   wk.nq = nq;
   wk.slots = a.slots + poff;
@@ -1241,7 +1249,7 @@ bool decode_fused_supported(int dtype, int D) { return D == kPD && (dtype == PH_
 
 int launch_decode_fused(const PrefixArgs& a, const ItemArgs& ia, int dtype, int num_groups, int max_group_reqs, int cus,
                         int prefix_wgs, hipStream_t st, const KernelEvents& ev) {
-  if (a.req_shift) {  // 64-wide heads: the prefix phase on head pairs, the suffix phase at its own width
+  if (a.req_shift && !a.gqa) {  // 64-wide heads: the prefix phase on head pairs, the suffix phase at its own width
     return dtype == PH_F16 ? launch_fused_t<F16, 64>(a, ia, num_groups, max_group_reqs, cus, prefix_wgs, st, ev)
                            : launch_fused_t<BF16, 64>(a, ia, num_groups, max_group_reqs, cus, prefix_wgs, st, ev);
   }

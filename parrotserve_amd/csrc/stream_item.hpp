@@ -12,7 +12,8 @@ namespace ph {
 
 // Streams the token rows slots[t0 .. t1) of one request through one wave (HPW adjacent heads) and
 // writes the (O, m, l) part at row `pr` of the partial buffers.  `myslot` holds the slot ids of the
-// first 64 tokens (lane i: token t0 + i, clamped), already fetched by the caller.
+// first 64 tokens (lane i: token t0 + i, clamped), already fetched by the caller.  `lane_off` = this lane's
+// element offset inside a token row of the K/V pools (its KV head's row, see kv_lane_off).
 template <typename E, int D, int TB, int STAGES>
 __device__ __forceinline__ void stream_item(const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
                                             int64_t row_stride, const int32_t* __restrict__ slots, int myslot,
@@ -178,12 +179,22 @@ __device__ __forceinline__ void stream_item_f32(const float* __restrict__ kc, co
   }
 }
 
-// One request's list [t0, t1) through one wave, whatever the element type: loads the query and runs the streaming body.
+// Element offset of this lane's 8 elements inside a token row of the K/V pools: the row of the lane's KV head --
+// the query head itself, or head_map[query head] when query heads share KV heads (grouped / multi-query
+// attention, csrc/attention/attention_post_kernels.cu:79,101: kv_head_idx = head_mapping[head_idx]).
+template <int D>
+__device__ __forceinline__ uint32_t kv_lane_off(const int32_t* head_map, int head, int lane) {
+  const int kvh = head_map ? head_map[head] : head;
+  return (uint32_t)(kvh * D + HeadLanes<D>::chunk(lane) * 8);
+}
+
+// One request's list [t0, t1) through one wave, whatever the element type: loads the query (at lane_off of the
+// query row) and runs the streaming body (K/V at kv_off of every token row).
 template <typename E, int D, int TB, int STAGES>
 __device__ __forceinline__ void stream_request(const uint16_t* q, int64_t q_off, const uint16_t* kc, const uint16_t* vc,
                                                int64_t row_stride, const int32_t* slots, int myslot, int t0, int t1,
-                                               uint32_t lane_off, float scale_log2e, bool head_ok, float* opart,
-                                               float* ml, int64_t pr) {
+                                               uint32_t lane_off, uint32_t kv_off, float scale_log2e, bool head_ok,
+                                               float* opart, float* ml, int64_t pr) {
   const int lane = threadIdx.x & 63;
   if constexpr (is_f32<E>::value) {
     float qf[8];
@@ -193,11 +204,11 @@ __device__ __forceinline__ void stream_request(const uint16_t* q, int64_t q_off,
       for (int i = 0; i < 8; ++i) qf[i] = 0.f;
     }
     stream_item_f32<D, TB>(reinterpret_cast<const float*>(kc), reinterpret_cast<const float*>(vc), row_stride, slots,
-                           myslot, t0, t1, qf, lane_off, scale_log2e, head_ok, opart, ml, pr);
+                           myslot, t0, t1, qf, kv_off, scale_log2e, head_ok, opart, ml, pr);
   } else {
     u32x4 qv = ld16(q + q_off + lane_off);
     if (!HeadLanes<D>::active(lane)) qv = u32x4{0u, 0u, 0u, 0u};
-    stream_item<E, D, TB, STAGES>(kc, vc, row_stride, slots, myslot, t0, t1, qv, lane_off, scale_log2e, head_ok, opart,
+    stream_item<E, D, TB, STAGES>(kc, vc, row_stride, slots, myslot, t0, t1, qv, kv_off, scale_log2e, head_ok, opart,
                                   ml, pr);
   }
 }
@@ -214,6 +225,7 @@ __device__ __forceinline__ void run_piece_rec(const ItemArgs& a, int hg, int4 re
   const bool head_ok = head < a.H;
   const int hclamp = head_ok ? head : a.H - 1;
   const uint32_t lane_off = (uint32_t)(hclamp * D + HeadLanes<D>::chunk(lane) * 8);
+  const uint32_t kv_off = kv_lane_off<D>(a.head_map, hclamp, lane);
   const int i0 = rec0.x, i1 = rec0.x + rec0.y;
   for (int it = i0; it < i1; ++it) {
     int4 meta = {rec0.z, rec0.w, rec1.x, 0};
@@ -222,7 +234,8 @@ __device__ __forceinline__ void run_piece_rec(const ItemArgs& a, int hg, int4 re
     const int32_t* slots = a.slots + (a.offsets ? a.offsets[b] : (int64_t)b * a.table_stride);
     const int myslot = slots[min(t0 + lane, t1 - 1)];
     stream_request<E, D, TB, STAGES>(a.q, (int64_t)b * a.q_stride, a.kc, a.vc, a.row_stride, slots, myslot, t0, t1,
-                                     lane_off, a.scale_log2e, head_ok, a.opart, a.ml, (int64_t)it * a.H + hclamp);
+                                     lane_off, kv_off, a.scale_log2e, head_ok, a.opart, a.ml,
+                                     (int64_t)it * a.H + hclamp);
   }
 }
 

@@ -650,16 +650,23 @@ def plan_suffix_items(lens: Sequence[int], num_lanes: int):
 
 def decode_attention(query: torch.Tensor, key_cache: torch.Tensor, value_cache: torch.Tensor, tables: DecodeTables,
                      scale: Optional[float] = None, out: Optional[torch.Tensor] = None,
-                     events6=None) -> torch.Tensor:
+                     events6=None, head_mapping: Optional[torch.Tensor] = None, kv_group: int = 0) -> torch.Tensor:
     """Shared-prefix (or plain ragged) decode attention: prefix phase on the
     matrix cores, per-request suffix phase, log-sum-exp merge.  ``events6``: optional array of six
     ``hipEvent_t`` handles that receive the begin / end timestamps of the call's prefix, suffix and merge
-    kernels (``ph_decode_attention_timed``)."""
+    kernels (``ph_decode_attention_timed``).  ``head_mapping`` (int32 device ``[H]``): query head h reads KV head
+    ``head_mapping[h]`` of caches ``[slots, H_kv, D]``; ``kv_group = G > 0`` states that it is ``h // G``
+    (``ph_decode_attention_gqa``)."""
     _require_gpu(query, key_cache, value_cache)
     assert query.dim() == 3 and key_cache.dim() == 3 and value_cache.shape == key_cache.shape
     B, H, D = query.shape
     assert B == tables.num_reqs
-    assert key_cache.shape[1:] == (H, D), "cache head shape mismatch"
+    if head_mapping is None:
+        assert key_cache.shape[1:] == (H, D), "cache head shape mismatch"
+    else:
+        assert events6 is None, "the timed call has no head mapping"
+        assert key_cache.shape[2] == D and head_mapping.dtype == torch.int32 and head_mapping.numel() == H
+        assert head_mapping.is_contiguous() and head_mapping.device == query.device
     assert query.dtype == key_cache.dtype == value_cache.dtype
     assert query.stride(2) == 1 and query.stride(1) == D
     assert key_cache.stride(2) == 1 and key_cache.stride(1) == D and key_cache.stride() == value_cache.stride()
@@ -682,7 +689,12 @@ def decode_attention(query: torch.Tensor, key_cache: torch.Tensor, value_cache: 
         tables.suffix_slots_count(), _ptr(tables.suffix_lens),
         tables.max_suffix_len, tables.chunk_tokens, None if plan is None else ctypes.byref(plan),
         _ptr(ws), ws.numel(), _stream())
-    rc = lib.ph_decode_attention(*args) if events6 is None else lib.ph_decode_attention_timed(*args, events6)
+    if head_mapping is not None:
+        rc = lib.ph_decode_attention_gqa(*args[:6], key_cache.shape[1], _ptr(head_mapping), int(kv_group), *args[6:])
+    elif events6 is None:
+        rc = lib.ph_decode_attention(*args)
+    else:
+        rc = lib.ph_decode_attention_timed(*args, events6)
     check(rc, "decode_attention")
     return out
 
@@ -730,33 +742,47 @@ def _single_group_cu(P: int, B: int, device) -> Tuple[torch.Tensor, torch.Tensor
     return hit
 
 
-_identity_head_maps: Dict[Tuple[int, int, int], bool] = {}
+# head mappings seen before: id of the tensor -> (the tensor itself, its version, what it was found to be).  The
+# entry holds the tensor, so its id and address cannot pass to another tensor while the entry lives.
+_head_maps: "collections.OrderedDict[int, Tuple[torch.Tensor, int, int, Tuple[Optional[torch.Tensor], int]]]" = \
+    collections.OrderedDict()
 
 
-def _check_head_mapping(head_mapping: torch.Tensor, num_heads: int) -> None:
+def _head_mapping_info(head_mapping: torch.Tensor, num_heads: int, num_kv_heads: int) -> Tuple[Optional[torch.Tensor], int]:
     """``head_mapping[h]`` names the KV head of query head h (3rdparty/vllm/csrc/attention/attention_kernels.cu:
-    ``kv_head_idx = head_mapping[head_idx]``).  The reference's models always pass ``arange(num_heads)``
-    (models/llama.py:95-97); the kernels here read KV head h for query head h, so anything else is refused rather
-    than silently ignored.  The contents are checked once per tensor (address and version): one small copy to the
-    host the first time a mapping is seen."""
+    ``kv_head_idx = head_mapping[head_idx]``).  Returns ``(None, 0)`` for the identity over as many KV heads as query
+    heads (what the reference's models pass, models/llama.py:95-97: the plain kernels), else ``(int32 mapping on
+    the device, G)`` with ``G > 0`` when the mapping is ``h // G`` and 0 for any other.  The contents are read
+    once per tensor and version (one small copy to the host)."""
     assert head_mapping.shape[0] == num_heads, "head_mapping must have one entry per head"
-    key = (head_mapping.data_ptr(), head_mapping._version, num_heads)
-    if key in _identity_head_maps:
-        return
-    if not torch.equal(head_mapping.detach().cpu().to(torch.int64), torch.arange(num_heads)):
-        raise ValueError("head_mapping must be arange(num_heads): grouped / multi-query KV heads are not supported")
-    if len(_identity_head_maps) > 64:
-        _identity_head_maps.clear()
-    _identity_head_maps[key] = True
+    hit = _head_maps.get(id(head_mapping))
+    if hit is not None and hit[0] is head_mapping and hit[1] == head_mapping._version and hit[2] == num_kv_heads:
+        return hit[3]
+    host = head_mapping.detach().cpu().to(torch.int64)
+    if int(host.min()) < 0 or int(host.max()) >= num_kv_heads:
+        raise ValueError("head_mapping names a KV head outside the cache")
+    if num_kv_heads == num_heads and torch.equal(host, torch.arange(num_heads)):
+        info: Tuple[Optional[torch.Tensor], int] = (None, 0)
+    else:
+        group = num_heads // num_kv_heads if num_heads % num_kv_heads == 0 else 0
+        if group and not torch.equal(host, torch.arange(num_heads) // group):
+            group = 0
+        info = (head_mapping.to(torch.int32).contiguous(), group)
+    _head_maps[id(head_mapping)] = (head_mapping, head_mapping._version, num_kv_heads, info)
+    while len(_head_maps) > 16:
+        _head_maps.popitem(last=False)
+    return info
 
 
 def _check_paged_args(query, key_cache, value_cache, head_mapping, context_lens, block_tables):
+    """Argument checks of the reference-named ops; returns the head mapping as ``decode_attention`` takes it."""
     if key_cache.dim() != 3 or value_cache.dim() != 3:
         raise ValueError("key_cache / value_cache must be token-granular [slots, H, D] (block_size 1)")
-    _check_head_mapping(head_mapping, query.shape[1])
     assert block_tables.dim() == 2 and block_tables.dtype == torch.int32
     assert context_lens.dtype == torch.int32 and context_lens.shape[0] == query.shape[0]
     assert block_tables.shape[0] == query.shape[0]
+    mapping, group = _head_mapping_info(head_mapping, query.shape[1], key_cache.shape[1])
+    return dict(head_mapping=mapping, kv_group=group)
 
 
 # Device tables (with the balanced suffix plan) of recent calls of the reference-named ops.  Unchanged model code
@@ -803,8 +829,8 @@ def _paged_tables(query, context_lens, block_tables, flash_context_len: int = 0,
 def vllm_paged_attention(query, key_cache, value_cache, head_mapping, context_lens, block_tables):
     """Non-shared ragged decode (parrot/engine/builtin/kernels/vllm/paged_attention.py:12-38):
     request i attends over ``block_tables[i, :context_lens[i]]``."""
-    _check_paged_args(query, key_cache, value_cache, head_mapping, context_lens, block_tables)
-    return decode_attention(query, key_cache, value_cache, _paged_tables(query, context_lens, block_tables))
+    heads = _check_paged_args(query, key_cache, value_cache, head_mapping, context_lens, block_tables)
+    return decode_attention(query, key_cache, value_cache, _paged_tables(query, context_lens, block_tables), **heads)
 
 
 def flash_paged_attention(query, key_cache, value_cache, head_mapping, flash_context_len, flash_block_table,
@@ -812,9 +838,9 @@ def flash_paged_attention(query, key_cache, value_cache, head_mapping, flash_con
     """Shared-prefix decode (parrot/engine/builtin/kernels/shared_flash_decoding.py:285-329):
     all requests attend over ``flash_block_table[:flash_context_len]`` plus their
     own ``paged_block_tables[i, :paged_context_lens[i]]``."""
-    _check_paged_args(query, key_cache, value_cache, head_mapping, paged_context_lens, paged_block_tables)
+    heads = _check_paged_args(query, key_cache, value_cache, head_mapping, paged_context_lens, paged_block_tables)
     t = _paged_tables(query, paged_context_lens, paged_block_tables, flash_context_len, flash_block_table)
-    return decode_attention(query, key_cache, value_cache, t)
+    return decode_attention(query, key_cache, value_cache, t, **heads)
 
 
 def paged_flash_attention(query, key_cache, value_cache, head_mapping, flash_context_len, flash_block_table,
@@ -823,7 +849,10 @@ def paged_flash_attention(query, key_cache, value_cache, head_mapping, flash_con
     first, exporting its row maxima and denominators (``single_query_cached_kv_prev_attention``), then the prefix
     phase merged on top of it in place (the Triton kernel with ``load_mid_results``) -- two calls of the library,
     ``ph_suffix_prev_attention`` and ``ph_prefix_post_attention``.  Same result as ``flash_paged_attention``."""
-    _check_paged_args(query, key_cache, value_cache, head_mapping, paged_context_lens, paged_block_tables)
+    heads = _check_paged_args(query, key_cache, value_cache, head_mapping, paged_context_lens, paged_block_tables)
+    if heads["head_mapping"] is not None:
+        raise ValueError("paged_flash_attention (the split entry points) takes the identity head_mapping only; "
+                         "flash_paged_attention serves grouped KV heads")
     _require_gpu(query, key_cache, value_cache, paged_context_lens, paged_block_tables)
     B, H, D = query.shape
     assert key_cache.shape[1:] == (H, D) and value_cache.shape == key_cache.shape

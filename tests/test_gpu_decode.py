@@ -360,22 +360,103 @@ def test_reference_named_ops_reuse_the_plan_across_layers_and_notice_new_lengths
     torch.testing.assert_close(out_c.cpu().float(), ref_c.float(), **TOL[torch.float16])
 
 
-def test_head_mapping_must_be_identity(dev):
-    """A mapping other than arange(H) (grouped KV heads) is refused, not silently ignored."""
-    from parrotserve_amd import kernels
+def _gqa_case(dtype, B, P, Hq, Hkv, D, seed, smax=90):
+    """A shared-prefix decode case with Hq query heads over Hkv KV heads: the case is drawn with Hkv heads and the
+    query widened to Hq."""
+    from parrotserve_amd import synth
 
-    B, H, D = 2, 4, 128
-    q = torch.zeros(B, H, D, dtype=torch.float16, device=dev)
-    kc = torch.zeros(8, H, D, dtype=torch.float16, device=dev)
-    table = torch.zeros(B, 4, dtype=torch.int32, device=dev)
-    lens = torch.full((B,), 2, dtype=torch.int32, device=dev)
-    gqa = torch.tensor([0, 0, 1, 1], dtype=torch.int32, device=dev)
-    for fn in (lambda hm: kernels.vllm_paged_attention(q, kc, kc, hm, lens, table),
-               lambda hm: kernels.flash_paged_attention(q, kc, kc, hm, 0, table[0, :0], lens, table),
-               lambda hm: kernels.paged_flash_attention(q, kc, kc, hm, 0, table[0, :0], lens, table)):
+    g = torch.Generator().manual_seed(seed)
+    s = torch.randint(1, smax, (B,), generator=g).tolist()
+    case = synth.make_decode_case("gqa", seed, dtype, 1, B, P, s, Hkv, D, 1 << 13)
+    q = torch.randn(B, Hq, D, generator=g).to(dtype)
+    return case, q
+
+
+def _paged_inputs(case, dev):
+    suf = case.pool_lists(case.suffix_lists)
+    mx = max(len(x) for x in suf)
+    table = torch.tensor([x + [0] * (mx - len(x)) for x in suf], dtype=torch.int32, device=dev)
+    lens = torch.tensor([len(x) for x in suf], dtype=torch.int32, device=dev)
+    flash = torch.tensor(case.pool_lists(case.prefix_lists)[0], dtype=torch.int32, device=dev)
+    return flash, lens, table
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("D", [128, 64])
+@pytest.mark.parametrize("B,P", [(48, 700), (7, 150)])
+def test_grouped_kv_heads(dev, dtype, D, B, P):
+    """head_mapping = repeat_interleave(arange(H / 4), 4): four query heads share each KV head
+    (csrc/attention/attention_post_kernels.cu:79,101).  flash_paged_attention and vllm_paged_attention against an
+    oracle that gathers KV head h // 4 for query head h."""
+    from parrotserve_amd import kernels, synth
+
+    Hq, Hkv = 16, 4
+    case, q = _gqa_case(dtype, B, P, Hq, Hkv, D, 300 + B + D)
+    hm = torch.arange(Hkv, dtype=torch.int32).repeat_interleave(Hq // Hkv)
+    kc, vc = synth.pool_to_device(case.k_rows, case.v_rows, case.used_slots, case.pool_slots, dev)
+    flash, lens, table = _paged_inputs(case, dev)
+    ref = ref_decode_attention(q, case.k_rows[:, hm.long()], case.v_rows[:, hm.long()], case.full_lists())
+    out = kernels.flash_paged_attention(q.to(dev), kc, vc, hm.to(dev), P, flash, lens, table)
+    torch.testing.assert_close(out.cpu().float(), ref.float(), **TOL[dtype])
+    full = [case.used_slots[l].tolist() for l in case.full_lists()]
+    mx = max(len(x) for x in full)
+    ftable = torch.tensor([x + [0] * (mx - len(x)) for x in full], dtype=torch.int32, device=dev)
+    flens = torch.tensor([len(x) for x in full], dtype=torch.int32, device=dev)
+    out1 = kernels.vllm_paged_attention(q.to(dev), kc, vc, hm.to(dev), flens, ftable)
+    torch.testing.assert_close(out1.cpu().float(), ref.float(), **TOL[dtype])
+
+
+def test_any_head_mapping_and_the_identity(dev):
+    """A mapping that is not h // G (here a permutation with repeats) runs per request; multi-query attention (one
+    KV head); and the identity mapping over equal head counts is the plain call, bit for bit.  The split entry
+    points (paged_flash_attention) take the identity only and say so."""
+    from parrotserve_amd import kernels, synth
+
+    dtype, D, B, P = torch.float16, 128, 20, 333
+    for Hq, Hkv, hm in ((6, 3, [2, 0, 0, 1, 2, 1]), (8, 1, [0] * 8), (12, 4, [0, 0, 0, 1, 1, 1, 2, 2, 2, 3, 3, 3])):
+        case, q = _gqa_case(dtype, B, P, Hq, Hkv, D, 400 + Hq)
+        hm_t = torch.tensor(hm, dtype=torch.int32)
+        kc, vc = synth.pool_to_device(case.k_rows, case.v_rows, case.used_slots, case.pool_slots, dev)
+        flash, lens, table = _paged_inputs(case, dev)
+        ref = ref_decode_attention(q, case.k_rows[:, hm_t.long()], case.v_rows[:, hm_t.long()], case.full_lists())
+        out = kernels.flash_paged_attention(q.to(dev), kc, vc, hm_t.to(dev), P, flash, lens, table)
+        torch.testing.assert_close(out.cpu().float(), ref.float(), **TOL[dtype])
         with pytest.raises(ValueError, match="head_mapping"):
-            fn(gqa)
-        fn(torch.arange(H, dtype=torch.int32, device=dev))
+            kernels.paged_flash_attention(q.to(dev), kc, vc, hm_t.to(dev), P, flash, lens, table)
+    # identity: the same kernels as a call without any mapping
+    case, q = _gqa_case(dtype, B, P, 8, 8, D, 77)
+    kc, vc = synth.pool_to_device(case.k_rows, case.v_rows, case.used_slots, case.pool_slots, dev)
+    flash, lens, table = _paged_inputs(case, dev)
+    ident = torch.arange(8, dtype=torch.int32, device=dev)
+    a = kernels.flash_paged_attention(q.to(dev), kc, vc, ident, P, flash, lens, table)
+    tabs = kernels.DecodeTables.build(case.pool_lists(case.prefix_lists), case.group_req_cu,
+                                      case.pool_lists(case.suffix_lists), dev, num_heads=8, head_dim=D)
+    b = kernels.decode_attention(q.to(dev), kc, vc, tabs)
+    assert torch.equal(a, b)
+    with pytest.raises(ValueError, match="head_mapping"):  # a KV head the cache does not have
+        kernels.flash_paged_attention(q.to(dev), kc, vc, ident + 1, P, flash, lens, table)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_grouped_kv_heads_on_the_matrix_cores_at_config2_proportions(dev, dtype):
+    """Grouped KV heads where the call runs the prefix and suffix phases in one launch with workgroups of their own:
+    64 requests x 32 query heads over 8 KV heads (G = 4: 256 query rows per KV head and tile), and two groups of
+    40 over 16 -> 8 heads (G = 2)."""
+    from parrotserve_amd import kernels, synth
+
+    for B, groups, P, Hq, Hkv, lo, hi in ((64, 1, 1536, 32, 8, 200, 700), (80, 2, 600, 16, 8, 100, 500)):
+        g = torch.Generator().manual_seed(500 + B)
+        s = torch.randint(lo, hi, (B,), generator=g).tolist()
+        case = synth.make_decode_case("gqa2", 500 + B, dtype, groups, B // groups, P, s, Hkv, 128, 1 << 17)
+        q = torch.randn(B, Hq, 128, generator=g).to(dtype)
+        hm = torch.arange(Hkv, dtype=torch.int32).repeat_interleave(Hq // Hkv)
+        kc, vc = synth.pool_to_device(case.k_rows, case.v_rows, case.used_slots, case.pool_slots, dev)
+        tabs = kernels.DecodeTables.build(case.pool_lists(case.prefix_lists), case.group_req_cu,
+                                          case.pool_lists(case.suffix_lists), dev, num_heads=Hq, head_dim=128,
+                                          dtype=dtype)
+        out = kernels.decode_attention(q.to(dev), kc, vc, tabs, head_mapping=hm.to(dev), kv_group=Hq // Hkv)
+        ref = ref_decode_attention(q, case.k_rows[:, hm.long()], case.v_rows[:, hm.long()], case.full_lists())
+        torch.testing.assert_close(out.cpu().float(), ref.float(), **TOL[dtype])
 
 
 def test_timed_call_is_the_same_call_with_timestamps(dev):
