@@ -310,22 +310,36 @@ def extras(torch, dev):
     return out
 
 
-TIMELINE_MARKS = ["kernel entry", "prefix slot window in LDS", "prefix ring requested, suffix stream starts",
-                  "suffix stream done", "prefix step 0 (tile landed, workgroup barrier passed)", "prefix step 1",
+TIMELINE_MARKS = ["kernel entry", "prefix slot window in LDS", "prefix ring requested, query loaded",
+                  None, "prefix step 0 (tile landed, workgroup barrier passed)", "prefix step 1",
                   "prefix step 2", "prefix step 3", "prefix main loop done", "token groups folded",
                   None, "kernel exit"]
 
 
-def fused_timeline(torch, lib, step, launches=8):
+def _mark_table(rel, marks):
+    out = {}
+    for i, name in enumerate(marks):
+        c = rel[:, i]
+        c = c[~__import__("numpy").isnan(c)]
+        if name is None or c.size == 0:
+            continue
+        out[name] = {k: round(float(v), 2) for k, v in
+                     zip(("min", "p10", "p50", "p90", "max"), __import__("numpy").percentile(c, [0, 10, 50, 90, 100]))}
+    return out
+
+
+def fused_timeline(torch, lib, step, prefix_wgs, launches=8):
     """Per-wave timestamps at the marks of the fused prefix + suffix kernel (profiling variant of the library), in
     microseconds from the first wave's entry; the median over the launches of every wave's time, then its spread
-    over the 2048 waves.  The marks cost a store each: the instrumented kernel runs about 2 us longer."""
+    over the waves of each kind of workgroup: workgroups [0, prefix_wgs) run prefix units only, the others suffix
+    pieces only.  The marks cost a store each: the instrumented kernel runs about 2 us longer.  The shader clock
+    between the first prefix step and the end of the prefix loop comes from the same marks."""
     import numpy as np
 
     for i in range(16):
         step(i)
     torch.cuda.synchronize()
-    runs = []
+    runs, mhz = [], []
     for i in range(launches):
         lib.ph_timeline_clear()
         torch.cuda.synchronize()
@@ -333,20 +347,27 @@ def fused_timeline(torch, lib, step, launches=8):
         torch.cuda.synchronize()
         buf = np.zeros(4096 * 12, dtype=np.uint64)
         assert lib.ph_timeline_read(buf.ctypes.data_as(ctypes.c_void_p), buf.nbytes) == 0
+        clk = np.zeros(4096 * 12, dtype=np.uint64)
+        assert lib.ph_timeline_read_clocks(clk.ctypes.data_as(ctypes.c_void_p), clk.nbytes) == 0
         t = buf.reshape(4096, 12).astype(np.float64)
-        t = t[t[:, 0] > 0]
+        c = clk.reshape(4096, 12).astype(np.float64)
+        n = int((t[:, 0] > 0).sum())
+        ok = (t[:n, 4] > 0) & (t[:n, 8] > t[:n, 4])
+        if ok.any():
+            mhz.append(float(np.median((c[:n][ok, 8] - c[:n][ok, 4]) / ((t[:n][ok, 8] - t[:n][ok, 4]) / 100.0))))
+        t = t[:n]
         runs.append(np.where(t > 0, (t - t[:, 0].min()) / 100.0, np.nan))
     rel = np.nanmedian(np.stack(runs), axis=0)
-    out = {"waves": int(rel.shape[0]), "unit": "us from the first wave's entry", "marks": {}}
-    for i, name in enumerate(TIMELINE_MARKS):
-        c = rel[:, i]
-        c = c[~np.isnan(c)]
-        if name is None or c.size == 0:
-            continue
-        out["marks"][name] = {k: round(float(v), 2) for k, v in
-                              zip(("min", "p10", "p50", "p90", "max"), np.percentile(c, [0, 10, 50, 90, 100]))}
+    out = {"waves": int(rel.shape[0]), "unit": "us from the first wave's entry", "prefix_workgroups": int(prefix_wgs),
+           "suffix_workgroups": int(rel.shape[0] // 8 - prefix_wgs)}
+    if prefix_wgs > 0:
+        out["prefix_marks"] = _mark_table(rel[: prefix_wgs * 8], TIMELINE_MARKS)
+        out["suffix_marks"] = _mark_table(rel[prefix_wgs * 8:], TIMELINE_MARKS)
+    else:
+        out["marks"] = _mark_table(rel, TIMELINE_MARKS)
+    if mhz:
+        out["shader_clock_mhz_during_prefix_loop"] = round(float(np.median(mhz)), 0)
     wg = rel.reshape(-1, 8, 12)
-    out["suffix_done_spread_inside_workgroup_p50"] = round(float(np.nanmedian(wg[:, :, 3].max(1) - wg[:, :, 3].min(1))), 2)
     out["exit_by_xcd_p50"] = [round(float(np.nanmedian(wg[x::8, :, 11].max(1))), 2) for x in range(8)]
     return out
 
@@ -373,18 +394,26 @@ def prefill_timeline(torch, lib, dev, launches=6):
     for _ in range(5):
         kernels.prefill_attention(q, kc, vc, tab, out=o)
     torch.cuda.synchronize()
-    runs = []
+    runs, mhz = [], []
     for _ in range(launches):
         lib.ph_timeline_clear()
         torch.cuda.synchronize()
         kernels.prefill_attention(q, kc, vc, tab, out=o)
         torch.cuda.synchronize()
         buf = np.zeros(4096 * 12, dtype=np.uint64)
+        clk = np.zeros(4096 * 12, dtype=np.uint64)
         assert lib.ph_timeline_read(buf.ctypes.data_as(ctypes.c_void_p), buf.nbytes) == 0
+        assert lib.ph_timeline_read_clocks(clk.ctypes.data_as(ctypes.c_void_p), clk.nbytes) == 0
         t = buf.reshape(4096, 12).astype(np.float64)[: H * 8]
+        c = clk.reshape(4096, 12).astype(np.float64)[: H * 8]
+        ok = (t[:, 7] > 0) & (t[:, 8] > t[:, 7])
+        if ok.any():
+            mhz.append(float(np.median((c[ok, 8] - c[ok, 7]) / ((t[ok, 8] - t[ok, 7]) / 100.0))))
         runs.append(np.where(t > 0, (t - t[:, 0][t[:, 0] > 0].min()) / 100.0, np.nan))
     rel = np.nanmedian(np.stack(runs), axis=0)
     out = {"waves": int(rel.shape[0]), "steps": (par + n) // 64, "unit": "us from the first wave's entry", "marks": {}}
+    if mhz:
+        out["shader_clock_mhz_during_tile_loop"] = round(float(np.median(mhz)), 0)
     for i, name in enumerate(PREFILL_TIMELINE_MARKS):
         c = rel[:, i]
         c = c[~np.isnan(c)]
@@ -393,6 +422,53 @@ def prefill_timeline(torch, lib, dev, launches=6):
         out["marks"][name] = {k: round(float(v), 2) for k, v in
                               zip(("min", "p10", "p50", "p90", "max"), np.percentile(c, [0, 10, 50, 90, 100]))}
     return out
+
+
+def prefix_timeline(torch, lib, dev, launches=6):
+    """The prefix kernel where the matrix pipe is the bound (one group of 1024 requests over 8192 tokens, 32 x 128
+    fp16: 256 workgroups of 256 queries x 4096 tokens each, the same tile loop as the prefill's): time per 64-token
+    step of a workgroup and the shader clock the compute units hold while every one of them runs the loop, from the
+    marks at the fourth step and at the end of the loop.  (The prefill timeline gives the same for 40 workgroups on
+    256 compute units.)"""
+    import numpy as np
+
+    from parrotserve_amd import kernels
+
+    B, H, D, P = 1024, 32, 128, 8192
+    g = torch.Generator(device=dev).manual_seed(11)
+    kc = torch.randn((2 * P, H, D), generator=g, device=dev, dtype=torch.float16)
+    vc = torch.randn((2 * P, H, D), generator=g, device=dev, dtype=torch.float16)
+    perm = torch.randperm(2 * P, generator=torch.Generator().manual_seed(11))
+    q = torch.randn((B, H, D), generator=g, device=dev, dtype=torch.float16)
+    o = torch.empty_like(q)
+    tabs = [kernels.DecodeTables.build([perm[i * P:(i + 1) * P].tolist()], [0, B], [[] for _ in range(B)], dev,
+                                       num_heads=H, head_dim=D) for i in range(2)]
+    for i in range(4):
+        kernels.decode_attention(q, kc, vc, tabs[i % 2], out=o)
+    torch.cuda.synchronize()
+    loop_us, mhz, wgs, first = [], [], 0, []
+    for i in range(launches):
+        lib.ph_timeline_clear()
+        torch.cuda.synchronize()
+        kernels.decode_attention(q, kc, vc, tabs[i % 2], out=o)
+        torch.cuda.synchronize()
+        buf = np.zeros(4096 * 12, dtype=np.uint64)
+        clk = np.zeros(4096 * 12, dtype=np.uint64)
+        assert lib.ph_timeline_read(buf.ctypes.data_as(ctypes.c_void_p), buf.nbytes) == 0
+        assert lib.ph_timeline_read_clocks(clk.ctypes.data_as(ctypes.c_void_p), clk.nbytes) == 0
+        t = buf.reshape(4096, 12).astype(np.float64)
+        c = clk.reshape(4096, 12).astype(np.float64)
+        ok = (t[:, 7] > 0) & (t[:, 8] > t[:, 7])
+        wgs = int(ok.sum()) // 8
+        us = (t[ok, 8] - t[ok, 7]) / 100.0
+        mhz.append(float(np.median((c[ok, 8] - c[ok, 7]) / us)))
+        loop_us.append(float(np.median(us)))
+        first.append(float(np.median((t[ok, 4] - t[ok, 1].min()) / 100.0)))
+    steps = P // 2 // 64  # two splits of 4096 tokens, 64-token steps
+    return {"batch": B, "prefix_len": P, "workgroups": wgs, "steps_per_workgroup": steps,
+            "first_step_us_after_first_window": round(float(np.median(first)), 2),
+            "us_per_step": round(float(np.median(loop_us)) / (steps - 4), 3),
+            "shader_clock_mhz_during_tile_loop": round(float(np.median(mhz)), 0)}
 
 
 def head_size_64_step(torch, dev):
@@ -771,6 +847,9 @@ def main():
     ap.add_argument("--prefix-regimes-only", action="store_true",
                     help="only run the prefix phase over batch sizes from the bandwidth-bound to the matrix-bound "
                          "regime, and the reference benchmark's shape, and exit")
+    ap.add_argument("--prefix-point-only", action="store_true",
+                    help="only run the prefix phase of one group of 256 requests over 8192 tokens (32 x 128 fp16, empty "
+                         "suffixes) a few times (for profiler counter passes on the 256-query tile) and exit")
     ap.add_argument("--prefill-only", action="store_true",
                     help="only run config 4's prefill kernel a few times (for profiler counter passes) and exit")
     args = ap.parse_args()
@@ -801,6 +880,23 @@ def main():
     if args.prefix_regimes_only:
         print(json.dumps({"prefix_regimes": prefix_regimes(torch, dev),
                           "bench_kernel_shape": bench_kernel_shape(torch, dev)}))
+        return
+
+    if args.prefix_point_only:
+        B, H, D, P = 256, 32, 128, 8192
+        g = torch.Generator(device=dev).manual_seed(11)
+        kc = torch.randn((4 * P, H, D), generator=g, device=dev, dtype=torch.float16)
+        vc = torch.randn((4 * P, H, D), generator=g, device=dev, dtype=torch.float16)
+        perm = torch.randperm(4 * P, generator=torch.Generator().manual_seed(11))
+        q = torch.randn((B, H, D), generator=g, device=dev, dtype=torch.float16)
+        o = torch.empty_like(q)
+        tabs = [kernels.DecodeTables.build([perm[i * P:(i + 1) * P].tolist()], [0, B], [[] for _ in range(B)], dev,
+                                           num_heads=H, head_dim=D) for i in range(4)]
+        rot = _Rotor(4)
+        t = _time_gpu(torch, lambda: kernels.decode_attention(q, kc, vc, tabs[rot.next()], out=o), iters=3, warmup=1,
+                      inner=4)
+        flops = 4 * B * H * P * D
+        print(json.dumps({"prefix_point_only": {"batch": B, "prefix_len": P, "us_with_merge": t * 1e6, "flops": flops}}))
         return
 
     if args.prefill_only:
@@ -871,8 +967,12 @@ def main():
         return (time.perf_counter() - t0) / steps
 
     if args.timeline:
-        print(json.dumps({"fused_kernel_timeline": fused_timeline(torch, lib, step),
-                          "prefill_kernel_timeline": prefill_timeline(torch, lib, dev)}))
+        hgroups = (H + 3) // 4  # four 128-wide heads per wave
+        cus = torch.cuda.get_device_properties(dev).multi_processor_count
+        prefix_wgs = cus - (int(tables[0].plan.num_lanes) * hgroups + 7) // 8  # what the plan's lane count leaves
+        print(json.dumps({"fused_kernel_timeline": fused_timeline(torch, lib, step, max(0, prefix_wgs)),
+                          "prefill_kernel_timeline": prefill_timeline(torch, lib, dev),
+                          "prefix_kernel_timeline": prefix_timeline(torch, lib, dev)}))
         return
 
     t_step = timed(step, args.steps, args.warmup)

@@ -4,7 +4,6 @@
 #include "decode.hpp"
 
 #include <algorithm>
-#include <cstdlib>
 #include <mutex>
 
 namespace ph {

@@ -27,7 +27,6 @@
 //
 // Math restated from parrot/engine/builtin/kernels/shared_flash_decoding.py:34-134.
 #include "stream_item.hpp"
-#include <cstdlib>
 
 namespace ph {
 
