@@ -132,6 +132,7 @@ struct PrefillArgs {
   int H;
   float scale_log2e;
   int pair;                  // 1: heads are 64 wide and run as halves of 128-wide head pairs (q, out, caches [.., H, 64])
+  int tile_row0;             // first tile row of this launch (grid.y covers rows tile_row0 ..)
 };
 
 int launch_partial(const PartialArgs& a, int dtype, int D, hipStream_t st, const KernelEvents& ev = KernelEvents());

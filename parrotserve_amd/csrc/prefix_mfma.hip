@@ -1119,18 +1119,17 @@ __device__ __forceinline__ void prefill_tile8(const PrefillArgs& a, int tile_row
 }
 
 // Prefill with parent context, eight waves: workgroup = (head, tile of 32 * (8 / TQ) queries of one chunk); grid.y
-// covers the tile rows, striding over them when there are more than the grid's y extent holds
+// covers the tile rows from a.tile_row0 on (more rows than a grid's y extent holds take several launches; a loop
+// over rows inside the kernel cost the common single-launch case 6 %)
 // HALF (64-wide heads, 256-query tiles): only this head's half of the pair's output is computed
 template <typename E, int TQ, int SUB, bool HALF = false>
 __global__ __launch_bounds__(512) void prefill_mfma8_kernel(PrefillArgs a) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   PH_TL(0);
   if ((int)blockIdx.x >= a.H) return;
-  const int tiles = a.tile_cu[a.num_chunks];
-  for (int row = blockIdx.y; row < tiles; row += gridDim.y) {
-    if (row != (int)blockIdx.y) __syncthreads();  // the last tile's fold scratch is the next tile's staging ring
-    prefill_tile8<E, TQ, SUB, HALF>(a, row, smem);
-  }
+  const int row = a.tile_row0 + (int)blockIdx.y;
+  if (row >= a.tile_cu[a.num_chunks]) return;
+  prefill_tile8<E, TQ, SUB, HALF>(a, row, smem);
   PH_TL(11);
 }
 
@@ -1186,10 +1185,14 @@ static int launch_prefill_tq(const PrefillArgs& a, int64_t num_tokens, hipStream
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_mfma8_kernel<E, TQ, SUB, HALF>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, kTile8Lds);
   const int hx = (a.H + 7) / 8 * 8;  // keeps head == linear id mod 8 for every tile row
-  int64_t max_tiles = num_tokens / QT + a.num_chunks;  // >= sum of ceil(n_c / QT)
-  if (max_tiles > kMaxGridY) max_tiles = kMaxGridY;      // the kernel strides over the tile rows beyond the grid
-  hipLaunchKernelGGL((prefill_mfma8_kernel<E, TQ, SUB, HALF>), dim3(hx, (unsigned)max_tiles), dim3(512), kTile8Lds, st,
-                     a);
+  const int64_t max_tiles = num_tokens / QT + a.num_chunks;  // >= sum of ceil(n_c / QT)
+  for (int64_t row0 = 0; row0 < max_tiles; row0 += kMaxGridY) {
+    PrefillArgs part = a;
+    part.tile_row0 = (int)row0;
+    const int64_t rows = max_tiles - row0 < kMaxGridY ? max_tiles - row0 : kMaxGridY;
+    hipLaunchKernelGGL((prefill_mfma8_kernel<E, TQ, SUB, HALF>), dim3(hx, (unsigned)rows), dim3(512), kTile8Lds, st,
+                       part);
+  }
   return launch_status();
 }
 
