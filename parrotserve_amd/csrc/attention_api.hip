@@ -371,7 +371,7 @@ extern "C" const char* ph_status_string(int status) {
   }
 }
 
-extern "C" int ph_abi_version(void) { return 2; }
+extern "C" int ph_abi_version(void) { return 3; }
 
 extern "C" size_t ph_decode_workspace_bytes(int64_t num_reqs, int64_t num_heads, int64_t head_dim,
                                             int64_t num_groups, int64_t max_prefix_len, int64_t max_suffix_len,
