@@ -107,6 +107,7 @@ struct PrefixArgs {
                                //   gqa == 1: G = 1 << req_shift query heads share each KV head -- row b G + j is
                                //     request b, query head (KV head) G + j; H counts KV heads, q is [B][H G][128]
   int gqa;
+  int head_dim;                // 0 / 128, or 80 / 96 / 112: a short head on the 128-wide tile (set by launch_prefix_mfma)
   int fixed_prefix_len;        // used when prefix_cu is null: one group, all requests, slots[0 .. len)
   int split_tokens;            // tokens per split (multiple of the tile)
   int n_splits;                // parts [0, n_splits)
@@ -133,6 +134,7 @@ struct PrefillArgs {
   float scale_log2e;
   int pair;                  // 1: heads are 64 wide and run as halves of 128-wide head pairs (q, out, caches [.., H, 64])
   int tile_row0;             // first tile row of this launch (grid.y covers rows tile_row0 ..)
+  int head_dim;              // 0 / 128, or 80 / 96 / 112: a short head on the 128-wide tile (set by launch_prefill_mfma)
 };
 
 int launch_partial(const PartialArgs& a, int dtype, int D, hipStream_t st, const KernelEvents& ev = KernelEvents());

@@ -97,6 +97,11 @@ struct TileWork {
   //   0 / 1: every row of the tile is that half, qrow0 points at the half's 64 values;
   //   2: rows alternate, row q = request q >> 1 (rows of q_stride from qrow0, the pair's first value), half q & 1
   int pair_half = -1;
+  // Head sizes 80, 96 and 112 on the 128-wide tile: a head's row in the pools and in q is head_dim elements long;
+  // the lanes that would load the chunks beyond it load the row's first chunk instead (valid memory, finite
+  // values), the query's dims beyond it are zero (so those K values never reach a score) and the output's are not
+  // written.  HBM traffic stays that of the real rows; LDS and the matrix pipe carry the padding.
+  int head_dim = 128;
   // grouped KV heads: row q of the tile is request q >> gshift, member q & (G - 1) of the G = 1 << gshift query
   // heads that share this KV head; qrow0 points at the group's first query head of the tile's first request
   int gshift = 0;
@@ -574,8 +579,11 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
   const char* gbase[LPT];
 #pragma unroll
   for (int i = 0; i < LPT; ++i)
-    gbase[i] = isv ? reinterpret_cast<const char*>(vc + (int64_t)head * kPD + ((c ^ (4 * tl)) * 8))
-                   : reinterpret_cast<const char*>(kc + (int64_t)head * kPD + ((c ^ ((4 * (r0 + i) + tl) & 15)) * 8));
+  {
+    const int cg = isv ? (c ^ (4 * tl)) : (c ^ ((4 * (r0 + i) + tl) & 15));  // the 16-byte chunk of the row this lane loads
+    const int cl = cg * 8 < wk.head_dim ? cg : 0;                            // chunks beyond a short head: its first chunk
+    gbase[i] = reinterpret_cast<const char*>((isv ? vc : kc) + (int64_t)head * wk.head_dim + cl * 8);
+  }
   const uint32_t dst0 = lds_addr_of(gl) + sub0 * kStage + (isv ? kVtOff : 0) + r0 * 1024;
   const uint32_t pf_lds = lds_addr_of(smem + kPfOff) + w8 * 256;
   const int pf_steps =
@@ -617,10 +625,12 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
     if (wk.gshift > 0)
       qp = wk.qrow0 + (int64_t)(ok ? q >> wk.gshift : 0) * wk.q_stride + (q & ((1 << wk.gshift) - 1)) * kPD + 64 * h;
     const bool mine = wk.pair_half < 0 || h == half;
+    const bool padded = wk.head_dim < kPD;  // (never together with head pairs or grouped rows)
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
-      u32x4 v = ld16(qp + 8 * s);
-      if (!ok || !mine) v = u32x4{0, 0, 0, 0};
+      const bool in = !padded || 64 * h + 8 * s < wk.head_dim;  // dims beyond a short head: read its first dims, use zero
+      u32x4 v = ld16(in ? qp + 8 * s : qp - 64 * h);
+      if (!ok || !mine || !in) v = u32x4{0, 0, 0, 0};
       if (PRESC) {
         // PRESC: q takes the factor scale * log2(e) here and is rounded to the element type again (what the
         // reference's own prefix kernel does, shared_flash_decoding.py:100), and the exponent reference enters
@@ -698,8 +708,8 @@ __device__ __forceinline__ void attn_tile8(const TileWork& wk, const uint16_t* _
         // token (of all four groups) and line of the step after `front`, clamped into the list and the window
         const int pt = min(min(front + STEP * TQ + (int)(threadIdx.x >> 2), s1 - 1), win0 + kWin - 1);
         const uint32_t slot = (uint32_t)win[pt - win0];
-        const char* base = reinterpret_cast<const char*>((threadIdx.x & 2) ? vc : kc) + (int64_t)head * (kPD * 2) +
-                           (threadIdx.x & 1) * 128;
+        const char* base = reinterpret_cast<const char*>((threadIdx.x & 2) ? vc : kc) +
+                           (int64_t)head * (wk.head_dim * 2) + (threadIdx.x & 1) * 128;
         lds_dma4(base + (uint64_t)slot * row_bytes, pf_lds);
       }
     }
@@ -934,7 +944,9 @@ __device__ __forceinline__ void prefix_unit8(const PrefixArgs& a, int split, int
   // req_shift > 0: B counts rows (1 << req_shift per request).  Head pairs: H counts pairs, q is the real
   // [B][2 H][64] tensor (a pair is 128 values wide).  Grouped KV heads: H counts KV heads, `head` is one, and its
   // G query heads lie side by side in the query row.
-  wk.qrow0 = a.q + (int64_t)(qbase >> a.req_shift) * a.q_stride + (a.gqa ? (head << a.req_shift) : head) * kPD;
+  const int hd = a.head_dim ? a.head_dim : kPD;  // 80 / 96 / 112: a short head on the 128-wide tile
+  wk.qrow0 = a.q + (int64_t)(qbase >> a.req_shift) * a.q_stride + (a.gqa ? (head << a.req_shift) : head) * hd;
+  wk.head_dim = hd;
   wk.pair_half = (a.req_shift && !a.gqa) ? 2 : -1;
   wk.gshift = a.gqa ? a.req_shift : 0;
   wk.q_stride = a.q_stride;
@@ -957,11 +969,12 @@ __device__ __forceinline__ void prefix_unit8(const PrefixArgs& a, int split, int
     const int64_t pr = ((int64_t)split * a.B + qbase + q) * a.H + head;
 #pragma unroll
     for (int nd = 0; nd < NDB; ++nd) {
-      float* op = a.opart + pr * kPD + 32 * (NDB * tq + nd) + 4 * h;
+      const int d0 = 32 * (NDB * tq + nd) + 4 * h;
+      float* op = a.opart + pr * hd + d0;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         float4_t v = {of[nd][4 * j] * inv, of[nd][4 * j + 1] * inv, of[nd][4 * j + 2] * inv, of[nd][4 * j + 3] * inv};
-        *reinterpret_cast<float4_t*>(op + 8 * j) = v;
+        if (d0 + 8 * j < hd) *reinterpret_cast<float4_t*>(op + 8 * j) = v;  // (a short head's row is hd floats long)
       }
     }
     if (h == 0 && tq == 0) {
@@ -1083,7 +1096,9 @@ __device__ __forceinline__ void prefill_tile8(const PrefillArgs& a, int tile_row
   const int q0 = (ti - a.tile_cu[lo]) * QT;
   const int nq = min(QT, n - q0);
   TileWork wk;
-  wk.qrow0 = a.q + (int64_t)(cq0 + q0) * a.q_stride + (a.pair ? (int)blockIdx.x * 64 : head * kPD);
+  const int hd = a.head_dim ? a.head_dim : kPD;  // 80 / 96 / 112: a short head on the 128-wide tile
+  wk.qrow0 = a.q + (int64_t)(cq0 + q0) * a.q_stride + (a.pair ? (int)blockIdx.x * 64 : head * hd);
+  wk.head_dim = a.pair ? kPD : hd;
   wk.pair_half = half;
   wk.q_stride = a.q_stride;
   wk.nq = nq;
@@ -1107,12 +1122,12 @@ __device__ __forceinline__ void prefill_tile8(const PrefillArgs& a, int tile_row
       if (a.pair && (db >> 1) != half) continue;  // the other half holds the neighbouring head's values: dropped
       // paired: head 2 * pair + half, dims 32 * (db & 1) ..; else head, dims 32 * db ..
       uint16_t* op = a.out + (int64_t)(cq0 + q0 + q) * a.out_stride +
-                     (a.pair ? (int)blockIdx.x * 64 + 32 * (db & 1) : head * kPD + 32 * db) + 4 * h;
+                     (a.pair ? (int)blockIdx.x * 64 + 32 * (db & 1) : head * hd + 32 * db) + 4 * h;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         u32x2 v = {pack2<E>(of[nd][4 * j] * inv, of[nd][4 * j + 1] * inv),
                    pack2<E>(of[nd][4 * j + 2] * inv, of[nd][4 * j + 3] * inv)};
-        *reinterpret_cast<u32x2*>(op + 8 * j) = v;
+        if (a.pair || 32 * db + 4 * h + 8 * j < hd) *reinterpret_cast<u32x2*>(op + 8 * j) = v;
       }
     }
   }
@@ -1159,7 +1174,7 @@ static void launch_prefix8(const PrefixArgs& a, int num_groups, int max_group_re
 template <typename E>
 static int launch_prefix_t(const PrefixArgs& a, int num_groups, int max_group_reqs, bool internal_ml, hipStream_t st,
                            const KernelEvents& ev) {
-  if (max_group_reqs <= 32 && a.req_shift == 0) {  // four waves, one 32-query block
+  if (max_group_reqs <= 32 && a.req_shift == 0 && (a.head_dim == 0 || a.head_dim == kPD)) {  // four waves, one 32-query block
     dim3 grid(a.n_splits, a.H, num_groups), block(256);
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefix_mfma_kernel<E, 1>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, tile_lds_bytes<1>());
@@ -1259,19 +1274,26 @@ int launch_decode_fused(const PrefixArgs& a, const ItemArgs& ia, int dtype, int 
                          : launch_fused_t<BF16, kPD>(a, ia, num_groups, max_group_reqs, cus, prefix_wgs, st, ev);
 }
 
-bool prefix_mfma_supported(int dtype, int D) { return D == kPD && (dtype == PH_F16 || dtype == PH_BF16); }
+// head size 128, and 80 / 96 / 112 as short heads on the 128-wide tile (TileWork::head_dim)
+bool prefix_mfma_supported(int dtype, int D) {
+  return (D == kPD || D == 112 || D == 96 || D == 80) && (dtype == PH_F16 || dtype == PH_BF16);
+}
 
-int launch_prefix_mfma(const PrefixArgs& a, int dtype, int D, int num_groups, int max_group_reqs, bool internal_ml,
+int launch_prefix_mfma(const PrefixArgs& a0, int dtype, int D, int num_groups, int max_group_reqs, bool internal_ml,
                        hipStream_t st, const KernelEvents& ev) {
-  if (D != kPD) return PH_ERR_HEAD_DIM;
-  if (num_groups <= 0 || max_group_reqs <= 0 || a.n_splits <= 0) return PH_OK;
+  if (!prefix_mfma_supported(dtype, D)) return PH_ERR_HEAD_DIM;
+  if (num_groups <= 0 || max_group_reqs <= 0 || a0.n_splits <= 0) return PH_OK;
+  PrefixArgs a = a0;
+  a.head_dim = D;
   return dtype == PH_F16 ? launch_prefix_t<F16>(a, num_groups, max_group_reqs, internal_ml, st, ev)
                          : launch_prefix_t<BF16>(a, num_groups, max_group_reqs, internal_ml, st, ev);
 }
 
-int launch_prefill_mfma(const PrefillArgs& a, int dtype, int D, int64_t num_tokens, hipStream_t st) {
-  if (D != kPD) return PH_ERR_HEAD_DIM;
-  if (num_tokens <= 0 || a.num_chunks <= 0) return PH_OK;
+int launch_prefill_mfma(const PrefillArgs& a0, int dtype, int D, int64_t num_tokens, hipStream_t st) {
+  if (!prefix_mfma_supported(dtype, D)) return PH_ERR_HEAD_DIM;
+  if (num_tokens <= 0 || a0.num_chunks <= 0) return PH_OK;
+  PrefillArgs a = a0;
+  a.head_dim = a.pair ? kPD : D;
   return dtype == PH_F16 ? launch_prefill_t<F16>(a, num_tokens, st) : launch_prefill_t<BF16>(a, num_tokens, st);
 }
 

@@ -219,6 +219,23 @@ def test_other_head_sizes_and_odd_head_counts(dev, D, H):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("D", [80, 96, 112])
+def test_short_heads_on_the_wide_prefix_tile(dev, D, dtype):
+    """Head sizes 80 / 96 / 112: the prefix phase on the matrix cores as short heads on the 128-wide tile (their
+    padding lanes re-read the row's first chunk, the query's padding dims are zero, the partial rows are D floats
+    long), in every query-tile form (groups of 20, 70, 150 and 300 requests), several groups, a prefix longer than
+    one split; the suffix phase per request at the head's own size."""
+    from parrotserve_amd import synth
+
+    for sizes, P, H in (([20], 300, 5), ([70, 33], 700, 3), ([150], 1300, 2), ([300, 9], 520, 2)):
+        g = torch.Generator().manual_seed(600 + D + sizes[0])
+        s = torch.randint(0, 60, (sum(sizes),), generator=g).tolist()
+        case = synth.make_decode_case("sh", 600 + D + sizes[0], dtype, len(sizes), 0, P, s, H, D, 1 << 15,
+                                      group_sizes=sizes)
+        _check(case, dev)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("D", [64, 80, 96, 112, 128, 256])
 def test_vllm_test_distribution_over_head_sizes(dev, D, dtype):
     """The vendored vLLM kernel test's inputs (3rdparty/vllm/tests/kernels/test_attention.py:159-246): q, k, v uniform

@@ -142,8 +142,9 @@ def test_prefill_heads_not_multiple_of_eight_and_tail_tiles(dev):
 
 @pytest.mark.parametrize("D,H", [(64, 6), (64, 5), (256, 2), (80, 5), (96, 3), (112, 2)])
 def test_prefill_other_head_sizes(dev, D, H):
-    """Head sizes the matrix-core kernel does not cover run every query row through the per-request kernel
-    over its visible slots; same results."""
+    """The other head sizes the reference dispatches: 80, 96 and 112 run on the matrix-core kernel as short heads
+    on its 128-wide tile, 64 on head pairs (even head counts); 256 and 64 with an odd head count run every query
+    row through the per-request kernel over its visible slots.  Same results."""
     from parrotserve_amd import synth
 
     case = synth.make_prefill_case("hd", 300 + D, torch.float16, [33, 5, 70], 41, H, D, 1 << 12)
@@ -169,6 +170,20 @@ def test_randomized_prefill_shapes(dev, seed, D):
     case = synth.make_prefill_case("rnd", 2000 + seed, dtype, q_lens, ri(0, 700), ri(1, 6), D, 1 << 13)
     out, ref = run_prefill_case(case, dev)
     torch.testing.assert_close(out.float(), ref.float(), **TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("D", [80, 96, 112])
+def test_prefill_short_heads_on_the_wide_tile(dev, D, dtype):
+    """Head sizes 80 / 96 / 112 on the 128-wide matrix-core tile, every query-tile form (chunks averaging 270, 130
+    and 40 tokens), partial tiles on both axes, parents longer than a tile; the last head of the last slot row
+    included (its padding lanes must stay inside the pool)."""
+    from parrotserve_amd import synth
+
+    for q_lens, parent, H in (([300, 240], 600, 3), ([129, 131], 257, 5), ([33, 64, 20, 41], 90, 2)):
+        case = synth.make_prefill_case("sh", 500 + D + H, dtype, q_lens, parent, H, D, 1 << 11)
+        out, ref = run_prefill_case(case, dev)
+        torch.testing.assert_close(out.float(), ref.float(), **TOL[dtype])
 
 
 def test_more_tile_rows_than_the_grid_holds(dev):
