@@ -865,6 +865,8 @@ def main():
     if args.timeline:  # before the first load(): this run binds the profiling variant of the library
         from parrotserve_amd import build as _build
 
+        if not os.path.exists(_build.TIMELINE_LIB_PATH):  # the profiling variant is only built when asked for
+            _build.build(verbose=False, timeline=True)
         _lib.LIB_PATH = _build.TIMELINE_LIB_PATH
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
