@@ -249,9 +249,11 @@ size_t ph_decode_workspace_bytes(int64_t num_reqs, int64_t num_heads, int64_t he
  * suffix phases of a call in one launch with workgroups of their own (16-bit
  * elements, head size 128 or paired 64, a suffix that moves about as many
  * bytes as the prefixes or more): there the prefix keeps the compute units a
- * cost model gives it and the suffix takes the rest.  A plan cut into more or
- * fewer pieces stays correct (pieces beyond one round are taken in further
- * rounds by the same waves); it is only slower.  Host-only, no launch.  The
+ * cost model gives it and the suffix takes the rest.  A plan cut into another
+ * number of pieces stays correct: with more pieces than that (a plan cut for
+ * the whole device) the call runs both phases in every workgroup
+ * instead, as it does for a short suffix; with fewer, waves idle.  Host-only,
+ * no launch.  The
  * reference has no counterpart (fixed (request, block) grids,
  * attention_post_kernels.cu:395-418). */
 int64_t ph_decode_suffix_lanes(int64_t num_reqs, int64_t num_heads, int64_t head_dim, int dtype,

@@ -452,8 +452,19 @@ static int decode_attention_impl(void* out, const void* q, const void* k_cache, 
   const bool mfma_prefix = kv.map ? gshift > 0 : (paired || prefix_mfma_supported(dtype, D));
   const bool roles = mfma_prefix && roles_possible(num_reqs, num_heads, head_dim, dtype, has_prefix, has_suffix,
                                                    planned, chunk_tokens);
-  const DecodePlan p = plan_decode(num_reqs, num_heads, has_prefix ? num_groups : 0, max_prefix_len, max_suffix_len,
-                                   chunk_tokens, planned ? plan->num_items : 0, head_dim, pair_heads(D, H), roles);
+  DecodePlan p = plan_decode(num_reqs, num_heads, has_prefix ? num_groups : 0, max_prefix_len, max_suffix_len,
+                             chunk_tokens, planned ? plan->num_items : 0, head_dim, pair_heads(D, H), roles);
+  if (planned && p.prefix_wgs > 0) {
+    // A caller's plan cut into more pieces than the suffix-only workgroups have waves (a plan made for the whole
+    // device: ph_decode_suffix_lanes was not asked, or for another shape) would take them a second round (config 2
+    // with 170 pieces for 160 workgroups: 93 us against 66 us): such a plan gets the form it was cut for, every
+    // workgroup running both phases (75 us).
+    const int64_t hpw = std::max(1, 64 / lanes_per_head(D));
+    const int64_t fit = ((int64_t)device_cus() - p.prefix_wgs) * 8 / cdiv(H, hpw);
+    if (plan->num_lanes > fit)
+      p = plan_decode(num_reqs, num_heads, num_groups, max_prefix_len, max_suffix_len, chunk_tokens, plan->num_items,
+                      head_dim, pair_heads(D, H), false);
+  }
   if (plan_bytes(p, B, H, D) > workspace_bytes || ((p.parts() > 0 || p.items > 0) && !workspace))
     return PH_ERR_WORKSPACE;
   if (((uintptr_t)workspace & 255u) != 0) return PH_ERR_ALIGN;
