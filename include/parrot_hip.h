@@ -247,12 +247,13 @@ size_t ph_decode_workspace_bytes(int64_t num_reqs, int64_t num_heads, int64_t he
  * per SIMD, on the compute units the suffix phase runs on.  That is every
  * compute unit of the device, except where the library runs the prefix and
  * suffix phases of a call in one launch with workgroups of their own (16-bit
- * elements, head size 128 or paired 64, a suffix that moves about as many
- * bytes as the prefixes or more): there the prefix keeps the compute units a
+ * elements, head size 128 or paired 64, and a shape for which the library's
+ * cost estimate favours that form: most, except prefixes that want the whole
+ * device): there the prefix keeps the compute units a
  * cost model gives it and the suffix takes the rest.  A plan cut into another
  * number of pieces stays correct: with more pieces than that (a plan cut for
  * the whole device) the call runs both phases in every workgroup
- * instead, as it does for a short suffix; with fewer, waves idle.  Host-only,
+ * instead; with fewer, waves idle.  Host-only,
  * no launch.  The
  * reference has no counterpart (fixed (request, block) grids,
  * attention_post_kernels.cu:395-418). */

@@ -66,45 +66,50 @@ static int device_cus() {
   return cached[dev];
 }
 
-// How the fused launch divides the compute units (see decode_fused_kernel): a suffix that moves at least half as
-// many bytes as the prefixes (and 64 MB) gets workgroups of its own (roles), a shorter one rides inside the prefix
-// workgroups (shared); measured at batch 64 over 4096- and 8192-token prefixes, roles win from there on (by 11 %
-// at half the prefix's bytes over 8192 tokens, a tie at equal bytes over 4096) and lose below.  The suffix volume
-// is an estimate from what the host knows -- half the longest list per request.
+// What the planner knows of a decode call's two phases.  The suffix volume is an estimate from what the host
+// knows -- half the longest list per request.
 struct FusedShape {
   int64_t units_per_split;  // prefix units (head x group x query tile) per split of the prefix
+  int64_t reqs, head_groups;  // requests; waves that one suffix piece occupies (heads / heads per wave)
+  int64_t group_rows, query_tile;  // query rows of a group as the matrix-core kernel sees them; its tile: 64 / 128 / 256
   double prefix_mb, suffix_mb;
-  bool roles;
 };
 static FusedShape fused_shape(int64_t B, int64_t H, int64_t D, int64_t groups, int64_t max_prefix, int64_t max_suffix,
                               bool paired) {
   FusedShape f{};
   if (groups <= 0 || max_prefix <= 0) return f;
   const int64_t rows_b = paired ? 2 * B : B, rows_h = paired ? H / 2 : H;  // what the matrix-core kernel sees
-  const int64_t per_group = cdiv(rows_b, groups);
-  const int64_t qtile = per_group <= 64 ? 64 : per_group <= 128 ? 128 : 256;
-  const int64_t mtiles = cdiv(per_group, qtile);
+  f.group_rows = cdiv(rows_b, groups);
+  f.query_tile = f.group_rows <= 64 ? 64 : f.group_rows <= 128 ? 128 : 256;
+  const int64_t mtiles = cdiv(f.group_rows, f.query_tile);
   f.units_per_split = groups * rows_h * (mtiles > 0 ? mtiles : 1);
+  f.reqs = B;
+  f.head_groups = cdiv(H, std::max(1, 64 / lanes_per_head((int)D)));
   const double row_mb = (double)H * D * 4 / 1e6;  // K and V of one token, 16-bit elements
   f.prefix_mb = (double)groups * max_prefix * row_mb;
   f.suffix_mb = (double)B * max_suffix / 2 * row_mb;
-  f.roles = f.suffix_mb >= 64.0 && f.suffix_mb >= 0.5 * f.prefix_mb;
   return f;
 }
+
+constexpr double kHbmMbPerUs = 6.9;  // what the device sustains on this access mix
 
 // Roles: the split count and the number of prefix-only workgroups.  A prefix workgroup is latency-bound next to
 // the suffix stream -- one 128-token step (64 KB) in flight ahead of the one it multiplies, about 2.7 us per step
 // with the memory system saturated, 12 us from launch to its first step -- so the prefix wants enough workgroups
 // to be done a little before the stream, and the stream wants the rest (it holds about 40 GB/s per compute unit).
+// A suffix wave spends about 4 us per piece before it streams (slot ids, then rows, then the partial's write), and
+// a lane walks at least requests / lanes pieces: with many short lists on few lanes that, not the bytes, is what
+// the suffix workgroups take (256 requests x 16 tokens on 32 lanes: 69 us; on 64 lanes: 54.5 us).
 // Both end no earlier than the bytes of the launch take at the rate the device sustains.
 struct RoleChoice {
   int splits, prefix_wgs;
+  double cost_us;
 };
 static RoleChoice choose_roles(const FusedShape& f, int64_t max_prefix, int64_t cus) {
-  constexpr double kHbm = 6.9, kCu = 0.040;  // MB per us: the device under this access mix, one compute unit streaming
-  constexpr double kStep = 2.7, kFirst = 12.0, kFold = 2.0, kNext = 6.0, kMargin = 3.0;
+  constexpr double kHbm = kHbmMbPerUs, kCu = 0.040;  // MB per us: the device, one compute unit streaming
+  constexpr double kStep = 2.7, kFirst = 12.0, kFold = 2.0, kNext = 6.0, kMargin = 3.0, kPiece = 4.0;
   const double floor_us = 4.0 + (f.prefix_mb + f.suffix_mb) / kHbm;
-  RoleChoice best{1, 1};
+  RoleChoice best{1, 1, 0.0};
   double best_cost = -1.0;
   const int64_t max_splits = std::max<int64_t>(1, cdiv(max_prefix, 4 * kPrefixTile));
   for (int64_t s = 1; s <= 64 && s <= max_splits; ++s) {
@@ -116,15 +121,54 @@ static RoleChoice choose_roles(const FusedShape& f, int64_t max_prefix, int64_t 
       const int64_t np = cdiv(units, r);
       if (np > cus - 1) continue;
       const double t_prefix = kFirst + r * (steps * kStep + kFold) + (r - 1) * kNext + kMargin;
-      const double t_suffix = 6.0 + f.suffix_mb / std::min(kHbm, (double)(cus - np) * kCu);
+      const int64_t lanes = std::max<int64_t>(1, (cus - np) * 8 / f.head_groups);
+      const double t_suffix =
+          6.0 + (double)cdiv(f.reqs, lanes) * kPiece + f.suffix_mb / std::min(kHbm, (double)(cus - np) * kCu);
       const double cost = std::max(std::max(t_prefix, t_suffix), floor_us) + 0.25 * s;
       if (best_cost < 0 || cost < best_cost) {
         best_cost = cost;
-        best = RoleChoice{(int)s, (int)np};
+        best = RoleChoice{(int)s, (int)np, cost};
       }
     }
   }
   return best;
+}
+
+// The other form: every workgroup runs both phases, its suffix pieces first (groups of over 32 rows; smaller ones
+// take a prefix launch on the four-wave tile, then the suffix launch) -- the phases one after the other, each on
+// every compute unit.  Split count: one workgroup per compute unit at a time (the kernel uses most of the register
+// file), so the count whose workgroup total wastes the least of a whole number of rounds over the device, at
+// rounds x (tokens per split + a fixed prologue / epilogue worth ~96 tokens).  cost_us in the units of
+// choose_roles' cost, less what that overstates a lightly loaded launch by (its 12 us to the first step and 2.7 us
+// per step are what a prefix workgroup sees next to a saturating stream): fitted, with the step time of this form
+// (3.1 us; x 1.44 on the 256-query tile, x 0.87 on the four-wave tile), to 106 shapes measured in both forms --
+// 1 .. 16 groups of 1 .. 256 requests, prefixes of 128 .. 16384 tokens, suffixes of up to 8 .. 4096 tokens, 32 and
+// 40 heads of 128.  Choosing by the two costs is within 0.3 % of the better form on average over those shapes and
+// 9 % at worst; the two phases in workgroups of their own win by 3 .. 25 % on most (small launches are chains of
+// memory latencies, which then run side by side: 16 requests x 256 over 1024 tokens 19.3 against 25.6 us; the
+// reference benchmark's 64 x 20 over 8192 at 40 heads 49.3 against 52.6 us) and lose by 3 .. 19 % where the prefix
+// wants every compute unit: long prefixes under tiny suffixes, 256-query tiles under short suffixes, and many
+// small groups whose units fill the device evenly (8 groups of 8 over 2000 tokens: 77 against 66 us).
+struct SharedChoice {
+  int splits;
+  double cost_us;
+};
+static SharedChoice choose_shared(const FusedShape& f, int64_t max_prefix, int64_t cus) {
+  const int64_t max_splits = std::max<int64_t>(1, cdiv(max_prefix, 4 * kPrefixTile));
+  int64_t splits = 1, best = -1;
+  for (int64_t s = 1; s <= 64 && s <= max_splits; ++s) {
+    const int64_t tok = round_up(cdiv(max_prefix, s), 2 * kPrefixTile);
+    const int64_t cost = cdiv(f.units_per_split * s, cus) * (tok + 96);
+    if (best < 0 || cost < best) {
+      best = cost;
+      splits = s;
+    }
+  }
+  const int64_t tok = round_up(cdiv(max_prefix, splits), 2 * kPrefixTile);
+  const double steps = (double)cdiv(tok, 2 * kPrefixTile), rounds = (double)cdiv(f.units_per_split * cdiv(max_prefix, tok), cus);
+  const double step_us = 3.1 * (f.query_tile == 256 ? 1.44 : 1.0) * (f.group_rows <= 32 ? 0.87 : 1.0);
+  const double t = 9.3 + f.suffix_mb / kHbmMbPerUs + rounds * (steps * step_us + 2.0);
+  return SharedChoice{(int)splits, std::max(t, 4.0 + (f.prefix_mb + f.suffix_mb) / kHbmMbPerUs) + 11.5};
 }
 
 // plan_head_dim > 0: a caller without a plan of its own that leaves the chunk size to the library gets the
@@ -139,24 +183,13 @@ static DecodePlan plan_decode(int64_t B, int64_t H, int64_t groups, int64_t max_
   if (groups > 0 && max_prefix > 0) {
     p.paired = paired;
     const FusedShape f = fused_shape(B, H, plan_head_dim > 0 ? plan_head_dim : 128, groups, max_prefix, max_suffix, paired);
-    int64_t splits = 1;
-    if (roles && f.roles && max_suffix > 0) {
+    const SharedChoice sc = choose_shared(f, max_prefix, cus);
+    int64_t splits = sc.splits;
+    if (roles && max_suffix > 0) {
       const RoleChoice rc = choose_roles(f, max_prefix, cus);
-      splits = rc.splits;
-      p.prefix_wgs = rc.prefix_wgs;
-    } else {
-      // One workgroup per CU at a time (the kernel uses most of the register file), so pick the
-      // split count whose workgroup total wastes the least of a whole number of rounds over the device's CUs.
-      // Cost model: rounds x (tokens per split + a fixed prologue/epilogue worth ~96 tokens).
-      const int64_t max_splits = cdiv(max_prefix, 4 * kPrefixTile);
-      int64_t best = -1;
-      for (int64_t s = 1; s <= 64 && s <= (max_splits > 0 ? max_splits : 1); ++s) {
-        const int64_t tok = round_up(cdiv(max_prefix, s), 2 * kPrefixTile);
-        const int64_t cost = cdiv(f.units_per_split * s, cus) * (tok + 96);
-        if (best < 0 || cost < best) {
-          best = cost;
-          splits = s;
-        }
+      if (rc.cost_us < sc.cost_us) {
+        splits = rc.splits;
+        p.prefix_wgs = rc.prefix_wgs;
       }
     }
     const int64_t st = round_up(cdiv(max_prefix, splits), 2 * kPrefixTile);

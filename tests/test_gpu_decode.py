@@ -97,7 +97,8 @@ def _role_split(dev, case):
     cus = torch.cuda.get_device_properties(dev).multi_processor_count
     lanes = kernels.suffix_lane_capacity(dev, H, D, num_reqs=B, num_groups=len(case.prefix_lists), max_prefix_len=P,
                                          max_suffix_len=S, dtype=case.dtype)
-    hgroups = (H + 3) // 4
+    heads_per_wave = 4 if D > 64 else 8  # a head takes D / 8 lanes of a wave, rounded up to a power of two
+    hgroups = (H + heads_per_wave - 1) // heads_per_wave
     return cus - (lanes * hgroups + 7) // 8, cus
 
 
@@ -123,6 +124,22 @@ def test_prefix_and_suffix_workgroups_of_their_own(dev, dtype):
         tables.plan_on_device(lanes, dev)
         other = kernels.decode_attention(case.q.to(dev), kc, vc, tables).cpu()
         torch.testing.assert_close(other.float(), out.float(), **TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype,H,D", [(torch.float16, 8, 128), (torch.bfloat16, 8, 128), (torch.float16, 16, 64)])
+def test_every_workgroup_runs_both_phases_when_the_launch_is_all_prefix(dev, dtype, H, D):
+    """A long prefix under a handful of own tokens per request: the prefix wants every compute unit, so the library
+    keeps the launch in which each workgroup streams its suffix pieces and then runs a prefix unit (no prefix-only
+    workgroups: the lane count it asks for is the whole device's)."""
+    from parrotserve_amd import synth
+
+    g = torch.Generator().manual_seed(25)
+    s = torch.randint(0, 9, (64,), generator=g).tolist()
+    s[5] = 8
+    case = synth.make_decode_case("allprefix", 25, dtype, 1, 64, 8192, s, H, D, 1 << 15)
+    np_, cus = _role_split(dev, case)
+    assert np_ == 0, "this shape is meant to take the launch whose workgroups run both phases"
+    _check(case, dev)
 
 
 def test_prefix_workgroups_walk_several_units_each(dev):
@@ -500,12 +517,13 @@ def test_timed_call_is_the_same_call_with_timestamps(dev):
         return ms.value
 
     g = torch.Generator().manual_seed(77)
-    for B, expect_prefix_pair in ((64, False), (16, True)):  # 64 requests: one launch for both phases; 16: two
+    # head size 128: one launch for both phases; 96 (a short head on the wide tile): a prefix launch of its own
+    for B, D, expect_prefix_pair in ((64, 128, False), (16, 128, False), (16, 96, True)):
         s = torch.randint(1, 150, (B,), generator=g).tolist()
-        case = synth.make_decode_case("t", 500 + B, torch.float16, 1, B, 700, s, 8, 128, 1 << 14)
+        case = synth.make_decode_case("t", 500 + B, torch.float16, 1, B, 700, s, 8, D, 1 << 14)
         kc, vc = synth.pool_to_device(case.k_rows, case.v_rows, case.used_slots, case.pool_slots, dev)
         tables = kernels.DecodeTables.build(case.pool_lists(case.prefix_lists), case.group_req_cu,
-                                            case.pool_lists(case.suffix_lists), dev, num_heads=8, head_dim=128)
+                                            case.pool_lists(case.suffix_lists), dev, num_heads=8, head_dim=D)
         q = case.q.to(dev)
         plain = kernels.decode_attention(q, kc, vc, tables)
         evs = (ctypes.c_void_p * 6)()
@@ -906,7 +924,7 @@ def test_captured_decode_step_replays_while_contexts_grow(dev):
     spare = [s for s in range(case.pool_slots) if s not in used][: 6 * B]
     tables = kernels.DecodeTables.build(prefix, case.group_req_cu, suffix, dev, num_heads=H, head_dim=D)
     table_cache._widen(tables, max(lens) + 8, dev)          # room for the tokens to come
-    lanes = kernels.suffix_lane_capacity(dev, H, D)
+    lanes = tables.plan.num_lanes                           # the recorded launch is shaped for this many pieces
     q_static = case.q.to(dev)
     out_static = torch.empty_like(q_static)
     side = torch.cuda.Stream()
