@@ -138,10 +138,11 @@ static RoleChoice choose_roles(const FusedShape& f, int64_t max_prefix, int64_t 
 // take a prefix launch on the four-wave tile, then the suffix launch) -- the phases one after the other, each on
 // every compute unit.  Split count: one workgroup per compute unit at a time (the kernel uses most of the register
 // file), so the count whose workgroup total wastes the least of a whole number of rounds over the device, at
-// rounds x (tokens per split + a fixed prologue / epilogue worth ~96 tokens).  cost_us in the units of
-// choose_roles' cost, less what that overstates a lightly loaded launch by (its 12 us to the first step and 2.7 us
-// per step are what a prefix workgroup sees next to a saturating stream): fitted, with the step time of this form
-// (3.1 us; x 1.44 on the 256-query tile, x 0.87 on the four-wave tile), to 106 shapes measured in both forms --
+// rounds x (tokens per split + a fixed prologue / epilogue worth ~96 tokens).  cost_us is on the scale of
+// choose_roles' cost, which overstates a lightly loaded launch (its 12 us to the first step and 2.7 us per step are
+// what a prefix workgroup sees next to a saturating stream): the estimate of this form's time plus 11.5 us, that
+// offset fitted, with the step time of this form (3.1 us; x 1.44 on the 256-query tile, x 0.87 on the four-wave
+// tile) and its 9.3 us of start and end, to 106 shapes measured in both forms --
 // 1 .. 16 groups of 1 .. 256 requests, prefixes of 128 .. 16384 tokens, suffixes of up to 8 .. 4096 tokens, 32 and
 // 40 heads of 128.  Choosing by the two costs is within 0.3 % of the better form on average over those shapes and
 // 9 % at worst; the two phases in workgroups of their own win by 3 .. 25 % on most (small launches are chains of
@@ -168,7 +169,8 @@ static SharedChoice choose_shared(const FusedShape& f, int64_t max_prefix, int64
   const double steps = (double)cdiv(tok, 2 * kPrefixTile), rounds = (double)cdiv(f.units_per_split * cdiv(max_prefix, tok), cus);
   const double step_us = 3.1 * (f.query_tile == 256 ? 1.44 : 1.0) * (f.group_rows <= 32 ? 0.87 : 1.0);
   const double t = 9.3 + f.suffix_mb / kHbmMbPerUs + rounds * (steps * step_us + 2.0);
-  return SharedChoice{(int)splits, std::max(t, 4.0 + (f.prefix_mb + f.suffix_mb) / kHbmMbPerUs) + 11.5};
+  constexpr double kRolesScale = 11.5;
+  return SharedChoice{(int)splits, std::max(t, 4.0 + (f.prefix_mb + f.suffix_mb) / kHbmMbPerUs) + kRolesScale};
 }
 
 // plan_head_dim > 0: a caller without a plan of its own that leaves the chunk size to the library gets the
