@@ -253,12 +253,19 @@ size_t ph_decode_workspace_bytes(int64_t num_reqs, int64_t num_heads, int64_t he
  * cost model gives it and the suffix takes the rest.  A plan cut into another
  * number of pieces stays correct: with more pieces than that (a plan cut for
  * the whole device) the call runs both phases in every workgroup
- * instead; with fewer, waves idle.  Host-only,
+ * instead; with fewer, waves idle.  kv_group: 1 (or 0) for a plain call; G for
+ * a ph_decode_attention_gqa call that will state kv_group = G -- the planner
+ * then counts the K/V bytes and matrix rows of that call, and with G a power of
+ * two from 4 on (head size 128, 16-bit elements) and lists long enough to gain
+ * from it the suffix waves stream every token row for four query heads of its
+ * KV head at once, so a piece occupies a quarter of the waves and the device
+ * takes four times the pieces.  Host-only,
  * no launch.  The
  * reference has no counterpart (fixed (request, block) grids,
  * attention_post_kernels.cu:395-418). */
 int64_t ph_decode_suffix_lanes(int64_t num_reqs, int64_t num_heads, int64_t head_dim, int dtype,
-                               int64_t num_groups, int64_t max_prefix_len, int64_t max_suffix_len);
+                               int64_t num_groups, int64_t max_prefix_len, int64_t max_suffix_len,
+                               int64_t kv_group);
 
 int ph_decode_attention(void* out, const void* q, const void* k_cache, const void* v_cache,
                         int64_t num_reqs, int64_t num_heads, int64_t head_dim, int dtype,

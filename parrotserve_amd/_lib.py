@@ -32,7 +32,7 @@ SIGNATURES: Dict[str, Tuple[object, List[object]]] = {
     "ph_rope_neox": (I, [P, P, P, P, L, L, L, L, L, L, L, I, P]),
     "ph_rotary_embedding": (I, [P, P, P, L, L, L, L, L, L, I, P]),
     "ph_decode_workspace_bytes": (Z, [L, L, L, L, L, L, L, L]),
-    "ph_decode_suffix_lanes": (L, [L, L, L, I, L, L, L]),
+    "ph_decode_suffix_lanes": (L, [L, L, L, I, L, L, L, L]),
     "ph_decode_attention": (I, [P, P, P, P, L, L, L, I, L, L, L, F, L, P, P, P, P, L, P, P, L, L, P, L, L, P, P, Z, P]),
     "ph_decode_attention_gqa": (I, [P, P, P, P, L, L, L, P, L, L, I, L, L, L, F, L, P, P, P, P, L, P, P, L, L, P, L, L, P, P, Z,
                                     P]),

@@ -66,6 +66,20 @@ static int device_cus() {
   return cached[dev];
 }
 
+// Query heads that share KV heads, as the planner sees them: mfma_group = G when the prefix phase runs the G query
+// heads of a KV head as G rows per request on H / G heads (1: plain), stream_group = query heads the suffix waves
+// stream together per KV head (grouped_stream_heads: G or 1).
+struct HeadGrouping {
+  int64_t mfma_group = 1;
+  int stream_group = 1;
+};
+
+// waves that one suffix piece occupies: the streamed heads (KV heads when their query heads go together) over the
+// heads a wave holds
+static int64_t suffix_head_groups(int64_t H, int64_t D, int stream_group) {
+  return cdiv(H / std::max(1, stream_group), std::max(1, 64 / lanes_per_head((int)D)));
+}
+
 // What the planner knows of a decode call's two phases.  The suffix volume is an estimate from what the host
 // knows -- half the longest list per request.
 struct FusedShape {
@@ -73,19 +87,25 @@ struct FusedShape {
   int64_t reqs, head_groups;  // requests; waves that one suffix piece occupies (heads / heads per wave)
   int64_t group_rows, query_tile;  // query rows of a group as the matrix-core kernel sees them; its tile: 64 / 128 / 256
   double prefix_mb, suffix_mb;
+  double stream_mb_per_us;  // what one compute unit of suffix waves streams
 };
 static FusedShape fused_shape(int64_t B, int64_t H, int64_t D, int64_t groups, int64_t max_prefix, int64_t max_suffix,
-                              bool paired) {
+                              bool paired, const HeadGrouping& hg = HeadGrouping()) {
   FusedShape f{};
   if (groups <= 0 || max_prefix <= 0) return f;
-  const int64_t rows_b = paired ? 2 * B : B, rows_h = paired ? H / 2 : H;  // what the matrix-core kernel sees
+  const int64_t G = std::max<int64_t>(1, hg.mfma_group);
+  // what the matrix-core kernel sees
+  const int64_t rows_b = paired ? 2 * B : B * G, rows_h = paired ? H / 2 : H / G;
   f.group_rows = cdiv(rows_b, groups);
   f.query_tile = f.group_rows <= 64 ? 64 : f.group_rows <= 128 ? 128 : 256;
   const int64_t mtiles = cdiv(f.group_rows, f.query_tile);
   f.units_per_split = groups * rows_h * (mtiles > 0 ? mtiles : 1);
   f.reqs = B;
-  f.head_groups = cdiv(H, std::max(1, 64 / lanes_per_head((int)D)));
-  const double row_mb = (double)H * D * 4 / 1e6;  // K and V of one token, 16-bit elements
+  f.head_groups = suffix_head_groups(H, D, hg.stream_group);
+  const double row_mb = (double)(H / G) * D * 4 / 1e6;  // K and V of one token, 16-bit elements
+  // 40 GB/s when every load instruction brings rows of its own; query heads that share a KV head re-read its rows
+  // (G loads per row), or, streamed together, meet each row with stream_group queries (bound by the vector ALUs)
+  f.stream_mb_per_us = hg.stream_group > 1 ? 0.096 / hg.stream_group : 0.040 / (double)G;
   f.prefix_mb = (double)groups * max_prefix * row_mb;
   f.suffix_mb = (double)B * max_suffix / 2 * row_mb;
   return f;
@@ -106,7 +126,8 @@ struct RoleChoice {
   double cost_us;
 };
 static RoleChoice choose_roles(const FusedShape& f, int64_t max_prefix, int64_t cus) {
-  constexpr double kHbm = kHbmMbPerUs, kCu = 0.040;  // MB per us: the device, one compute unit streaming
+  constexpr double kHbm = kHbmMbPerUs;  // MB per us
+  const double kCu = f.stream_mb_per_us;
   constexpr double kStep = 2.7, kFirst = 12.0, kFold = 2.0, kNext = 6.0, kMargin = 3.0, kPiece = 4.0;
   const double floor_us = 4.0 + (f.prefix_mb + f.suffix_mb) / kHbm;
   RoleChoice best{1, 1, 0.0};
@@ -178,13 +199,14 @@ static SharedChoice choose_shared(const FusedShape& f, int64_t max_prefix, int64
 // plain (request, chunk) grid.  roles: the fused launch may give the two phases workgroups of their own.
 static DecodePlan plan_decode(int64_t B, int64_t H, int64_t groups, int64_t max_prefix, int64_t max_suffix,
                               int64_t chunk_tokens, int64_t num_items = 0, int64_t plan_head_dim = 0,
-                              bool paired = false, bool roles = false) {
+                              bool paired = false, bool roles = false, const HeadGrouping& hg = HeadGrouping()) {
   DecodePlan p{};
   p.items = num_items;
   const int64_t cus = device_cus();
   if (groups > 0 && max_prefix > 0) {
     p.paired = paired;
-    const FusedShape f = fused_shape(B, H, plan_head_dim > 0 ? plan_head_dim : 128, groups, max_prefix, max_suffix, paired);
+    const FusedShape f =
+        fused_shape(B, H, plan_head_dim > 0 ? plan_head_dim : 128, groups, max_prefix, max_suffix, paired, hg);
     const SharedChoice sc = choose_shared(f, max_prefix, cus);
     int64_t splits = sc.splits;
     if (roles && max_suffix > 0) {
@@ -202,9 +224,8 @@ static DecodePlan plan_decode(int64_t B, int64_t H, int64_t groups, int64_t max_
     p.chunk = 32;
     p.n_chunks = 0;
   } else if (max_suffix > 0 && chunk_tokens <= 0 && plan_head_dim >= 8 && B <= kPlanMaxReqs) {
-    const int64_t heads_per_wave = 64 / lanes_per_head((int)plan_head_dim) > 0 ? 64 / lanes_per_head((int)plan_head_dim) : 1;
     // two waves per SIMD on the compute units the suffix phase has to itself
-    const int64_t lanes = (cus - p.prefix_wgs) * 4 * 2 / cdiv(H, heads_per_wave);
+    const int64_t lanes = (cus - p.prefix_wgs) * 4 * 2 / suffix_head_groups(H, plan_head_dim, hg.stream_group);
     p.dev_lanes = (int)(lanes > 0 ? lanes : 1);
     p.items = p.dev_lanes + B;  // capacity: a cut at every lane mark and every request boundary
     p.chunk = 32;
@@ -413,14 +434,42 @@ extern "C" size_t ph_decode_workspace_bytes(int64_t num_reqs, int64_t num_heads,
                                             int64_t chunk_tokens, int64_t num_items) {
   if (num_reqs <= 0 || num_heads <= 0 || head_dim <= 0) return 0;
   // the call picks one of two layouts (prefix and suffix workgroups of their own, or not) by what the element type
-  // and the group sizes allow, which this query does not see: large enough for either
+  // and the group sizes allow, and its split count and plan size follow how query heads share KV heads -- none of
+  // which this query sees: large enough for every case
   size_t need = 0;
-  for (int roles = 0; roles < 2; ++roles) {
-    const DecodePlan p = plan_decode(num_reqs, num_heads, num_groups, max_prefix_len, max_suffix_len, chunk_tokens,
-                                     num_items, head_dim, pair_heads(head_dim, num_heads), roles != 0);
-    need = std::max(need, plan_bytes(p, num_reqs, num_heads, head_dim));
+  for (int64_t group = 1; group <= 64 && group <= num_heads; group *= 2) {
+    if (num_heads % group != 0) break;
+    for (int stream = 0; stream < 2; ++stream) {
+      HeadGrouping hg;
+      hg.mfma_group = group;
+      hg.stream_group = stream ? grouped_stream_heads(group, (int)head_dim, PH_F16) : 1;  // whatever the lengths
+      if (stream && hg.stream_group == 1) continue;
+      for (int roles = 0; roles < 2; ++roles) {
+        const DecodePlan p = plan_decode(num_reqs, num_heads, num_groups, max_prefix_len, max_suffix_len, chunk_tokens,
+                                         num_items, head_dim, pair_heads(head_dim, num_heads), roles != 0, hg);
+        need = std::max(need, plan_bytes(p, num_reqs, num_heads, head_dim));
+      }
+    }
   }
   return need;
+}
+
+// How a call whose query heads share KV heads as h -> h / kv_group is planned: on the matrix cores with the group's
+// heads as rows (a power of two up to 64, head size 128, 16-bit elements; gqa_shift() is the call's own test) and,
+// where that form exists and the lists are long enough, with runs of the group streamed together in the suffix
+// phase.  Long enough: the grouped form cuts the suffix into four times the pieces (a piece occupies a quarter of
+// the waves), each with its ~4 us of start and its partial rows for the merge, so it wins from lists of ~100 tokens
+// and ~8000 tokens in all on (64 requests x 32 / 8 heads, <= 512 tokens over 4096: 41.7 against 49.8 us; four
+// groups of 32 x 64 / 8 heads, <= 1024 tokens over 6000: 134.5 against 195.6 us) and loses below (16 requests x
+// <= 256 tokens: 28.4 against 23.4 us; 256 x <= 128 tokens: 67.1 against 64.5 us).  kv_group <= 1: plain.
+static HeadGrouping head_grouping(int64_t kv_group, int64_t H, int64_t D, int dtype, int64_t B, int64_t max_suffix) {
+  HeadGrouping hg;
+  if (kv_group >= 2 && kv_group <= 64 && (kv_group & (kv_group - 1)) == 0 && D == 128 &&
+      prefix_mfma_supported(dtype, 128) && H % kv_group == 0) {
+    hg.mfma_group = kv_group;
+    if (max_suffix >= 200 && B * max_suffix / 2 >= 8000) hg.stream_group = grouped_stream_heads(kv_group, (int)D, dtype);
+  }
+  return hg;
 }
 
 // can the prefix and suffix phases of this call share one launch with workgroups of their own?
@@ -432,14 +481,18 @@ static bool roles_possible(int64_t B, int64_t H, int64_t D, int dtype, bool has_
 }
 
 extern "C" int64_t ph_decode_suffix_lanes(int64_t num_reqs, int64_t num_heads, int64_t head_dim, int dtype,
-                                          int64_t num_groups, int64_t max_prefix_len, int64_t max_suffix_len) {
+                                          int64_t num_groups, int64_t max_prefix_len, int64_t max_suffix_len,
+                                          int64_t kv_group) {
   if (num_reqs <= 0 || num_heads <= 0 || head_dim < 8) return 1;
   const bool has_prefix = num_groups > 0 && max_prefix_len > 0;
-  const bool roles = roles_possible(num_reqs, num_heads, head_dim, dtype, has_prefix, max_suffix_len > 0, true, 0);
+  const HeadGrouping hg = head_grouping(kv_group, num_heads, head_dim, dtype, num_reqs, max_suffix_len);
+  const bool mfma_prefix = kv_group <= 1 || hg.mfma_group > 1;  // another mapping runs every phase per request
+  const bool roles =
+      mfma_prefix && roles_possible(num_reqs, num_heads, head_dim, dtype, has_prefix, max_suffix_len > 0, true, 0);
   const DecodePlan p = plan_decode(num_reqs, num_heads, has_prefix ? num_groups : 0, max_prefix_len, max_suffix_len, 0,
-                                   1, head_dim, pair_heads(head_dim, num_heads), roles);
-  const int64_t heads_per_wave = std::max(1, 64 / lanes_per_head((int)head_dim));
-  const int64_t lanes = ((int64_t)device_cus() - p.prefix_wgs) * 4 * 2 / cdiv(num_heads, heads_per_wave);
+                                   1, head_dim, pair_heads(head_dim, num_heads), roles, hg);
+  const int64_t lanes =
+      ((int64_t)device_cus() - p.prefix_wgs) * 4 * 2 / suffix_head_groups(num_heads, head_dim, hg.stream_group);
   return lanes > 0 ? lanes : 1;
 }
 
@@ -487,18 +540,20 @@ static int decode_attention_impl(void* out, const void* q, const void* k_cache, 
   const bool mfma_prefix = kv.map ? gshift > 0 : (paired || prefix_mfma_supported(dtype, D));
   const bool roles = mfma_prefix && roles_possible(num_reqs, num_heads, head_dim, dtype, has_prefix, has_suffix,
                                                    planned, chunk_tokens);
+  // the planner's view of shared KV heads is the call's own: the same test as gqa_shift()
+  const HeadGrouping hg =
+      gshift > 0 ? head_grouping(kv.group, num_heads, head_dim, dtype, num_reqs, max_suffix_len) : HeadGrouping();
   DecodePlan p = plan_decode(num_reqs, num_heads, has_prefix ? num_groups : 0, max_prefix_len, max_suffix_len,
-                             chunk_tokens, planned ? plan->num_items : 0, head_dim, pair_heads(D, H), roles);
+                             chunk_tokens, planned ? plan->num_items : 0, head_dim, pair_heads(D, H), roles, hg);
   if (planned && p.prefix_wgs > 0) {
     // A caller's plan cut into more pieces than the suffix-only workgroups have waves (a plan made for the whole
     // device: ph_decode_suffix_lanes was not asked, or for another shape) would take them a second round (config 2
     // with 170 pieces for 160 workgroups: 93 us against 66 us): such a plan gets the form it was cut for, every
     // workgroup running both phases (75 us).
-    const int64_t hpw = std::max(1, 64 / lanes_per_head(D));
-    const int64_t fit = ((int64_t)device_cus() - p.prefix_wgs) * 8 / cdiv(H, hpw);
+    const int64_t fit = ((int64_t)device_cus() - p.prefix_wgs) * 8 / suffix_head_groups(H, D, hg.stream_group);
     if (plan->num_lanes > fit)
       p = plan_decode(num_reqs, num_heads, num_groups, max_prefix_len, max_suffix_len, chunk_tokens, plan->num_items,
-                      head_dim, pair_heads(D, H), false);
+                      head_dim, pair_heads(D, H), false, hg);
   }
   if (plan_bytes(p, B, H, D) > workspace_bytes || ((p.parts() > 0 || p.items > 0) && !workspace))
     return PH_ERR_WORKSPACE;
@@ -579,6 +634,8 @@ static int decode_attention_impl(void* out, const void* q, const void* k_cache, 
     ia.H = H;
     ia.scale_log2e = sl2;
     ia.head_map = kv.map;
+    ia.nq = hg.stream_group;
+    for (int64_t runs = hg.stream_group > 1 ? hg.mfma_group / hg.stream_group : 1; runs > 1; runs >>= 1) ++ia.kv_shift;
     rc = fuse ? launch_decode_fused(fused_pa, ia, dtype, fused_groups, fused_max_reqs, device_cus(), p.prefix_wgs, st,
                                       ev_suffix)
               : launch_items(ia, dtype, D, st, ev_suffix);

@@ -73,14 +73,15 @@ __global__ __launch_bounds__(256) void decode_partial_kernel(PartialArgs a) {
 // Balanced form: the host cut the batch's token stream into `num_lanes` near-equal pieces; a piece is
 // one or more items (request, first token, count) and is streamed by hgroups waves (one per HPW heads),
 // so every wave of the launch moves the same number of bytes and the launch is a single round.
-template <typename E, int D, int TB, int STAGES>
+// NQ > 1 (a.nq): the NQ query heads of a KV head go through one wave's lanes together (stream_item)
+template <typename E, int D, int TB, int STAGES, int NQ = 1>
 __global__ __launch_bounds__(256) void decode_items_kernel(ItemArgs a) {
   constexpr int HPW = HeadLanes<D>::HPW;
   const int wave = __builtin_amdgcn_readfirstlane(blockIdx.x * 4 + (threadIdx.x >> 6));
-  const int hgroups = (a.H + HPW - 1) / HPW;
+  const int hgroups = (a.H / NQ + HPW - 1) / HPW;
   const int piece = wave / hgroups;
   if (piece >= a.num_lanes) return;
-  run_piece<E, D, TB, STAGES>(a, piece, wave - piece * hgroups);
+  run_piece<E, D, TB, STAGES, NQ>(a, piece, wave - piece * hgroups);
 }
 
 // One workgroup per (request, HPW heads); its four waves fold every fourth part each
@@ -222,10 +223,18 @@ static int launch_partial_t(const PartialArgs& a, hipStream_t st, const KernelEv
 template <typename E, int D>
 static int launch_items_t(const ItemArgs& a, hipStream_t st, const KernelEvents& ev) {
   constexpr int HPW = HeadLanes<D>::HPW;
-  const int64_t hgroups = (a.H + HPW - 1) / HPW;
+  const int nq = a.nq > 1 ? a.nq : 1;
+  const int64_t hgroups = (a.H / nq + HPW - 1) / HPW;
   const int64_t waves = (int64_t)a.num_lanes * hgroups;
   if (waves == 0) return PH_OK;
   dim3 grid((unsigned)((waves + 3) / 4)), block(256);
+  if constexpr (D == 128 && !is_f32<E>::value) {
+    if (nq == 4) {
+      PH_LAUNCH_TIMED((decode_items_kernel<E, D, 4, 2, 4>), grid, block, 0, st, ev, a);
+      return launch_status();
+    }
+  }
+  if (nq != 1) return PH_ERR_ARG;  // grouped_stream_heads() says which shapes have the grouped form
   PH_LAUNCH_TIMED((decode_items_kernel<E, D, 4, 2>), grid, block, 0, st, ev, a);
   return launch_status();
 }

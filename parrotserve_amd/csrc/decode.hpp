@@ -51,7 +51,19 @@ struct ItemArgs {
   int H;
   float scale_log2e;
   const int32_t* head_map;     // KV head of each query head (device, [H]); null = identity
+  int nq;                      // > 1: runs of nq adjacent query heads are streamed together against the KV head they
+                               // share, the waves dividing the H / nq runs (head size 128, 16-bit); else 0 / 1
+  int kv_shift;                // nq > 1: run r reads KV head r >> kv_shift (query head h reads KV head h / (nq << kv_shift))
 };
+
+// Query heads streamed together in the balanced suffix form (ItemArgs.nq) where the form exists: 4 when the
+// mapping is the plain h / G with G a power of two from 4 on (a KV head's heads are G / 4 runs of 4) at head size 128
+// and 16-bit elements, else 1.  (Runs of 8 for G = 8 were measured slower than two runs of 4: 72 against 57 us at
+// 64 requests x 64 / 8 heads, suffixes of up to 512 tokens over a 4096-token prefix.)
+inline int grouped_stream_heads(int64_t kv_group, int D, int dtype) {
+  const bool pow2 = kv_group >= 4 && kv_group <= 64 && (kv_group & (kv_group - 1)) == 0;
+  return pow2 && D == 128 && (dtype == PH_F16 || dtype == PH_BF16) ? 4 : 1;
+}
 
 struct MergeArgs {
   const float* opart;

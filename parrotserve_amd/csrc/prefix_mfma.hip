@@ -1014,7 +1014,9 @@ struct WideTile {
 //
 // The merge stays a separate launch: it needs every part.
 // DS = head size of the suffix phase: 128, or 64 when the prefix phase runs on head pairs (pa.req_shift == 1).
-template <typename E, int TQ, int DS = kPD>
+// NQ > 1 (grouped KV heads, ia.nq): the suffix waves divide runs of NQ query heads that share a KV head and stream a
+// row for the run at once.
+template <typename E, int TQ, int DS = kPD, int NQ = 1>
 __global__ __launch_bounds__(512) void decode_fused_kernel(PrefixArgs pa, int mtiles, int n_units, int np,
                                                            ItemArgs ia) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -1022,7 +1024,7 @@ __global__ __launch_bounds__(512) void decode_fused_kernel(PrefixArgs pa, int mt
   constexpr bool PRESC = WideTile<TQ>::PRESC;
   PH_TL(0);
   constexpr int HPW = HeadLanes<DS>::HPW;
-  const int hgroups = (ia.H + HPW - 1) / HPW;
+  const int hgroups = (ia.H / NQ + HPW - 1) / HPW;
   const int slots = ia.num_lanes * hgroups;
   if (np > 0) {
     if ((int)blockIdx.x < np) {
@@ -1037,7 +1039,7 @@ __global__ __launch_bounds__(512) void decode_fused_kernel(PrefixArgs pa, int mt
       const int wave = __builtin_amdgcn_readfirstlane(((int)blockIdx.x - np) * 8 + (int)(threadIdx.x >> 6));
       for (int s = wave; s < slots; s += stride) {
         const int piece = s / hgroups;
-        run_piece<E, DS, 4, 2>(ia, piece, s - piece * hgroups);
+        run_piece<E, DS, 4, 2, NQ>(ia, piece, s - piece * hgroups);
       }
     }
     PH_TL(11);
@@ -1052,10 +1054,10 @@ __global__ __launch_bounds__(512) void decode_fused_kernel(PrefixArgs pa, int mt
     rec1 = ia.lane_rec[2 * piece0 + 1];
   }
   auto suffix = [&]() {
-    if (piece0 >= 0) run_piece_rec<E, DS, 4, 2>(ia, wave - piece0 * hgroups, rec0, rec1);
+    if (piece0 >= 0) run_piece_rec<E, DS, 4, 2, NQ>(ia, wave - piece0 * hgroups, rec0, rec1);
     for (int s = wave + gridDim.x * 8; s < slots; s += gridDim.x * 8) {
       const int piece = s / hgroups;
-      run_piece<E, DS, 4, 2>(ia, piece, s - piece * hgroups);
+      run_piece<E, DS, 4, 2, NQ>(ia, piece, s - piece * hgroups);
     }
   };
   if ((int)blockIdx.x < n_units) {
@@ -1222,14 +1224,14 @@ static int launch_prefill_t(const PrefillArgs& a, int64_t num_tokens, hipStream_
   return launch_prefill_tq<E, 4, 1>(a, num_tokens, st);
 }
 
-template <typename E, int TQ, int DS>
+template <typename E, int TQ, int DS, int NQ = 1>
 static int launch_fused_tq(const PrefixArgs& a, const ItemArgs& ia, int num_groups, int max_group_reqs, int cus,
                            int np, hipStream_t st, const KernelEvents& ev) {
   constexpr int QT = 32 * (8 / TQ);
   constexpr int HPW = HeadLanes<DS>::HPW;
   const int mtiles = (max_group_reqs + QT - 1) / QT;
   const int n_units = a.n_splits * a.H * num_groups * mtiles;
-  const int hgroups = (ia.H + HPW - 1) / HPW;
+  const int hgroups = (ia.H / NQ + HPW - 1) / HPW;
   const int wave_slots = ia.num_lanes * hgroups;
   int grid;
   if (np > 0) {
@@ -1245,20 +1247,30 @@ static int launch_fused_tq(const PrefixArgs& a, const ItemArgs& ia, int num_grou
     if (grid < unit_grid) grid = unit_grid;
   }
   if (grid <= 0) return PH_OK;
-  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&decode_fused_kernel<E, TQ, DS>),
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&decode_fused_kernel<E, TQ, DS, NQ>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, kTile8Lds);
-  PH_LAUNCH_TIMED((decode_fused_kernel<E, TQ, DS>), dim3(grid), dim3(512), kTile8Lds, st, ev, a, mtiles,
+  PH_LAUNCH_TIMED((decode_fused_kernel<E, TQ, DS, NQ>), dim3(grid), dim3(512), kTile8Lds, st, ev, a, mtiles,
                         n_units, np, ia);
   return launch_status();
 }
 
 // query tile by the largest group: 64, 128 or 256 requests share each K/V tile of the prefix
-template <typename E, int DS>
+template <typename E, int DS, int NQ = 1>
 static int launch_fused_t(const PrefixArgs& a, const ItemArgs& ia, int num_groups, int max_group_reqs, int cus, int np,
                           hipStream_t st, const KernelEvents& ev) {
-  if (max_group_reqs <= 64) return launch_fused_tq<E, 4, DS>(a, ia, num_groups, max_group_reqs, cus, np, st, ev);
-  if (max_group_reqs <= 128) return launch_fused_tq<E, 2, DS>(a, ia, num_groups, max_group_reqs, cus, np, st, ev);
-  return launch_fused_tq<E, 1, DS>(a, ia, num_groups, max_group_reqs, cus, np, st, ev);
+  if (max_group_reqs <= 64) return launch_fused_tq<E, 4, DS, NQ>(a, ia, num_groups, max_group_reqs, cus, np, st, ev);
+  if (max_group_reqs <= 128) return launch_fused_tq<E, 2, DS, NQ>(a, ia, num_groups, max_group_reqs, cus, np, st, ev);
+  return launch_fused_tq<E, 1, DS, NQ>(a, ia, num_groups, max_group_reqs, cus, np, st, ev);
+}
+
+template <typename E>
+static int launch_fused_e(const PrefixArgs& a, const ItemArgs& ia, int num_groups, int max_group_reqs, int cus, int np,
+                          hipStream_t st, const KernelEvents& ev) {
+  if (a.req_shift && !a.gqa)  // 64-wide heads: the prefix phase on head pairs, the suffix phase at its own width
+    return launch_fused_t<E, 64>(a, ia, num_groups, max_group_reqs, cus, np, st, ev);
+  if (ia.nq == 4) return launch_fused_t<E, kPD, 4>(a, ia, num_groups, max_group_reqs, cus, np, st, ev);
+  if (ia.nq > 1) return PH_ERR_ARG;  // grouped_stream_heads() says which shapes have the grouped form
+  return launch_fused_t<E, kPD>(a, ia, num_groups, max_group_reqs, cus, np, st, ev);
 }
 
 // One launch for the prefix and suffix phases: head size 128 (the eight-wave prefix form), balanced suffix plan present.
@@ -1266,12 +1278,8 @@ bool decode_fused_supported(int dtype, int D) { return D == kPD && (dtype == PH_
 
 int launch_decode_fused(const PrefixArgs& a, const ItemArgs& ia, int dtype, int num_groups, int max_group_reqs, int cus,
                         int prefix_wgs, hipStream_t st, const KernelEvents& ev) {
-  if (a.req_shift && !a.gqa) {  // 64-wide heads: the prefix phase on head pairs, the suffix phase at its own width
-    return dtype == PH_F16 ? launch_fused_t<F16, 64>(a, ia, num_groups, max_group_reqs, cus, prefix_wgs, st, ev)
-                           : launch_fused_t<BF16, 64>(a, ia, num_groups, max_group_reqs, cus, prefix_wgs, st, ev);
-  }
-  return dtype == PH_F16 ? launch_fused_t<F16, kPD>(a, ia, num_groups, max_group_reqs, cus, prefix_wgs, st, ev)
-                         : launch_fused_t<BF16, kPD>(a, ia, num_groups, max_group_reqs, cus, prefix_wgs, st, ev);
+  return dtype == PH_F16 ? launch_fused_e<F16>(a, ia, num_groups, max_group_reqs, cus, prefix_wgs, st, ev)
+                         : launch_fused_e<BF16>(a, ia, num_groups, max_group_reqs, cus, prefix_wgs, st, ev);
 }
 
 // head size 128, and 80 / 96 / 112 as short heads on the 128-wide tile (TileWork::head_dim)

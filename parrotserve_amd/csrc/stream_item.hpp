@@ -14,18 +14,26 @@ namespace ph {
 // writes the (O, m, l) part at row `pr` of the partial buffers.  `myslot` holds the slot ids of the
 // first 64 tokens (lane i: token t0 + i, clamped), already fetched by the caller.  `lane_off` = this lane's
 // element offset inside a token row of the K/V pools (its KV head's row, see kv_lane_off).
-template <typename E, int D, int TB, int STAGES>
+// NQ > 1 (grouped KV heads): a wave's head slot holds a run of NQ adjacent query heads that share a KV head, and every
+// token row meets the NQ queries at once -- one load of the row, NQ scores, NQ parts at rows pr .. pr + NQ - 1 --
+// instead of being loaded once per query head.
+template <typename E, int D, int TB, int STAGES, int NQ = 1>
 __device__ __forceinline__ void stream_item(const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
                                             int64_t row_stride, const int32_t* __restrict__ slots, int myslot,
-                                            int t0, int t1, u32x4 qv, uint32_t lane_off, float scale_log2e,
-                                            bool head_ok, float* __restrict__ opart, float* __restrict__ ml,
-                                            int64_t pr) {
+                                            int t0, int t1, const u32x4 (&qv)[NQ], uint32_t lane_off,
+                                            float scale_log2e, bool head_ok, float* __restrict__ opart,
+                                            float* __restrict__ ml, int64_t pr) {
   constexpr int LPH = HeadLanes<D>::LPH;
   const int lane = threadIdx.x & 63;
-  float m = -INFINITY, l = 0.f;
-  float o[8];
+  float m[NQ], l[NQ];
+  float o[NQ][8];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) o[i] = 0.f;
+  for (int n = 0; n < NQ; ++n) {
+    m[n] = -INFINITY;
+    l[n] = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o[n][i] = 0.f;
+  }
 
   u32x4 kb[STAGES][TB], vb[STAGES][TB];
 
@@ -45,33 +53,36 @@ __device__ __forceinline__ void stream_item(const uint16_t* __restrict__ kc, con
       }
     };
     auto compute = [&](const u32x4(&kk)[TB], const u32x4(&vv)[TB], int j0) {
-      float s[TB];
-      float mb = -INFINITY;
 #pragma unroll
-      for (int j = 0; j < TB; ++j) {
-        float d = 0.f;
+      for (int n = 0; n < NQ; ++n) {
+        float s[TB];
+        float mb = -INFINITY;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) d = Elem<E>::dot2(qv[w], kk[j][w], d);
-        d = group_sum<LPH>(d) * scale_log2e;
-        s[j] = (j0 + j < nb) ? d : -INFINITY;
-        mb = fmaxf(mb, s[j]);
-      }
-      const float mn = fmaxf(m, mb);
-      const float alpha = __builtin_amdgcn_exp2f(m - mn);
-      l *= alpha;
+        for (int j = 0; j < TB; ++j) {
+          float d = 0.f;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) o[i] *= alpha;
-#pragma unroll
-      for (int j = 0; j < TB; ++j) {
-        const float p = __builtin_amdgcn_exp2f(s[j] - mn);
-        l += p;
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-          o[2 * w] = __builtin_fmaf(p, Elem<E>::lo(vv[j][w]), o[2 * w]);
-          o[2 * w + 1] = __builtin_fmaf(p, Elem<E>::hi(vv[j][w]), o[2 * w + 1]);
+          for (int w = 0; w < 4; ++w) d = Elem<E>::dot2(qv[n][w], kk[j][w], d);
+          d = group_sum<LPH>(d) * scale_log2e;
+          s[j] = (j0 + j < nb) ? d : -INFINITY;
+          mb = fmaxf(mb, s[j]);
         }
+        const float mn = fmaxf(m[n], mb);
+        const float alpha = __builtin_amdgcn_exp2f(m[n] - mn);
+        l[n] *= alpha;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o[n][i] *= alpha;
+#pragma unroll
+        for (int j = 0; j < TB; ++j) {
+          const float p = __builtin_amdgcn_exp2f(s[j] - mn);
+          l[n] += p;
+#pragma unroll
+          for (int w = 0; w < 4; ++w) {
+            o[n][2 * w] = __builtin_fmaf(p, Elem<E>::lo(vv[j][w]), o[n][2 * w]);
+            o[n][2 * w + 1] = __builtin_fmaf(p, Elem<E>::hi(vv[j][w]), o[n][2 * w + 1]);
+          }
+        }
+        m[n] = mn;
       }
-      m = mn;
     };
 
     if (STAGES == 2) {
@@ -93,15 +104,18 @@ __device__ __forceinline__ void stream_item(const uint16_t* __restrict__ kc, con
   }
 
   if (!head_ok || !HeadLanes<D>::active(lane)) return;
-  const float inv = 1.f / l;
-  float* op = opart + pr * D + (lane % LPH) * 8;
-  float4_t o0 = {o[0] * inv, o[1] * inv, o[2] * inv, o[3] * inv};
-  float4_t o1 = {o[4] * inv, o[5] * inv, o[6] * inv, o[7] * inv};
-  *reinterpret_cast<float4_t*>(op) = o0;
-  *reinterpret_cast<float4_t*>(op + 4) = o1;
-  if (lane % LPH == 0) {
-    ml[pr * 2] = m;
-    ml[pr * 2 + 1] = l;
+#pragma unroll
+  for (int n = 0; n < NQ; ++n) {
+    const float inv = 1.f / l[n];
+    float* op = opart + (pr + n) * D + (lane % LPH) * 8;
+    float4_t o0 = {o[n][0] * inv, o[n][1] * inv, o[n][2] * inv, o[n][3] * inv};
+    float4_t o1 = {o[n][4] * inv, o[n][5] * inv, o[n][6] * inv, o[n][7] * inv};
+    *reinterpret_cast<float4_t*>(op) = o0;
+    *reinterpret_cast<float4_t*>(op + 4) = o1;
+    if (lane % LPH == 0) {
+      ml[(pr + n) * 2] = m[n];
+      ml[(pr + n) * 2 + 1] = l[n];
+    }
   }
 }
 
@@ -189,14 +203,16 @@ __device__ __forceinline__ uint32_t kv_lane_off(const int32_t* head_map, int hea
 }
 
 // One request's list [t0, t1) through one wave, whatever the element type: loads the query (at lane_off of the
-// query row) and runs the streaming body (K/V at kv_off of every token row).
-template <typename E, int D, int TB, int STAGES>
+// query row; NQ > 1: the NQ adjacent query heads from there on) and runs the streaming body (K/V at kv_off of every
+// token row).
+template <typename E, int D, int TB, int STAGES, int NQ = 1>
 __device__ __forceinline__ void stream_request(const uint16_t* q, int64_t q_off, const uint16_t* kc, const uint16_t* vc,
                                                int64_t row_stride, const int32_t* slots, int myslot, int t0, int t1,
                                                uint32_t lane_off, uint32_t kv_off, float scale_log2e, bool head_ok,
                                                float* opart, float* ml, int64_t pr) {
   const int lane = threadIdx.x & 63;
   if constexpr (is_f32<E>::value) {
+    static_assert(NQ == 1, "grouped streaming is built for 16-bit elements");
     float qf[8];
     load8f<F32>(q, q_off + lane_off, qf);
     if (!HeadLanes<D>::active(lane)) {
@@ -206,26 +222,34 @@ __device__ __forceinline__ void stream_request(const uint16_t* q, int64_t q_off,
     stream_item_f32<D, TB>(reinterpret_cast<const float*>(kc), reinterpret_cast<const float*>(vc), row_stride, slots,
                            myslot, t0, t1, qf, kv_off, scale_log2e, head_ok, opart, ml, pr);
   } else {
-    u32x4 qv = ld16(q + q_off + lane_off);
-    if (!HeadLanes<D>::active(lane)) qv = u32x4{0u, 0u, 0u, 0u};
-    stream_item<E, D, TB, STAGES>(kc, vc, row_stride, slots, myslot, t0, t1, qv, kv_off, scale_log2e, head_ok, opart,
-                                  ml, pr);
+    u32x4 qv[NQ];
+#pragma unroll
+    for (int n = 0; n < NQ; ++n) {
+      qv[n] = ld16(q + q_off + lane_off + n * D);
+      if (!HeadLanes<D>::active(lane)) qv[n] = u32x4{0u, 0u, 0u, 0u};
+    }
+    stream_item<E, D, TB, STAGES, NQ>(kc, vc, row_stride, slots, myslot, t0, t1, qv, kv_off, scale_log2e, head_ok,
+                                      opart, ml, pr);
   }
 }
 
 // One piece of the balanced form for one head group: the piece's items (request, first token, count) are
 // streamed one after the other by this wave, one partial row per item.
 // (rec0, rec1) = the piece's lane record, already loaded by the caller
-template <typename E, int D, int TB, int STAGES>
+// NQ > 1: the waves divide the a.H / NQ runs of NQ adjacent query heads; run r reads KV head r >> a.kv_shift (a KV
+// head's query heads are one run, or 2, 4 .. adjacent runs).
+template <typename E, int D, int TB, int STAGES, int NQ = 1>
 __device__ __forceinline__ void run_piece_rec(const ItemArgs& a, int hg, int4 rec0, int4 rec1) {
   constexpr int LPH = HeadLanes<D>::LPH;
   constexpr int HPW = HeadLanes<D>::HPW;
   const int lane = threadIdx.x & 63;
+  const int heads = NQ > 1 ? a.H / NQ : a.H;  // the heads the waves divide among themselves
   const int head = hg * HPW + lane / LPH;
-  const bool head_ok = head < a.H;
-  const int hclamp = head_ok ? head : a.H - 1;
-  const uint32_t lane_off = (uint32_t)(hclamp * D + HeadLanes<D>::chunk(lane) * 8);
-  const uint32_t kv_off = kv_lane_off<D>(a.head_map, hclamp, lane);
+  const bool head_ok = head < heads;
+  const int hclamp = head_ok ? head : heads - 1;
+  const uint32_t lane_off = (uint32_t)(hclamp * NQ * D + HeadLanes<D>::chunk(lane) * 8);  // the (first) query head
+  const uint32_t kv_off = NQ > 1 ? (uint32_t)((hclamp >> a.kv_shift) * D + HeadLanes<D>::chunk(lane) * 8)
+                                 : kv_lane_off<D>(a.head_map, hclamp, lane);
   const int i0 = rec0.x, i1 = rec0.x + rec0.y;
   for (int it = i0; it < i1; ++it) {
     int4 meta = {rec0.z, rec0.w, rec1.x, 0};
@@ -233,17 +257,17 @@ __device__ __forceinline__ void run_piece_rec(const ItemArgs& a, int hg, int4 re
     const int b = meta.x, t0 = meta.y, t1 = meta.y + meta.z;
     const int32_t* slots = a.slots + (a.offsets ? a.offsets[b] : (int64_t)b * a.table_stride);
     const int myslot = slots[min(t0 + lane, t1 - 1)];
-    stream_request<E, D, TB, STAGES>(a.q, (int64_t)b * a.q_stride, a.kc, a.vc, a.row_stride, slots, myslot, t0, t1,
-                                     lane_off, kv_off, a.scale_log2e, head_ok, a.opart, a.ml,
-                                     (int64_t)it * a.H + hclamp);
+    stream_request<E, D, TB, STAGES, NQ>(a.q, (int64_t)b * a.q_stride, a.kc, a.vc, a.row_stride, slots, myslot, t0, t1,
+                                         lane_off, kv_off, a.scale_log2e, head_ok, a.opart, a.ml,
+                                         (int64_t)it * a.H + hclamp * NQ);
   }
 }
 
-template <typename E, int D, int TB, int STAGES>
+template <typename E, int D, int TB, int STAGES, int NQ = 1>
 __device__ __forceinline__ void run_piece(const ItemArgs& a, int piece, int hg) {
   // lane record: (first item, item count, then the first item's request / first token / count inline,
   // so the first K/V rows are three dependent loads away from launch, not five)
-  run_piece_rec<E, D, TB, STAGES>(a, hg, a.lane_rec[2 * piece], a.lane_rec[2 * piece + 1]);
+  run_piece_rec<E, D, TB, STAGES, NQ>(a, hg, a.lane_rec[2 * piece], a.lane_rec[2 * piece + 1]);
 }
 
 }  // namespace ph

@@ -491,11 +491,12 @@ class DecodeTables:
     @staticmethod
     def build(prefix_lists: Sequence[Sequence[int]], group_req_cu: Sequence[int],
               suffix_lists: Sequence[Sequence[int]], device, num_heads: int = 32, head_dim: int = 128,
-              balanced: bool = True, dtype: torch.dtype = torch.float16) -> "DecodeTables":
+              balanced: bool = True, dtype: torch.dtype = torch.float16, kv_group: int = 1) -> "DecodeTables":
         """From python lists: ``prefix_lists[g]`` is group g's slot list shared by
         requests ``group_req_cu[g] .. group_req_cu[g+1]-1``; ``suffix_lists[b]`` is
         request b's own slot list.  ``balanced`` adds the item list of the
-        suffix phase, cut for ``num_heads x head_dim`` heads of ``dtype`` elements."""
+        suffix phase, cut for ``num_heads x head_dim`` heads of ``dtype`` elements (``kv_group = G``: for calls
+        whose query heads share KV heads as ``h // G``)."""
         B = len(suffix_lists)
         t = DecodeTables(num_reqs=B)
         G = len(prefix_lists)
@@ -540,7 +541,7 @@ class DecodeTables:
             t.chunk_tokens = chunk
             if balanced:
                 shape = dict(num_reqs=B, num_groups=t.num_groups, max_prefix_len=t.max_prefix_len,
-                             max_suffix_len=t.max_suffix_len, dtype=dtype)
+                             max_suffix_len=t.max_suffix_len, dtype=dtype, kv_group=kv_group)
                 if B <= PLAN_MAX_REQS and t.suffix_offsets is None:
                     t.plan_on_device(suffix_lane_capacity(device, num_heads, head_dim, **shape), device)
                 else:
@@ -598,10 +599,13 @@ def _heads_per_wave(head_dim: int) -> int:
 
 
 def suffix_lane_capacity(device, num_heads: int, head_dim: int, num_reqs: int = 0, num_groups: int = 0,
-                         max_prefix_len: int = 0, max_suffix_len: int = 0, dtype: torch.dtype = torch.float16) -> int:
+                         max_prefix_len: int = 0, max_suffix_len: int = 0, dtype: torch.dtype = torch.float16,
+                         kv_group: int = 1) -> int:
     """Lanes the balanced suffix plan should be cut into (``ph_decode_suffix_lanes``): one launch-wide round of waves
     at two waves per SIMD on the compute units the suffix phase runs on -- all of them, or, for a batch whose
-    prefix and suffix phases get workgroups of their own inside one launch, the ones the prefix leaves."""
+    prefix and suffix phases get workgroups of their own inside one launch, the ones the prefix leaves.
+    ``kv_group = G > 1``: the call will name a head mapping ``h // G`` (``decode_attention(..., kv_group=G)``), where
+    the suffix waves may divide the KV heads instead of the query heads."""
     if num_reqs <= 0 or str(device) == "cpu" or not torch.cuda.is_available():
         heads_per_wave = _heads_per_wave(head_dim)
         hgroups = (num_heads + heads_per_wave - 1) // heads_per_wave
@@ -609,7 +613,7 @@ def suffix_lane_capacity(device, num_heads: int, head_dim: int, num_reqs: int = 
     code = {torch.float16: _lib.PH_F16, torch.bfloat16: _lib.PH_BF16, torch.float32: _lib.PH_F32}[dtype]
     with torch.cuda.device(device):
         return int(_lib.load().ph_decode_suffix_lanes(num_reqs, num_heads, head_dim, code, num_groups, max_prefix_len,
-                                                      max_suffix_len))
+                                                      max_suffix_len, max(1, int(kv_group))))
 
 
 def suffix_lanes(device, num_heads: int, head_dim: int, total_tokens: int, **shape) -> int:
@@ -795,12 +799,13 @@ _paged_tables_cache: "collections.OrderedDict[Tuple, Tuple[Tuple, DecodeTables]]
 _PAGED_TABLES_CACHE_ENTRIES = 8
 
 
-def _paged_tables(query, context_lens, block_tables, flash_context_len: int = 0, flash_block_table=None) -> DecodeTables:
+def _paged_tables(query, context_lens, block_tables, flash_context_len: int = 0, flash_block_table=None,
+                  kv_group: int = 0) -> DecodeTables:
     B, H, D = query.shape
     P = int(flash_context_len)
     key = (context_lens.data_ptr(), context_lens._version, B, block_tables.data_ptr(), block_tables.stride(0),
            block_tables.shape[1], H, D, query.dtype, P, 0 if flash_block_table is None else flash_block_table.data_ptr(),
-           str(query.device))
+           str(query.device), kv_group)
     hit = _paged_tables_cache.get(key)
     if hit is not None:
         _paged_tables_cache.move_to_end(key)
@@ -819,7 +824,7 @@ def _paged_tables(query, context_lens, block_tables, flash_context_len: int = 0,
     if 0 < B <= PLAN_MAX_REQS and t.max_suffix_len > 0:
         t.plan_on_device(suffix_lane_capacity(query.device, H, D, num_reqs=B, num_groups=t.num_groups,
                                               max_prefix_len=t.max_prefix_len, max_suffix_len=t.max_suffix_len,
-                                              dtype=query.dtype), query.device)
+                                              dtype=query.dtype, kv_group=kv_group), query.device)
     _paged_tables_cache[key] = ((context_lens, block_tables, flash_block_table), t)
     while len(_paged_tables_cache) > _PAGED_TABLES_CACHE_ENTRIES:
         _paged_tables_cache.popitem(last=False)
@@ -830,7 +835,8 @@ def vllm_paged_attention(query, key_cache, value_cache, head_mapping, context_le
     """Non-shared ragged decode (parrot/engine/builtin/kernels/vllm/paged_attention.py:12-38):
     request i attends over ``block_tables[i, :context_lens[i]]``."""
     heads = _check_paged_args(query, key_cache, value_cache, head_mapping, context_lens, block_tables)
-    return decode_attention(query, key_cache, value_cache, _paged_tables(query, context_lens, block_tables), **heads)
+    tables = _paged_tables(query, context_lens, block_tables, kv_group=heads["kv_group"])
+    return decode_attention(query, key_cache, value_cache, tables, **heads)
 
 
 def flash_paged_attention(query, key_cache, value_cache, head_mapping, flash_context_len, flash_block_table,
@@ -839,7 +845,8 @@ def flash_paged_attention(query, key_cache, value_cache, head_mapping, flash_con
     all requests attend over ``flash_block_table[:flash_context_len]`` plus their
     own ``paged_block_tables[i, :paged_context_lens[i]]``."""
     heads = _check_paged_args(query, key_cache, value_cache, head_mapping, paged_context_lens, paged_block_tables)
-    t = _paged_tables(query, paged_context_lens, paged_block_tables, flash_context_len, flash_block_table)
+    t = _paged_tables(query, paged_context_lens, paged_block_tables, flash_context_len, flash_block_table,
+                      kv_group=heads["kv_group"])
     return decode_attention(query, key_cache, value_cache, t, **heads)
 
 

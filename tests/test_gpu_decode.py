@@ -394,14 +394,14 @@ def test_reference_named_ops_reuse_the_plan_across_layers_and_notice_new_lengths
     torch.testing.assert_close(out_c.cpu().float(), ref_c.float(), **TOL[torch.float16])
 
 
-def _gqa_case(dtype, B, P, Hq, Hkv, D, seed, smax=90):
+def _gqa_case(dtype, B, P, Hq, Hkv, D, seed, smax=90, pool=1 << 13):
     """A shared-prefix decode case with Hq query heads over Hkv KV heads: the case is drawn with Hkv heads and the
     query widened to Hq."""
     from parrotserve_amd import synth
 
     g = torch.Generator().manual_seed(seed)
     s = torch.randint(1, smax, (B,), generator=g).tolist()
-    case = synth.make_decode_case("gqa", seed, dtype, 1, B, P, s, Hkv, D, 1 << 13)
+    case = synth.make_decode_case("gqa", seed, dtype, 1, B, P, s, Hkv, D, pool)
     q = torch.randn(B, Hq, D, generator=g).to(dtype)
     return case, q
 
@@ -438,6 +438,35 @@ def test_grouped_kv_heads(dev, dtype, D, B, P):
     flens = torch.tensor([len(x) for x in full], dtype=torch.int32, device=dev)
     out1 = kernels.vllm_paged_attention(q.to(dev), kc, vc, hm.to(dev), flens, ftable)
     torch.testing.assert_close(out1.cpu().float(), ref.float(), **TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("Hq,Hkv", [(16, 2), (12, 3), (40, 5), (8, 2)])
+def test_query_heads_of_a_kv_head_streamed_together(dev, dtype, Hq, Hkv):
+    """Groups of 8 and of 4 query heads per KV head at head size 128: the suffix waves divide runs of four query heads
+    that share a KV head and meet every token row with the run's queries at once (run counts that fill a wave's four
+    head slots, leave some empty, and need further waves).  Through the reference-named ops (plan cut for the grouped form), with a plan
+    cut for the plain form (fewer pieces than the grouped launch has room for), and without a prefix."""
+    from parrotserve_amd import kernels, synth
+
+    B, P, D, G = 70, 420, 128, Hq // Hkv
+    case, q = _gqa_case(dtype, B, P, Hq, Hkv, D, 600 + Hq, smax=260, pool=1 << 15)  # lists long enough for the form
+    hm = torch.arange(Hkv, dtype=torch.int32).repeat_interleave(G)
+    kc, vc = synth.pool_to_device(case.k_rows, case.v_rows, case.used_slots, case.pool_slots, dev)
+    flash, lens, table = _paged_inputs(case, dev)
+    ref = ref_decode_attention(q, case.k_rows[:, hm.long()], case.v_rows[:, hm.long()], case.full_lists())
+    out = kernels.flash_paged_attention(q.to(dev), kc, vc, hm.to(dev), P, flash, lens, table)
+    torch.testing.assert_close(out.cpu().float(), ref.float(), **TOL[dtype])
+    plain = kernels.DecodeTables.build(case.pool_lists(case.prefix_lists), case.group_req_cu,
+                                       case.pool_lists(case.suffix_lists), dev, num_heads=Hq, head_dim=D, dtype=dtype)
+    out2 = kernels.decode_attention(q.to(dev), kc, vc, plain, head_mapping=hm.to(dev), kv_group=G)
+    torch.testing.assert_close(out2.cpu().float(), ref.float(), **TOL[dtype])
+    full = [case.used_slots[l].tolist() for l in case.full_lists()]
+    mx = max(len(x) for x in full)
+    ftable = torch.tensor([x + [0] * (mx - len(x)) for x in full], dtype=torch.int32, device=dev)
+    flens = torch.tensor([len(x) for x in full], dtype=torch.int32, device=dev)
+    out3 = kernels.vllm_paged_attention(q.to(dev), kc, vc, hm.to(dev), flens, ftable)
+    torch.testing.assert_close(out3.cpu().float(), ref.float(), **TOL[dtype])
 
 
 def test_any_head_mapping_and_the_identity(dev):
