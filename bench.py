@@ -307,6 +307,7 @@ def extras(torch, dev):
                                  "algorithmic_bytes": nbytes}
     out["sampler_64x32000"] = sampler_cost(torch, dev)
     out["c2_shape_head_size_64"] = head_size_64_step(torch, dev)
+    out["c2_shape_grouped_kv_heads_32_over_8"] = grouped_kv_heads_step(torch, dev)
     return out
 
 
@@ -505,6 +506,40 @@ def head_size_64_step(torch, dev):
     res["prefill_c4_chunks_40x64"] = {"tokens": int(sum(p4.q_lens)), "ms": tp * 1e3, "flops": flops,
                                       "TFLOP/s": flops / tp / 1e12}
     return res
+
+
+def grouped_kv_heads_step(torch, dev):
+    """Config 2's batch with grouped KV heads (32 query heads over 8 KV heads, head_mapping h // 4 -- the
+    argument of csrc/attention/attention_post_kernels.cu:79,101 that the reference's own models leave at the
+    identity): the decode step through ``ph_decode_attention_gqa`` over K/V sets that rotate out of the caches."""
+    from parrotserve_amd import kernels
+
+    B, P, H, HKV, D, pool = 64, 4096, 32, 8, 128, 1 << 20
+    g = torch.Generator().manual_seed(1)
+    lens = torch.randint(16, 513, (B,), generator=g).tolist()
+    need = P + sum(lens)
+    nbytes = 2 * need * HKV * D * 2
+    nsets = 8
+    kc = torch.randn((pool, HKV, D), device=dev, dtype=torch.float16)
+    vc = torch.randn_like(kc)
+    perm = torch.randperm(pool, generator=g)
+    tabs = []
+    for i in range(nsets):
+        sl = perm[i * need:(i + 1) * need].tolist()
+        pos, suf = P, []
+        for n in lens:
+            suf.append(sl[pos:pos + n])
+            pos += n
+        tabs.append(kernels.DecodeTables.build([sl[:P]], [0, B], suf, dev, num_heads=H, head_dim=D, kv_group=H // HKV))
+    q = torch.randn((B, H, D), device=dev, dtype=torch.float16)
+    o = torch.empty_like(q)
+    hm = (torch.arange(H, dtype=torch.int32) // (H // HKV)).to(dev)
+    rot = _Rotor(nsets)
+    t = _time_gpu(torch, lambda: kernels.decode_attention(q, kc, vc, tabs[rot.next()], out=o, head_mapping=hm,
+                                                          kv_group=H // HKV))
+    return {"batch": B, "prefix": P, "sum_suffix": sum(lens), "heads": H, "kv_heads": HKV, "kv_sets": nsets,
+            "us": t * 1e6, "GB/s": nbytes / t / 1e9, "frac_hbm": nbytes / t / 1e9 / HBM_PEAK_GBS,
+            "algorithmic_bytes": nbytes, "tokens/s/layer": B / t}
 
 
 def sampler_cost(torch, dev):
