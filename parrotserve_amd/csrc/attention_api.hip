@@ -130,6 +130,8 @@ static RoleChoice choose_roles(const FusedShape& f, int64_t max_prefix, int64_t 
   const double kCu = f.stream_mb_per_us;
   constexpr double kStep = 2.7, kFirst = 12.0, kFold = 2.0, kNext = 6.0, kMargin = 3.0, kPiece = 4.0;
   const double floor_us = 4.0 + (f.prefix_mb + f.suffix_mb) / kHbm;
+  // a step of the 128- and 256-query tiles is twice and four times the matrix work of the 64-query tile's
+  const double tile_mul = f.query_tile == 256 ? 1.5 : f.query_tile == 128 ? 1.1 : 1.0;
   RoleChoice best{1, 1, 0.0};
   double best_cost = -1.0;
   const int64_t max_splits = std::max<int64_t>(1, cdiv(max_prefix, 4 * kPrefixTile));
@@ -141,7 +143,7 @@ static RoleChoice choose_roles(const FusedShape& f, int64_t max_prefix, int64_t 
     for (int64_t r = 1; r <= 8; ++r) {
       const int64_t np = cdiv(units, r);
       if (np > cus - 1) continue;
-      const double t_prefix = kFirst + r * (steps * kStep + kFold) + (r - 1) * kNext + kMargin;
+      const double t_prefix = kFirst + r * (steps * kStep * tile_mul + kFold) + (r - 1) * kNext + kMargin;
       const int64_t lanes = std::max<int64_t>(1, (cus - np) * 8 / f.head_groups);
       const double t_suffix =
           6.0 + (double)cdiv(f.reqs, lanes) * kPiece + f.suffix_mb / std::min(kHbm, (double)(cus - np) * kCu);
