@@ -441,9 +441,9 @@ def test_grouped_kv_heads(dev, dtype, D, B, P):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("Hq,Hkv", [(16, 2), (12, 3), (40, 5), (8, 2)])
+@pytest.mark.parametrize("Hq,Hkv", [(16, 2), (12, 3), (40, 5), (8, 2), (32, 2)])
 def test_query_heads_of_a_kv_head_streamed_together(dev, dtype, Hq, Hkv):
-    """Groups of 8 and of 4 query heads per KV head at head size 128: the suffix waves divide runs of four query heads
+    """Groups of 16, 8 and 4 query heads per KV head at head size 128: the suffix waves divide runs of four query heads
     that share a KV head and meet every token row with the run's queries at once (run counts that fill a wave's four
     head slots, leave some empty, and need further waves).  Through the reference-named ops (plan cut for the grouped form), with a plan
     cut for the plain form (fewer pieces than the grouped launch has room for), and without a prefix."""
