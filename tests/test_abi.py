@@ -52,6 +52,29 @@ def test_workspace_queries_are_host_only():
     assert lib.ph_prefill_workspace_bytes(1000, 40, 128, 2, 3000) > lib.ph_prefill_workspace_bytes(1000, 40, 128, 1, 3000)
 
 
+def test_how_the_planner_divides_a_256_unit_device():
+    """``ph_decode_suffix_lanes`` is host arithmetic (without a device it plans for 256 compute units): the lane
+    counts behind the measured configurations, so that a change of the cost models shows up here and not only as a
+    slower benchmark.  lanes = 8 waves x (256 - prefix-only workgroups) / waves per piece."""
+    from parrotserve_amd import _lib
+
+    lanes = _lib.load().ph_decode_suffix_lanes
+    f16 = _lib.PH_F16
+    assert lanes(64, 32, 128, f16, 1, 4096, 512, 1) == 160    # config 2: 96 prefix-only workgroups (3 splits x 32 heads)
+    assert lanes(128, 40, 128, f16, 4, 6000, 1024, 1) == 119  # config 5: 107 (2 splits x 160 units in three rounds)
+    assert lanes(64, 40, 128, f16, 1, 8192, 20, 1) == 12      # the reference benchmark's shape: 240 (6 splits x 40)
+    # all prefix (a long prefix under a few own tokens), no prefix, no matrix-core form: every compute unit streams
+    assert lanes(64, 8, 128, f16, 1, 8192, 8, 1) == 256 * 8 // 2
+    assert lanes(64, 32, 128, f16, 0, 0, 512, 1) == 256
+    assert lanes(64, 32, 128, _lib.PH_F32, 1, 4096, 512, 1) == 256
+    assert lanes(64, 32, 256, f16, 1, 4096, 512, 1) == 256 * 8 // 16
+    # grouped KV heads: long lists are streamed for four query heads at once (a piece takes a quarter of the waves);
+    # short ones, and groups the grouped stream is not built for, keep one piece per four query heads
+    assert lanes(64, 32, 128, f16, 1, 4096, 512, 4) > 2 * lanes(64, 32, 128, f16, 1, 4096, 512, 1)
+    assert lanes(64, 32, 128, f16, 1, 4096, 60, 4) <= 256
+    assert lanes(64, 32, 128, f16, 0, 0, 512, 2) == 256
+
+
 def test_argument_validation_needs_no_gpu():
     """Bad arguments are rejected before any launch."""
     from parrotserve_amd import _lib
