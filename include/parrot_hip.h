@@ -296,8 +296,12 @@ int ph_decode_attention(void* out, const void* q, const void* k_cache, const voi
  *                 the prefix phase then runs on the matrix cores with the G
  *                 query heads of a KV head as G rows per request of one tile,
  *                 so a group's prefix K/V is still read once -- and at G times
- *                 the arithmetic per byte.  0 = any mapping: every phase runs
- *                 per request.
+ *                 the arithmetic per byte; from G = 4 on, suffix lists of 200
+ *                 tokens and more (about 8000 in all) are streamed for four
+ *                 query heads of a KV head at once, one load of a token row
+ *                 for the four (a suffix plan for such a call is cut for the
+ *                 count ph_decode_suffix_lanes(.., kv_group = G) returns).
+ *                 0 = any mapping: every phase runs per request.
  * Everything else as ph_decode_attention (workspace: the same
  * ph_decode_workspace_bytes). */
 int ph_decode_attention_gqa(void* out, const void* q, const void* k_cache, const void* v_cache,
